@@ -1,0 +1,168 @@
+/*
+ * svodk — C ABI of the MI355X (gfx950) implementation of Svod's `tk`
+ * flash-attention forward op and of the attention prologue ("heads").
+ *
+ * Every entry point replaces one item of the reference's op layer; the
+ * citation beside it is into the reference checkout.  The library follows the
+ * op layer's contract: an op either launches a kernel, or says that the
+ * caller's graph must run and why, or rejects arguments the graph would
+ * reject too (tk/src/ops/mod.rs:1-4).  It computes nothing on the host and
+ * allocates no device memory: the caller owns every buffer.
+ *
+ * All pointers in tensor descriptors are DEVICE pointers (dense, row-major,
+ * in the layouts the reference op takes).  Launches are enqueued on the HIP
+ * stream given and return without synchronising.
+ */
+#ifndef SVODK_H
+#define SVODK_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SVODK_ABI_VERSION 1
+
+/* Element types of a tensor descriptor. */
+typedef enum svodk_dtype {
+  SVODK_BF16 = 0,
+  SVODK_F16 = 1,
+  SVODK_F32 = 2,
+  SVODK_I32 = 3,
+  SVODK_I64 = 4,
+  SVODK_BOOL = 5 /* one byte per element, nonzero = true */
+} svodk_dtype;
+
+/*
+ * What an op call did.  Mirrors the three outcomes of the reference op layer:
+ *   0   a kernel was enqueued             (Plan::Kernel, tk/src/ops/shape.rs:19-24)
+ *   > 0 the caller's graph must run, why  (Plan::Graph(Fallback), shape.rs:26-39)
+ *   < 0 the arguments are invalid         (ops::Error, tk/src/ops/mod.rs:132-157)
+ */
+typedef enum svodk_status {
+  SVODK_KERNEL = 0,
+  SVODK_GRAPH_TARGET = 1,   /* Fallback::Target: no gfx950 device / no kernels for it */
+  SVODK_GRAPH_DTYPE = 2,    /* Fallback::Dtype: f32, or a type without a kernel here */
+  SVODK_GRAPH_SYMBOLIC = 3, /* Fallback::Symbolic: a live batch that is not a leading bound */
+  SVODK_GRAPH_SHAPE = 4,    /* Fallback::Shape: a shape the kernels do not cover */
+  SVODK_GRAPH_CONFIG = 5,   /* Fallback::Config: an option no kernel config here holds */
+  SVODK_ERR_SHAPE = -1,     /* Error::Shape */
+  SVODK_ERR_DTYPE = -2,     /* Error::Dtype */
+  SVODK_ERR_HEADS = -3,     /* Error::Heads */
+  SVODK_ERR_LAUNCH = -4,    /* Error::Launch: aliased parameters, a HIP error */
+  SVODK_ERR_ARGUMENT = -5   /* a null or malformed descriptor (no reference counterpart:
+                               Rust's type system rules these out) */
+} svodk_status;
+
+/* A dense row-major device tensor.  `rank` <= 4; unused dims are ignored. */
+typedef struct svodk_tensor {
+  void *data;
+  int32_t dtype; /* svodk_dtype */
+  int32_t rank;
+  int64_t shape[4];
+} svodk_tensor;
+
+/* KeyMask of tk/src/ops/attention.rs:29-37. */
+typedef enum svodk_key_mask {
+  SVODK_KEYS_NONE = 0,
+  SVODK_KEYS_LENS = 1, /* [B] integer valid-key counts (I32 or I64) */
+  SVODK_KEYS_BOOL = 2  /* [B, Tk] BOOL or integer, nonzero = attended; rows are NOT padded */
+} svodk_key_mask;
+
+/*
+ * Attn of tk/src/ops/attention.rs:60-86.  Zero-initialise, then set fields.
+ * Options this library has no kernel for (window, chunk, seg_start, cache,
+ * bias, splits > 1) are still validated as the reference validates them and
+ * then answered with SVODK_GRAPH_CONFIG.
+ */
+typedef struct svodk_attn {
+  int32_t causal;
+  int32_t key_kind; /* svodk_key_mask */
+  const svodk_tensor *keys;
+  int32_t has_window;
+  int64_t window_left, window_right;
+  int32_t has_chunk;
+  int64_t chunk_size;
+  int32_t chunk_has_left;
+  int64_t chunk_left, chunk_right;
+  const svodk_tensor *seg_start; /* [B, T] integers or NULL */
+  int32_t has_cache;             /* Cache{..}: never a kernel here */
+  const svodk_tensor *bias;      /* [B|1, H, T, Tk] or NULL */
+  int32_t splits;                /* 0 = None */
+  int32_t has_scale;
+  float scale; /* used when has_scale; else 1/sqrt(D) */
+  /* Batch::Var of tk/src/kernels/mod.rs:221-259: buffers hold `q.shape[0]`
+   * batches, only the first `batch_live` are computed and written.
+   * <= 0 means all of them. */
+  int32_t batch_live;
+} svodk_attn;
+
+/* Qkv of tk/src/ops/heads.rs:19-31. */
+typedef struct svodk_qkv {
+  int32_t heads, kv_heads, head_dim;
+  const svodk_tensor *q_norm; /* [head_dim] or NULL */
+  const svodk_tensor *k_norm; /* [head_dim] or NULL */
+  double eps;
+  const svodk_tensor *cos; /* [1|B, T, 1, head_dim/2] or NULL (both or neither) */
+  const svodk_tensor *sin;
+  int32_t batch_live; /* as in svodk_attn */
+} svodk_qkv;
+
+/*
+ * ops::attention (tk/src/ops/attention.rs:100-103 -> attend, :126-303).
+ * q [B,T,H,D], k and v [B,Tk,Hkv,D], out [B,T,H,D], all of one 16-bit type.
+ * Query head h reads KV head h / (H / Hkv).  A query no key reaches comes out
+ * as zeros (tk/src/kernels/attention.rs:974-980).
+ */
+int svodk_attention(const svodk_tensor *q, const svodk_tensor *k, const svodk_tensor *v, const svodk_attn *opts,
+                    const svodk_tensor *out, void *hip_stream);
+
+/*
+ * ops::heads (tk/src/ops/heads.rs:37-102).
+ * qkv [B,T,(heads+2*kv_heads)*head_dim] -> q [B,T,heads,D], k and v
+ * [B,T,kv_heads,D]: q and k RMS-normalised over the head where a weight is
+ * given, then rotated (halves paired) where tables are given; v copied.
+ */
+int svodk_heads(const svodk_tensor *qkv, const svodk_qkv *opts, const svodk_tensor *q, const svodk_tensor *k,
+                const svodk_tensor *v, void *hip_stream);
+
+/*
+ * The shape gates as pure functions, no device needed
+ * (shape::attention, tk/src/ops/shape.rs:189-206; shape::heads, :209-218;
+ * gate, :92-99).  `has_target` stands for "the default device has kernels".
+ * `dtypes` are those of every operand (q, k, v[, bias] / qkv[, weights, tables]).
+ * `q_dims`/`k_dims` NULL means a symbolic dim past the batch.
+ */
+int svodk_plan_attention(int32_t has_target, const int32_t *dtypes, int32_t n_dtypes, const int64_t *q_dims,
+                         const int64_t *k_dims, int32_t causal, int32_t bias);
+int svodk_plan_heads(int32_t has_target, const int32_t *dtypes, int32_t n_dtypes, const int64_t *x_dims, int32_t x_rank,
+                     int32_t head_dim);
+
+/*
+ * ops::supported (tk/src/ops/mod.rs:164-166): 1 when the current HIP device is
+ * a gfx950 this library has kernels for.
+ */
+int svodk_supported(void);
+
+/*
+ * ops::chosen (tk/src/ops/mod.rs:83-118): what the last op on THIS thread
+ * ran, as text — `Kernel { op: "attention", family: "flash_attention", cfg: "..." }`
+ * or `Graph { op: "attention", why: Dtype }`.  Empty before any op ran.
+ * The pointer stays valid until the thread's next op call.
+ */
+const char *svodk_last_chosen(void);
+
+/* The message of the last negative status on this thread (Display of ops::Error). */
+const char *svodk_last_error(void);
+
+/* Name of a status code, e.g. "Fallback::Shape". */
+const char *svodk_status_name(int status);
+
+int svodk_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SVODK_H */

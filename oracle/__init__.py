@@ -1,0 +1,285 @@
+"""CPU oracle for the tk flash-attention forward path and its prologue.
+
+TEST INFRASTRUCTURE — NOT PRODUCT CODE.  Only the tests, the smoke check and
+the CPU-baseline leg of the benchmark may import this package; the shipped
+HIP path never does.  The arithmetic lives in ``svod_oracle.c`` (each function
+cites the reference lines it restates); this module is a thin numpy/ctypes
+binding plus the seeded input generators the parity tests and the benchmark
+share.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+from dataclasses import dataclass
+from typing import Optional
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libsvod_oracle.so")
+
+
+def build(force: bool = False) -> str:
+    """Compile ``svod_oracle.c`` with gcc (``make`` in this directory)."""
+    if force:
+        subprocess.run(["make", "-C", _HERE, "clean"], check=True, capture_output=True)
+    subprocess.run(["make", "-C", _HERE], check=True, capture_output=True)
+    return _LIB_PATH
+
+
+_lib = None
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        _lib = ctypes.CDLL(_LIB_PATH)
+        _declare(_lib)
+    return _lib
+
+
+_f32p = ctypes.POINTER(ctypes.c_float)
+_f64p = ctypes.POINTER(ctypes.c_double)
+_i32p = ctypes.POINTER(ctypes.c_int32)
+_u8p = ctypes.POINTER(ctypes.c_uint8)
+_i32 = ctypes.c_int32
+
+
+def _declare(l: ctypes.CDLL) -> None:
+    l.svod_oracle_round_bf16.restype = ctypes.c_double
+    l.svod_oracle_round_bf16.argtypes = [ctypes.c_double]
+    l.svod_oracle_trunc_bf16.restype = ctypes.c_double
+    l.svod_oracle_trunc_bf16.argtypes = [ctypes.c_double]
+    l.svod_oracle_bf16_bits.restype = ctypes.c_uint16
+    l.svod_oracle_bf16_bits.argtypes = [ctypes.c_float]
+    l.svod_oracle_lcg.restype = ctypes.c_double
+    l.svod_oracle_lcg.argtypes = [ctypes.POINTER(ctypes.c_uint64)]
+    l.svod_oracle_lcg_fill.restype = ctypes.c_uint64
+    l.svod_oracle_lcg_fill.argtypes = [_f32p, ctypes.c_int64, ctypes.c_uint64, ctypes.c_double, ctypes.c_double, ctypes.c_int]
+    l.svod_oracle_normal_fill.restype = ctypes.c_uint64
+    l.svod_oracle_normal_fill.argtypes = [_f32p, ctypes.c_int64, ctypes.c_uint64, ctypes.c_double, ctypes.c_int]
+    l.svod_oracle_rope_table.restype = None
+    l.svod_oracle_rope_table.argtypes = [ctypes.c_double, _i32, _i32, _f32p, _f32p]
+    l.svod_oracle_visible.restype = None
+    l.svod_oracle_visible.argtypes = [_i32, _i32, _i32, _i32, _i32, _i32, _i32p, _i32p, _i32, _u8p]
+    l.svod_oracle_visible_pairs.restype = ctypes.c_int64
+    l.svod_oracle_visible_pairs.argtypes = [_i32, _i32, _i32, _i32, _i32p]
+    common = [_i32] * 6 + [_i32, _i32, _i32, ctypes.c_float, _i32p, _i32p, _i32]
+    l.svod_oracle_attention_direct.restype = ctypes.c_int
+    l.svod_oracle_attention_direct.argtypes = common + [_f32p, _f32p, _f32p, _f64p, _i32]
+    l.svod_oracle_attention_graph.restype = ctypes.c_int
+    l.svod_oracle_attention_graph.argtypes = common + [_i32, _f32p, _f32p, _f32p, _f32p, _i32]
+    l.svod_oracle_attention_flash.restype = ctypes.c_int
+    l.svod_oracle_attention_flash.argtypes = common + [_i32, _i32, _i32, _f32p, _f32p, _f32p, _f32p, _i32]
+    heads = [_i32] * 5 + [_i32, _i32, ctypes.c_double, _i32] + [_f32p] * 5 + [_f32p] * 3
+    for name in ("svod_oracle_heads_direct", "svod_oracle_heads_kernel", "svod_oracle_heads_graph"):
+        getattr(l, name).restype = ctypes.c_int
+        getattr(l, name).argtypes = heads
+
+
+# --------------------------------------------------------------------------
+# small helpers
+# --------------------------------------------------------------------------
+def _f32(a) -> np.ndarray:
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def _ptr(a: Optional[np.ndarray], ty):
+    return a.ctypes.data_as(ty) if a is not None else ctypes.cast(None, ty)
+
+
+def round_bf16(x):
+    """tk/src/interp.rs:37-44 applied elementwise; returns float32 values that are bf16-exact."""
+    a = np.ascontiguousarray(x, dtype=np.float32)
+    bits = a.view(np.uint32).astype(np.uint64)
+    rounded = ((bits + 0x7FFF + ((bits >> 16) & 1)) & 0xFFFF0000).astype(np.uint32)
+    nan = np.isnan(a)
+    rounded = np.where(nan, (a.view(np.uint32) | 0x00400000) & 0xFFFF0000, rounded).astype(np.uint32)
+    return rounded.view(np.float32).reshape(a.shape)
+
+
+def bf16_bits(x) -> np.ndarray:
+    """The 16 stored bits of ``round_bf16(x)`` as uint16."""
+    return (round_bf16(x).view(np.uint32) >> 16).astype(np.uint16)
+
+
+def from_bf16_bits(bits) -> np.ndarray:
+    return (np.ascontiguousarray(bits, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def lcg_fill(n: int, seed: int, mul: float = 1.0, add: float = 0.0, bf16: bool = True):
+    """``rounded(dtype, n, seed, |x| mul*x + add)`` of tk/src/test/unit/mod.rs:447-450.
+
+    Returns ``(values float32[n], advanced_seed)``."""
+    out = np.empty(n, dtype=np.float32)
+    seed = lib().svod_oracle_lcg_fill(_ptr(out, _f32p), n, ctypes.c_uint64(seed), mul, add, int(bf16))
+    return out, int(seed)
+
+
+def normal_fill(n: int, seed: int, sigma: float = 1.0, bf16: bool = True):
+    out = np.empty(n, dtype=np.float32)
+    seed = lib().svod_oracle_normal_fill(_ptr(out, _f32p), n, ctypes.c_uint64(seed), sigma, int(bf16))
+    return out, int(seed)
+
+
+def rope_table(theta: float, seq_len: int, head_dim: int):
+    """f32 ``(cos, sin)`` of shape ``[seq_len, head_dim/2]`` (tensor/src/transformer.rs:130-164)."""
+    half = head_dim // 2
+    cos = np.empty((seq_len, half), dtype=np.float32)
+    sin = np.empty((seq_len, half), dtype=np.float32)
+    lib().svod_oracle_rope_table(theta, seq_len, head_dim, _ptr(cos, _f32p), _ptr(sin, _f32p))
+    return cos, sin
+
+
+# --------------------------------------------------------------------------
+# attention
+# --------------------------------------------------------------------------
+@dataclass
+class AttnProblem:
+    """q [B,T,H,D]; k, v [B,Tk,Hkv,D] float32 arrays (bf16-exact when ``bf16``)."""
+
+    q: np.ndarray
+    k: np.ndarray
+    v: np.ndarray
+    causal: bool = False
+    key_lens: Optional[np.ndarray] = None  # [B] int
+    key_mask: Optional[np.ndarray] = None  # [B, Tk] nonzero = visible
+    window: Optional[tuple] = None
+    scale: Optional[float] = None
+    bf16: bool = True
+
+    def dims(self):
+        b, t, h, d = self.q.shape
+        _, tk, hkv, _ = self.k.shape
+        return b, t, tk, h, hkv, d
+
+    def scale_f32(self) -> float:
+        d = self.q.shape[-1]
+        # tk/src/ops/attention.rs:230: 1.0 / (d as f32).sqrt()
+        return float(self.scale) if self.scale is not None else float(np.float32(1.0) / np.sqrt(np.float32(d)))
+
+    def _common(self):
+        b, t, tk, h, hkv, d = self.dims()
+        lens = None if self.key_lens is None else np.ascontiguousarray(self.key_lens, dtype=np.int32)
+        mask = None if self.key_mask is None else np.ascontiguousarray(np.asarray(self.key_mask) != 0, dtype=np.int32)
+        wl, wr = (-1, -1) if self.window is None else self.window
+        keep = (lens, mask)
+        args = [b, t, tk, h, hkv, d, int(self.causal), wl, wr, ctypes.c_float(self.scale_f32()),
+                _ptr(lens, _i32p), _ptr(mask, _i32p), tk]
+        return args, keep
+
+
+def attention_direct(p: AttnProblem, threads: int = 8) -> np.ndarray:
+    """f64 direct softmax (tk/src/test/unit/attention.rs:102-178); unrounded float64 [B,T,H,D]."""
+    q, k, v = _f32(p.q), _f32(p.k), _f32(p.v)
+    out = np.empty(q.shape, dtype=np.float64)
+    args, _keep = p._common()
+    rc = lib().svod_oracle_attention_direct(*args, _ptr(q, _f32p), _ptr(k, _f32p), _ptr(v, _f32p), _ptr(out, _f64p), threads)
+    if rc:
+        raise ValueError(f"oracle attention_direct rejected the problem (rc={rc})")
+    return out
+
+
+def attention_graph(p: AttnProblem, threads: int = 8) -> np.ndarray:
+    """The op's graph fallback (tk/src/ops/attention.rs:496-584); float32 [B,T,H,D]."""
+    q, k, v = _f32(p.q), _f32(p.k), _f32(p.v)
+    out = np.empty(q.shape, dtype=np.float32)
+    args, _keep = p._common()
+    rc = lib().svod_oracle_attention_graph(*args, int(p.bf16), _ptr(q, _f32p), _ptr(k, _f32p), _ptr(v, _f32p), _ptr(out, _f32p), threads)
+    if rc:
+        raise ValueError(f"oracle attention_graph rejected the problem (rc={rc})")
+    return out
+
+
+def attention_flash(p: AttnProblem, bq: int = 64, bkv: int = 64, threads: int = 8) -> np.ndarray:
+    """The tile program under the host interpreter (tk/src/kernels/attention.rs:381-450,466-924)."""
+    q, k, v = _f32(p.q), _f32(p.k), _f32(p.v)
+    out = np.zeros(q.shape, dtype=np.float32)
+    args, _keep = p._common()
+    rc = lib().svod_oracle_attention_flash(*args, int(p.bf16), bq, bkv, _ptr(q, _f32p), _ptr(k, _f32p), _ptr(v, _f32p), _ptr(out, _f32p), threads)
+    if rc:
+        raise ValueError(f"oracle attention_flash rejected the problem (rc={rc})")
+    return out
+
+
+def visible(batch, t, tk, causal=False, key_lens=None, key_mask=None, window=None) -> np.ndarray:
+    """uint8 [B,T,Tk]: 1 where key j is visible to query i (negated ``hidden`` of attention.rs:138-148)."""
+    lens = None if key_lens is None else np.ascontiguousarray(key_lens, dtype=np.int32)
+    mask = None if key_mask is None else np.ascontiguousarray(np.asarray(key_mask) != 0, dtype=np.int32)
+    wl, wr = (-1, -1) if window is None else window
+    out = np.empty((batch, t, tk), dtype=np.uint8)
+    lib().svod_oracle_visible(batch, t, tk, int(causal), wl, wr, _ptr(lens, _i32p), _ptr(mask, _i32p), tk, _ptr(out, _u8p))
+    return out
+
+
+def visible_pairs(batch, t, tk, causal=False, key_lens=None) -> int:
+    lens = None if key_lens is None else np.ascontiguousarray(key_lens, dtype=np.int32)
+    return int(lib().svod_oracle_visible_pairs(batch, t, tk, int(causal), _ptr(lens, _i32p)))
+
+
+# --------------------------------------------------------------------------
+# prologue
+# --------------------------------------------------------------------------
+@dataclass
+class HeadsProblem:
+    """qkv [B,T,(H+2Hkv)*D] float32 (bf16-exact); weights [D]; tables [T,D/2] or [B,T,D/2]."""
+
+    qkv: np.ndarray
+    heads: int
+    kv_heads: int
+    head_dim: int
+    q_w: Optional[np.ndarray] = None
+    k_w: Optional[np.ndarray] = None
+    eps: float = 1e-6
+    cos: Optional[np.ndarray] = None
+    sin: Optional[np.ndarray] = None
+
+    def rope_kind(self) -> int:
+        if self.cos is None:
+            return 0
+        b, t, _ = self.qkv.shape
+        rows = int(np.prod(self.cos.shape)) // (self.head_dim // 2)
+        if rows == t:
+            return 1
+        if rows == b * t:
+            return 2
+        raise ValueError("rope tables must hold t or batch*t rows")
+
+
+def _heads(fn_name: str, p: HeadsProblem):
+    b, t, width = p.qkv.shape
+    h, hkv, d = p.heads, p.kv_heads, p.head_dim
+    assert width == (h + 2 * hkv) * d
+    qkv = _f32(p.qkv)
+    q_w = None if p.q_w is None else _f32(p.q_w)
+    k_w = None if p.k_w is None else _f32(p.k_w)
+    cos = None if p.cos is None else _f32(p.cos)
+    sin = None if p.sin is None else _f32(p.sin)
+    q = np.zeros((b, t, h, d), dtype=np.float32)
+    k = np.zeros((b, t, hkv, d), dtype=np.float32)
+    v = np.zeros((b, t, hkv, d), dtype=np.float32)
+    rc = getattr(lib(), fn_name)(b, t, h, hkv, d, int(q_w is not None), int(k_w is not None), p.eps, p.rope_kind(),
+                                 _ptr(qkv, _f32p), _ptr(q_w, _f32p), _ptr(k_w, _f32p), _ptr(cos, _f32p), _ptr(sin, _f32p),
+                                 _ptr(q, _f32p), _ptr(k, _f32p), _ptr(v, _f32p))
+    if rc:
+        raise ValueError(f"oracle {fn_name} rejected the problem (rc={rc})")
+    return q, k, v
+
+
+def heads_direct(p: HeadsProblem):
+    """f64 reference rounded to bf16 at the store (tk/src/test/unit/heads.rs:59-105)."""
+    return _heads("svod_oracle_heads_direct", p)
+
+
+def heads_kernel(p: HeadsProblem):
+    """heads_body under the interpreter's f32 rounding (tk/src/kernels/heads.rs:73-124)."""
+    return _heads("svod_oracle_heads_kernel", p)
+
+
+def heads_graph(p: HeadsProblem):
+    """The op's graph fallback (tk/src/ops/heads.rs:115-134)."""
+    return _heads("svod_oracle_heads_graph", p)

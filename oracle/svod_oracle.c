@@ -1,0 +1,722 @@
+/*
+ * TEST INFRASTRUCTURE — NOT PRODUCT CODE.
+ *
+ * CPU restatement of the arithmetic of Svod's `tk` flash-attention forward op
+ * and of the attention prologue ("heads") that feeds it.  Only the tests, the
+ * smoke check and the CPU-baseline leg of the benchmark may load this file's
+ * library; the shipped HIP path never does.
+ *
+ * The reference is Rust and cannot be built in this environment, so every
+ * function restates reference source read as text and says which lines it
+ * follows (paths are relative to the reference checkout).
+ *
+ * Pinning status (what independent evidence fixes each function):
+ *   svod_oracle_round_bf16 / _bf16_bits / _trunc_bf16
+ *       pinned by the reference's own known-answer tests
+ *       (tk/src/test/unit/interp.rs:197-216) and by torch's bf16 cast.
+ *   svod_oracle_lcg / _lcg_fill
+ *       pinned by the recurrence constants (tk/src/test/unit/mod.rs:442-445)
+ *       and an independent big-integer evaluation in Python.
+ *   svod_oracle_visible
+ *       pinned by brute-force enumeration of the predicate on tiny shapes.
+ *   svod_oracle_attention_direct
+ *       pinned against torch.nn.functional.scaled_dot_product_attention in
+ *       float64 (a library routine, not the reference) and closed forms
+ *       (uniform scores -> mean of visible V; one visible key -> that V row;
+ *       fully hidden row -> zeros).
+ *   svod_oracle_attention_graph, svod_oracle_attention_flash
+ *       pinned against svod_oracle_attention_direct within the tolerances the
+ *       reference holds itself to (tk/src/test/unit/attention.rs:483,
+ *       tk/src/test/unit/mod.rs:526-536), plus the online-softmax normaliser
+ *       identity of tk/src/test/unit/interp.rs:144-179.  The f32 accumulation
+ *       ORDER of the reference's compiled CPU kernels is not observable from
+ *       source: bit patterns of these two are "parity unpinned" below 1e-6 rel.
+ *   svod_oracle_heads_direct
+ *       pinned by closed forms (unit-norm rows, rotation preserves pair norm,
+ *       v passes through) and an independent numpy float64 evaluation.
+ *   svod_oracle_heads_kernel, svod_oracle_heads_graph
+ *       pinned against svod_oracle_heads_direct within 2e-2 / 1e-2
+ *       (tk/src/test/unit/heads.rs:124,159); v is bit-exact.
+ *   svod_oracle_rope_table
+ *       restates tensor/src/transformer.rs:130-164 with libm powf/cosf/sinf;
+ *       the reference evaluates pow/cos/sin through its own f32 graph
+ *       lowering, so the last bit of a table entry is "parity unpinned".
+ *       Tables are an INPUT of the prologue op, so this affects only the
+ *       synthetic benchmark inputs, not op parity.
+ */
+#include <math.h>
+#include <pthread.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+/* ------------------------------------------------------------------ */
+/* rounding: tk/src/interp.rs:37-44 (round_to, BFloat16 arm)           */
+/* ------------------------------------------------------------------ */
+static inline uint32_t f32_bits(float x) {
+  uint32_t b;
+  memcpy(&b, &x, 4);
+  return b;
+}
+static inline float bits_f32(uint32_t b) {
+  float x;
+  memcpy(&x, &b, 4);
+  return x;
+}
+
+/* bits + 0x7fff + ((bits >> 16) & 1), low half cleared; a NaN is quieted. */
+static inline float round_bf16_f32(float x) {
+  uint32_t bits = f32_bits(x);
+  if (x != x) return bits_f32((bits | 0x00400000u) & 0xffff0000u);
+  uint32_t rounded = (bits + 0x7fffu + ((bits >> 16) & 1u)) & 0xffff0000u;
+  return bits_f32(rounded);
+}
+
+double svod_oracle_round_bf16(double x) { return (double)round_bf16_f32((float)x); }
+
+uint16_t svod_oracle_bf16_bits(float x) { return (uint16_t)(f32_bits(round_bf16_f32(x)) >> 16); }
+
+/* tk/src/interp.rs TileOp::Cast with Round::Zero: the low 16 bits dropped. */
+double svod_oracle_trunc_bf16(double x) { return (double)bits_f32(f32_bits((float)x) & 0xffff0000u); }
+
+/* ------------------------------------------------------------------ */
+/* deterministic inputs: tk/src/test/unit/mod.rs:442-450               */
+/* ------------------------------------------------------------------ */
+double svod_oracle_lcg(uint64_t *seed) {
+  *seed = *seed * 6364136223846793005ULL + 1442695040888963407ULL;
+  return ((double)(*seed >> 33) / (double)(1ULL << 31)) * 2.0 - 1.0;
+}
+
+/* `rounded(dtype, n, seed, |x| mul*x + add)`: n draws, each mapped and, when
+ * `to_bf16` is set, rounded to bf16.  Returns the advanced seed. */
+uint64_t svod_oracle_lcg_fill(float *out, int64_t n, uint64_t seed, double mul, double add, int to_bf16) {
+  for (int64_t i = 0; i < n; i++) {
+    double v = mul * svod_oracle_lcg(&seed) + add;
+    out[i] = to_bf16 ? round_bf16_f32((float)v) : (float)v;
+  }
+  return seed;
+}
+
+/* Standard normals by Box-Muller over the same LCG (two uniforms on (0,1] and
+ * [0,1) per pair), scaled by `sigma`; optional bf16 rounding.  Not a reference
+ * function: the benchmark configs ask for N(0,1) data "from a seed". */
+uint64_t svod_oracle_normal_fill(float *out, int64_t n, uint64_t seed, double sigma, int to_bf16) {
+  for (int64_t i = 0; i < n; i += 2) {
+    double u1 = (svod_oracle_lcg(&seed) + 1.0) * 0.5;
+    double u2 = (svod_oracle_lcg(&seed) + 1.0) * 0.5;
+    u1 = 1.0 - u1; /* (0, 1] so the log is finite */
+    double r = sqrt(-2.0 * log(u1)), a = 6.283185307179586476925286766559 * u2;
+    double z0 = sigma * r * cos(a), z1 = sigma * r * sin(a);
+    out[i] = to_bf16 ? round_bf16_f32((float)z0) : (float)z0;
+    if (i + 1 < n) out[i + 1] = to_bf16 ? round_bf16_f32((float)z1) : (float)z1;
+  }
+  return seed;
+}
+
+/* ------------------------------------------------------------------ */
+/* rotary tables: tensor/src/transformer.rs:130-164                    */
+/* inv_freq[i] = theta^(-2i/d) in f32, angle = pos * inv_freq in f32,  */
+/* cos/sin in f32, cast last (the cast is the caller's).               */
+/* ------------------------------------------------------------------ */
+void svod_oracle_rope_table(double theta, int32_t seq_len, int32_t head_dim, float *cos_out, float *sin_out) {
+  int32_t half = head_dim / 2;
+  float step = (float)(-2.0 / (double)head_dim);
+  for (int32_t s = 0; s < seq_len; s++) {
+    for (int32_t i = 0; i < half; i++) {
+      float exponent = (float)i * step;
+      float inv_freq = powf((float)theta, exponent);
+      float angle = (float)s * inv_freq;
+      cos_out[(int64_t)s * half + i] = cosf(angle);
+      sin_out[(int64_t)s * half + i] = sinf(angle);
+    }
+  }
+}
+
+/* ------------------------------------------------------------------ */
+/* the attention problem                                               */
+/* ------------------------------------------------------------------ */
+typedef struct {
+  int32_t batch, t, tk, heads, kv_heads, d;
+  int32_t causal;
+  int32_t window_left, window_right; /* < 0: no window */
+  float scale;
+  const int32_t *key_lens; /* [batch] or NULL */
+  const int32_t *key_mask; /* [batch, mask_stride], nonzero = visible, or NULL */
+  int32_t mask_stride;
+  int32_t bf16_stream; /* 1: q/k/v/o are bf16 values; 0: f32 */
+} attn_problem;
+
+/* hidden(j) of tk/src/test/unit/attention.rs:138-148, the in-scope arms:
+ * j >= len || (causal && j > i) || window || key_mask == 0.
+ * The kernel's keep predicate (tk/src/kernels/attention.rs:641-697) is its
+ * negation: col <= row, col < len (len = min(key_lens[b], tk), L533-536),
+ * row <= col + left && col <= row + right, key_mask != 0. */
+static inline int hidden(const attn_problem *p, int32_t b, int32_t i, int32_t j) {
+  int32_t len = p->tk;
+  if (p->key_lens) {
+    len = p->key_lens[b];
+    if (len > p->tk) len = p->tk;
+  }
+  if (j >= len) return 1;
+  if (p->causal && j > i) return 1;
+  if (p->window_left >= 0 && (j + p->window_left < i || j > i + p->window_right)) return 1;
+  if (p->key_mask && p->key_mask[(int64_t)b * p->mask_stride + j] == 0) return 1;
+  return 0;
+}
+
+/* Visibility of every (b, i, j): out[b][i][j] = 1 where key j is seen by query i. */
+void svod_oracle_visible(int32_t batch, int32_t t, int32_t tk, int32_t causal, int32_t window_left,
+                         int32_t window_right, const int32_t *key_lens, const int32_t *key_mask, int32_t mask_stride,
+                         uint8_t *out) {
+  attn_problem p = {batch, t, tk, 1, 1, 1, causal, window_left, window_right, 1.0f, key_lens, key_mask, mask_stride, 0};
+  for (int32_t b = 0; b < batch; b++)
+    for (int32_t i = 0; i < t; i++)
+      for (int32_t j = 0; j < tk; j++) out[((int64_t)b * t + i) * tk + j] = (uint8_t)!hidden(&p, b, i, j);
+}
+
+/* ------------------------------------------------------------------ */
+/* a small (b, h) work pool                                            */
+/* ------------------------------------------------------------------ */
+typedef void (*slice_fn)(const void *ctx, int32_t b, int32_t h);
+typedef struct {
+  slice_fn fn;
+  const void *ctx;
+  int32_t batch, heads;
+  int64_t *next;
+  pthread_mutex_t *lock;
+} pool_arg;
+
+static void *pool_main(void *argp) {
+  pool_arg *a = (pool_arg *)argp;
+  for (;;) {
+    pthread_mutex_lock(a->lock);
+    int64_t item = (*a->next)++;
+    pthread_mutex_unlock(a->lock);
+    if (item >= (int64_t)a->batch * a->heads) break;
+    a->fn(a->ctx, (int32_t)(item / a->heads), (int32_t)(item % a->heads));
+  }
+  return NULL;
+}
+
+static void run_slices(slice_fn fn, const void *ctx, int32_t batch, int32_t heads, int32_t threads) {
+  if (threads < 1) threads = 1;
+  int64_t next = 0;
+  pthread_mutex_t lock = PTHREAD_MUTEX_INITIALIZER;
+  pool_arg arg = {fn, ctx, batch, heads, &next, &lock};
+  if (threads == 1) {
+    pool_main(&arg);
+    return;
+  }
+  pthread_t *ids = (pthread_t *)malloc(sizeof(pthread_t) * (size_t)threads);
+  int started = 0;
+  for (int i = 0; i < threads; i++)
+    if (pthread_create(&ids[i], NULL, pool_main, &arg) == 0) ids[started++] = ids[i];
+  if (started == 0) pool_main(&arg);
+  for (int i = 0; i < started; i++) pthread_join(ids[i], NULL);
+  free(ids);
+}
+
+/* ------------------------------------------------------------------ */
+/* direct softmax in f64: tk/src/test/unit/attention.rs:102-178        */
+/* ------------------------------------------------------------------ */
+typedef struct {
+  attn_problem p;
+  const float *q, *k, *v;
+  double *out;
+} direct_ctx;
+
+static void direct_slice(const void *ctxp, int32_t b, int32_t h) {
+  const direct_ctx *c = (const direct_ctx *)ctxp;
+  const attn_problem *p = &c->p;
+  int32_t d = p->d, group = p->heads / p->kv_heads, kv_head = h / group;
+  int64_t stride = (int64_t)p->heads * d, kv_stride = (int64_t)p->kv_heads * d;
+  double *scores = (double *)malloc(sizeof(double) * (size_t)p->tk);
+  for (int32_t i = 0; i < p->t; i++) {
+    const float *qi = c->q + ((int64_t)b * p->t + i) * stride + (int64_t)h * d;
+    double *oi = c->out + ((int64_t)b * p->t + i) * stride + (int64_t)h * d;
+    double mx = -INFINITY;
+    for (int32_t j = 0; j < p->tk; j++) {
+      if (hidden(p, b, i, j)) {
+        scores[j] = -INFINITY;
+        continue;
+      }
+      const float *kj = c->k + ((int64_t)b * p->tk + j) * kv_stride + (int64_t)kv_head * d;
+      double dot = 0.0;
+      for (int32_t dd = 0; dd < d; dd++) dot += (double)qi[dd] * (double)kj[dd];
+      scores[j] = dot * (double)p->scale;
+      if (scores[j] > mx) mx = scores[j];
+    }
+    for (int32_t dd = 0; dd < d; dd++) oi[dd] = 0.0;
+    /* A query no key reaches attends to nothing: zeros (L162-165). */
+    if (mx == -INFINITY) continue;
+    double l = 0.0;
+    for (int32_t j = 0; j < p->tk; j++) {
+      scores[j] = exp(scores[j] - mx);
+      l += scores[j];
+    }
+    for (int32_t j = 0; j < p->tk; j++) {
+      if (scores[j] == 0.0) continue;
+      const float *vj = c->v + ((int64_t)b * p->tk + j) * kv_stride + (int64_t)kv_head * d;
+      for (int32_t dd = 0; dd < d; dd++) oi[dd] += scores[j] * (double)vj[dd];
+    }
+    for (int32_t dd = 0; dd < d; dd++) oi[dd] /= l;
+  }
+  free(scores);
+}
+
+static int check_problem(const attn_problem *p) {
+  if (p->batch < 0 || p->t <= 0 || p->tk <= 0 || p->heads <= 0 || p->kv_heads <= 0 || p->d <= 0) return -1;
+  if (p->heads % p->kv_heads != 0) return -3;
+  return 0;
+}
+
+/* q [B,T,H,D], k/v [B,Tk,Hkv,D] as f32 arrays (bf16-exact values when the
+ * stream is bf16); out [B,T,H,D] f64, unrounded. */
+int svod_oracle_attention_direct(int32_t batch, int32_t t, int32_t tk, int32_t heads, int32_t kv_heads, int32_t d,
+                                 int32_t causal, int32_t window_left, int32_t window_right, float scale,
+                                 const int32_t *key_lens, const int32_t *key_mask, int32_t mask_stride, const float *q,
+                                 const float *k, const float *v, double *out, int32_t threads) {
+  direct_ctx c = {{batch, t, tk, heads, kv_heads, d, causal, window_left, window_right, scale, key_lens, key_mask,
+                   mask_stride, 0},
+                  q, k, v, out};
+  int rc = check_problem(&c.p);
+  if (rc) return rc;
+  run_slices(direct_slice, &c, batch, heads, threads);
+  return 0;
+}
+
+/* ------------------------------------------------------------------ */
+/* the op's graph fallback: tk/src/ops/attention.rs:496-584 ->         */
+/* tensor/src/transformer.rs:358-531.  This is "the reference CPU      */
+/* path" the GPU kernel is timed beside.                               */
+/*   scores = sum_d (q*k)  with the product in the stream dtype and    */
+/*            the sum in f32 (tensor/src/matmul.rs:116-127,            */
+/*            tensor/src/reduce.rs:101-117), then * scale in f32       */
+/*   where(keep, scores, f32::MIN)            (transformer.rs:509-512) */
+/*   softmax = exp(x - max) / sum             (activation.rs:124-136)  */
+/*   masked weights re-zeroed                 (transformer.rs:517-525) */
+/*   weights cast to the stream dtype         (transformer.rs:526-529) */
+/*   out = sum_j (w*v) product in the stream dtype, f32 sum, cast      */
+/* ------------------------------------------------------------------ */
+typedef struct {
+  attn_problem p;
+  const float *q, *k, *v;
+  float *out;
+} graph_ctx;
+
+static void graph_slice(const void *ctxp, int32_t b, int32_t h) {
+  const graph_ctx *c = (const graph_ctx *)ctxp;
+  const attn_problem *p = &c->p;
+  const int32_t d = p->d, tk = p->tk, group = p->heads / p->kv_heads, kv_head = h / group;
+  const int64_t stride = (int64_t)p->heads * d, kv_stride = (int64_t)p->kv_heads * d;
+  const int bf = p->bf16_stream;
+  float *row = (float *)malloc(sizeof(float) * (size_t)tk);
+  uint8_t *keep = (uint8_t *)malloc((size_t)tk);
+  float *acc = (float *)malloc(sizeof(float) * (size_t)d);
+  /* K of this head gathered once so the inner loops stream. */
+  float *kh = (float *)malloc(sizeof(float) * (size_t)tk * (size_t)d);
+  float *vh = (float *)malloc(sizeof(float) * (size_t)tk * (size_t)d);
+  for (int32_t j = 0; j < tk; j++) {
+    memcpy(kh + (int64_t)j * d, c->k + ((int64_t)b * tk + j) * kv_stride + (int64_t)kv_head * d, sizeof(float) * (size_t)d);
+    memcpy(vh + (int64_t)j * d, c->v + ((int64_t)b * tk + j) * kv_stride + (int64_t)kv_head * d, sizeof(float) * (size_t)d);
+  }
+  const float fmin32 = -3.40282346638528859811704183484516925e+38f; /* f32::MIN */
+  for (int32_t i = 0; i < p->t; i++) {
+    const float *qi = c->q + ((int64_t)b * p->t + i) * stride + (int64_t)h * d;
+    float *oi = c->out + ((int64_t)b * p->t + i) * stride + (int64_t)h * d;
+    int any_mask = p->causal || p->window_left >= 0 || p->key_lens || p->key_mask;
+    float mx = -INFINITY;
+    for (int32_t j = 0; j < tk; j++) {
+      const float *kj = kh + (int64_t)j * d;
+      float s = 0.0f;
+      if (bf)
+        for (int32_t dd = 0; dd < d; dd++) s += round_bf16_f32(qi[dd] * kj[dd]);
+      else
+        for (int32_t dd = 0; dd < d; dd++) s += qi[dd] * kj[dd];
+      s *= p->scale;
+      keep[j] = (uint8_t)(!any_mask || !hidden(p, b, i, j));
+      if (!keep[j]) s = fmin32;
+      row[j] = s;
+      if (s > mx) mx = s;
+    }
+    float sum = 0.0f;
+    for (int32_t j = 0; j < tk; j++) {
+      row[j] = expf(row[j] - mx);
+      sum += row[j];
+    }
+    for (int32_t j = 0; j < tk; j++) {
+      float w = keep[j] ? row[j] / sum : 0.0f;
+      row[j] = bf ? round_bf16_f32(w) : w;
+    }
+    for (int32_t dd = 0; dd < d; dd++) acc[dd] = 0.0f;
+    for (int32_t j = 0; j < tk; j++) {
+      float w = row[j];
+      if (w == 0.0f) continue; /* +0 products leave an f32 sum unchanged */
+      const float *vj = vh + (int64_t)j * d;
+      if (bf)
+        for (int32_t dd = 0; dd < d; dd++) acc[dd] += round_bf16_f32(w * vj[dd]);
+      else
+        for (int32_t dd = 0; dd < d; dd++) acc[dd] += w * vj[dd];
+    }
+    for (int32_t dd = 0; dd < d; dd++) oi[dd] = bf ? round_bf16_f32(acc[dd]) : acc[dd];
+  }
+  free(row);
+  free(keep);
+  free(acc);
+  free(kh);
+  free(vh);
+}
+
+/* out [B,T,H,D] f32 (bf16-exact values when the stream is bf16).  Only the
+ * (b, h) slices with b in [b0, b1) are computed, so a benchmark can time a
+ * bounded sample of a large problem. */
+int svod_oracle_attention_graph(int32_t batch, int32_t t, int32_t tk, int32_t heads, int32_t kv_heads, int32_t d,
+                                int32_t causal, int32_t window_left, int32_t window_right, float scale,
+                                const int32_t *key_lens, const int32_t *key_mask, int32_t mask_stride,
+                                int32_t bf16_stream, const float *q, const float *k, const float *v, float *out,
+                                int32_t threads) {
+  graph_ctx c = {{batch, t, tk, heads, kv_heads, d, causal, window_left, window_right, scale, key_lens, key_mask,
+                  mask_stride, bf16_stream},
+                 q, k, v, out};
+  int rc = check_problem(&c.p);
+  if (rc) return rc;
+  run_slices(graph_slice, &c, batch, heads, threads);
+  return 0;
+}
+
+/* ------------------------------------------------------------------ */
+/* the tile program under the host interpreter:                        */
+/* tk/src/kernels/attention.rs:466-924 (blocks, masks, store) and      */
+/* :381-450 (step), evaluated as tk/src/interp.rs does — every tile op */
+/* in f64, rounded to its dtype (f32 state, stream-dtype P), and an    */
+/* MMA as `held as f32 + (f64 sum over k) as f32` (interp.rs:393-414). */
+/* Forms are the planned ones (FaCfg::new: all off), splits = 1,       */
+/* key_warps = 1.                                                      */
+/* ------------------------------------------------------------------ */
+typedef struct {
+  attn_problem p;
+  int32_t bq, bkv;
+  const float *q, *k, *v;
+  float *out;
+} flash_ctx;
+
+static inline double r32(double x) { return (double)(float)x; }
+
+static void flash_slice(const void *ctxp, int32_t b, int32_t h) {
+  const flash_ctx *c = (const flash_ctx *)ctxp;
+  const attn_problem *p = &c->p;
+  const int32_t d = p->d, t = p->t, tk = p->tk, bq = c->bq, bkv = c->bkv;
+  const int32_t group = p->heads / p->kv_heads, kv_head = h / group;
+  const int64_t stride = (int64_t)p->heads * d, kv_stride = (int64_t)p->kv_heads * d;
+  const int bf = p->bf16_stream;
+  /* L533-536: keys past the length are masked; past tk too when blocks overhang. */
+  const int keys_masked = p->key_lens != NULL || (tk % bkv) != 0;
+  int32_t len = tk;
+  if (p->key_lens) {
+    len = p->key_lens[b];
+    if (len > tk) len = tk;
+  }
+  /* L619: (scale * LOG2_E) evaluated in f32. */
+  const double scale_log2e = (double)(p->scale * 1.44269504088896340736f);
+  double *m = (double *)malloc(sizeof(double) * (size_t)bq);
+  double *l = (double *)malloc(sizeof(double) * (size_t)bq);
+  double *o = (double *)malloc(sizeof(double) * (size_t)bq * (size_t)d);
+  double *s = (double *)malloc(sizeof(double) * (size_t)bq * (size_t)bkv);
+  double *p16 = (double *)malloc(sizeof(double) * (size_t)bq * (size_t)bkv);
+  for (int32_t q_off = 0; q_off < t; q_off += bq) {
+    /* L584-612: the key blocks some query of the tile sees. */
+    int32_t first = 0, end = (tk + bkv - 1) / bkv;
+    if (p->window_left >= 0) {
+      int32_t lo = (q_off > p->window_left ? q_off : p->window_left) - p->window_left;
+      if (lo / bkv > first) first = lo / bkv;
+    }
+    if (p->causal) {
+      int32_t e = (q_off + bq + bkv - 1) / bkv;
+      if (e < end) end = e;
+    }
+    if (p->window_left >= 0) {
+      int32_t e = (q_off + bq + p->window_right + bkv - 1) / bkv;
+      if (e < end) end = e;
+    }
+    if (p->key_lens) {
+      int32_t e = (len + bkv - 1) / bkv;
+      if (e < end) end = e;
+    }
+    for (int32_t r = 0; r < bq; r++) {
+      m[r] = (double)(float)-1e30; /* L616 */
+      l[r] = 0.0;
+      for (int32_t dd = 0; dd < d; dd++) o[(int64_t)r * d + dd] = 0.0;
+    }
+    for (int32_t blk = first; blk < end; blk++) {
+      const int32_t k0 = blk * bkv;
+      /* s = q . k^T, rows past t and keys past the view's bound read as zero. */
+      for (int32_t r = 0; r < bq; r++) {
+        const int32_t i = q_off + r;
+        for (int32_t cc = 0; cc < bkv; cc++) {
+          const int32_t j = k0 + cc;
+          double dot = 0.0;
+          const int in_k = keys_masked ? (j < len) : 1;
+          if (i < t && in_k && j < tk) {
+            const float *qi = c->q + ((int64_t)b * t + i) * stride + (int64_t)h * d;
+            const float *kj = c->k + ((int64_t)b * tk + j) * kv_stride + (int64_t)kv_head * d;
+            for (int32_t dd = 0; dd < d; dd++) dot += (double)qi[dd] * (double)kj[dd];
+          }
+          double sv = r32(0.0f + (float)dot);
+          sv = r32(sv * scale_log2e);
+          /* L641-697: a hidden score is -inf.  Applying the predicate on every
+           * block equals applying it on edge blocks only (L698-733): on an
+           * interior block every key is kept. */
+          if (j >= tk || hidden(p, b, i, j)) sv = -INFINITY;
+          s[(int64_t)r * bkv + cc] = sv;
+        }
+      }
+      for (int32_t r = 0; r < bq; r++) {
+        double block_max = -INFINITY;
+        for (int32_t cc = 0; cc < bkv; cc++)
+          if (s[(int64_t)r * bkv + cc] > block_max) block_max = s[(int64_t)r * bkv + cc];
+        /* L418-427: lazy rescale, RESCALE_ABOVE = 8 (L379). */
+        const double m_max = m[r] > block_max ? m[r] : block_max;
+        const double growth = r32(m_max - m[r]);
+        const double m_new = (8.0 < growth) ? m_max : m[r];
+        const double corr = r32(exp2(r32(m[r] - m_new)));
+        double block_sum = 0.0;
+        for (int32_t cc = 0; cc < bkv; cc++) {
+          const double e = r32(exp2(r32(s[(int64_t)r * bkv + cc] - m_new)));
+          block_sum += e;
+          p16[(int64_t)r * bkv + cc] = bf ? (double)round_bf16_f32((float)e) : e;
+        }
+        block_sum = r32(block_sum);
+        l[r] = r32(r32(l[r] * corr) + block_sum);
+        m[r] = m_new;
+        for (int32_t dd = 0; dd < d; dd++) o[(int64_t)r * d + dd] = r32(o[(int64_t)r * d + dd] * corr);
+      }
+      /* o += p16 . v ; V rows past the view's bound read as zero. */
+      for (int32_t r = 0; r < bq; r++) {
+        for (int32_t dd = 0; dd < d; dd++) {
+          double dot = 0.0;
+          for (int32_t cc = 0; cc < bkv; cc++) {
+            const int32_t j = k0 + cc;
+            const int in_k = keys_masked ? (j < len) : 1;
+            if (!in_k || j >= tk) continue;
+            const double pv = p16[(int64_t)r * bkv + cc];
+            if (pv == 0.0) continue;
+            dot += pv * (double)c->v[((int64_t)b * tk + j) * kv_stride + (int64_t)kv_head * d + dd];
+          }
+          o[(int64_t)r * d + dd] = (double)((float)o[(int64_t)r * d + dd] + (float)dot);
+        }
+      }
+    }
+    /* L974-980 normalized, cast, bounded store. */
+    for (int32_t r = 0; r < bq; r++) {
+      const int32_t i = q_off + r;
+      if (i >= t) break;
+      const double ll = (l[r] == 0.0) ? 1.0 : l[r];
+      float *oi = c->out + ((int64_t)b * t + i) * stride + (int64_t)h * d;
+      for (int32_t dd = 0; dd < d; dd++) {
+        const float val = (float)r32(o[(int64_t)r * d + dd] / ll);
+        oi[dd] = bf ? round_bf16_f32(val) : val;
+      }
+    }
+  }
+  free(m);
+  free(l);
+  free(o);
+  free(s);
+  free(p16);
+}
+
+int svod_oracle_attention_flash(int32_t batch, int32_t t, int32_t tk, int32_t heads, int32_t kv_heads, int32_t d,
+                                int32_t causal, int32_t window_left, int32_t window_right, float scale,
+                                const int32_t *key_lens, const int32_t *key_mask, int32_t mask_stride,
+                                int32_t bf16_stream, int32_t bq, int32_t bkv, const float *q, const float *k,
+                                const float *v, float *out, int32_t threads) {
+  flash_ctx c = {{batch, t, tk, heads, kv_heads, d, causal, window_left, window_right, scale, key_lens, key_mask,
+                  mask_stride, bf16_stream},
+                 bq, bkv, q, k, v, out};
+  int rc = check_problem(&c.p);
+  if (rc) return rc;
+  if (bq <= 0 || bkv <= 0) return -1;
+  run_slices(flash_slice, &c, batch, heads, threads);
+  return 0;
+}
+
+/* ------------------------------------------------------------------ */
+/* the prologue                                                        */
+/* ------------------------------------------------------------------ */
+typedef struct {
+  int32_t batch, t, heads, kv_heads, d;
+  int32_t q_norm, k_norm;
+  double eps;
+  int32_t rope; /* 0: none, 1: tables [t, d/2], 2: tables [batch*t, d/2] */
+} heads_problem;
+
+/* f64 reference, rounded to bf16 at the store: tk/src/test/unit/heads.rs:59-105. */
+int svod_oracle_heads_direct(int32_t batch, int32_t t, int32_t heads, int32_t kv_heads, int32_t d, int32_t q_norm,
+                             int32_t k_norm, double eps, int32_t rope, const float *qkv, const float *q_w,
+                             const float *k_w, const float *cos_t, const float *sin_t, float *q, float *k, float *v) {
+  if (kv_heads <= 0 || heads % kv_heads != 0 || d <= 0 || (d & 1)) return -1;
+  const int32_t slots = heads + 2 * kv_heads, half = d / 2;
+  double *x = (double *)malloc(sizeof(double) * (size_t)d);
+  double *y = (double *)malloc(sizeof(double) * (size_t)d);
+  for (int32_t b = 0; b < batch; b++)
+    for (int32_t i = 0; i < t; i++)
+      for (int32_t slot = 0; slot < slots; slot++) {
+        const float *src = qkv + (((int64_t)b * t + i) * slots + slot) * d;
+        for (int32_t c = 0; c < d; c++) x[c] = (double)src[c];
+        int which, head;
+        const float *w;
+        if (slot < heads) {
+          which = 0, head = slot, w = q_norm ? q_w : NULL;
+        } else if (slot < heads + kv_heads) {
+          which = 1, head = slot - heads, w = k_norm ? k_w : NULL;
+        } else {
+          which = 2, head = slot - heads - kv_heads, w = NULL;
+        }
+        if (w) {
+          double ss = 0.0;
+          for (int32_t c = 0; c < d; c++) ss += x[c] * x[c];
+          const double inv = 1.0 / sqrt(ss / (double)d + eps);
+          for (int32_t c = 0; c < d; c++) x[c] = x[c] * inv * (double)w[c];
+        }
+        if (rope && which < 2) {
+          const int64_t row = (rope == 2) ? (int64_t)b * t + i : i;
+          for (int32_t c = 0; c < d; c++) {
+            const double cs = (double)cos_t[row * half + c % half], sn = (double)sin_t[row * half + c % half];
+            y[c] = (c < half) ? x[c] * cs - x[c + half] * sn : x[c - half] * sn + x[c] * cs;
+          }
+          memcpy(x, y, sizeof(double) * (size_t)d);
+        }
+        const int32_t width = which == 0 ? heads : kv_heads;
+        float *dst = (which == 0 ? q : which == 1 ? k : v) + (((int64_t)b * t + i) * width + head) * d;
+        for (int32_t c = 0; c < d; c++) dst[c] = round_bf16_f32((float)x[c]);
+      }
+  free(x);
+  free(y);
+  return 0;
+}
+
+/* The tile program heads_body (tk/src/kernels/heads.rs:73-124) under the
+ * interpreter's rounding: every op in f64 then rounded to f32; Σ over the row
+ * summed in f64 then rounded (interp.rs Reduce); affine = (x*mul)+add as two
+ * rounded ops (tk/src/kernels/mod.rs:297-302); store rounds to bf16. */
+int svod_oracle_heads_kernel(int32_t batch, int32_t t, int32_t heads, int32_t kv_heads, int32_t d, int32_t q_norm,
+                             int32_t k_norm, double eps, int32_t rope, const float *qkv, const float *q_w,
+                             const float *k_w, const float *cos_t, const float *sin_t, float *q, float *k, float *v) {
+  if (kv_heads <= 0 || heads % kv_heads != 0 || d <= 0 || (d & 1)) return -1;
+  const int32_t slots = heads + 2 * kv_heads, half = d / 2;
+  for (int32_t b = 0; b < batch; b++)
+    for (int32_t i = 0; i < t; i++)
+      for (int32_t slot = 0; slot < slots; slot++) {
+        const float *src = qkv + (((int64_t)b * t + i) * slots + slot) * d;
+        int which, head;
+        const float *w;
+        if (slot < heads) {
+          which = 0, head = slot, w = q_norm ? q_w : NULL;
+        } else if (slot < heads + kv_heads) {
+          which = 1, head = slot - heads, w = k_norm ? k_w : NULL;
+        } else {
+          which = 2, head = slot - heads - kv_heads, w = NULL;
+        }
+        const int32_t width = which == 0 ? heads : kv_heads;
+        float *dst = (which == 0 ? q : which == 1 ? k : v) + (((int64_t)b * t + i) * width + head) * d;
+        double inv = 1.0;
+        if (w) {
+          double sum = 0.0;
+          for (int32_t c = 0; c < half; c++) {
+            const double x1 = (double)src[c], x2 = (double)src[c + half];
+            sum += r32(r32(x1 * x1) + r32(x2 * x2));
+          }
+          sum = r32(sum);
+          const double var = r32(r32(sum * (double)(float)(1.0 / (double)d)) + (double)(float)eps);
+          inv = r32(1.0 / sqrt(var));
+        }
+        const int64_t row = (rope == 2) ? (int64_t)b * t + i : i;
+        for (int32_t c = 0; c < half; c++) {
+          double y1 = (double)src[c], y2 = (double)src[c + half];
+          if (w) {
+            y1 = r32(r32(y1 * inv) * (double)w[c]);
+            y2 = r32(r32(y2 * inv) * (double)w[c + half]);
+          }
+          if (rope && which < 2) {
+            const double cs = (double)cos_t[row * half + c], sn = (double)sin_t[row * half + c];
+            const double c1 = r32(y1 * cs), s2 = r32(y2 * sn), s1 = r32(y1 * sn), c2 = r32(y2 * cs);
+            y1 = r32(c1 - s2);
+            y2 = r32(s1 + c2);
+          }
+          dst[c] = round_bf16_f32((float)y1);
+          dst[c + half] = round_bf16_f32((float)y2);
+        }
+      }
+  return 0;
+}
+
+/* The op's graph fallback: tk/src/ops/heads.rs:115-134.
+ *   rms_norm_with (tensor/src/nn/norm.rs:146-168): x32 = f32(x);
+ *     inv = rsqrt(mean(x32^2) + eps) in f32; (x32 * inv) * f32(w) -> ONE cast
+ *     to the stream dtype (nn/norm.rs:349-358).
+ *   apply_rotary_emb(cos, sin, false) (tensor/src/transformer.rs:72-117) then
+ *     runs in the stream dtype: each product and each sum rounds to bf16. */
+int svod_oracle_heads_graph(int32_t batch, int32_t t, int32_t heads, int32_t kv_heads, int32_t d, int32_t q_norm,
+                            int32_t k_norm, double eps, int32_t rope, const float *qkv, const float *q_w,
+                            const float *k_w, const float *cos_t, const float *sin_t, float *q, float *k, float *v) {
+  if (kv_heads <= 0 || heads % kv_heads != 0 || d <= 0 || (d & 1)) return -1;
+  const int32_t slots = heads + 2 * kv_heads, half = d / 2;
+  float *x = (float *)malloc(sizeof(float) * (size_t)d);
+  for (int32_t b = 0; b < batch; b++)
+    for (int32_t i = 0; i < t; i++)
+      for (int32_t slot = 0; slot < slots; slot++) {
+        const float *src = qkv + (((int64_t)b * t + i) * slots + slot) * d;
+        int which, head;
+        const float *w;
+        if (slot < heads) {
+          which = 0, head = slot, w = q_norm ? q_w : NULL;
+        } else if (slot < heads + kv_heads) {
+          which = 1, head = slot - heads, w = k_norm ? k_w : NULL;
+        } else {
+          which = 2, head = slot - heads - kv_heads, w = NULL;
+        }
+        memcpy(x, src, sizeof(float) * (size_t)d);
+        if (w) {
+          float ss = 0.0f;
+          for (int32_t c = 0; c < d; c++) ss += x[c] * x[c];
+          const float mean = ss / (float)d;
+          const float inv = 1.0f / sqrtf(mean + (float)eps);
+          for (int32_t c = 0; c < d; c++) x[c] = round_bf16_f32((x[c] * inv) * w[c]);
+        }
+        const int32_t width = which == 0 ? heads : kv_heads;
+        float *dst = (which == 0 ? q : which == 1 ? k : v) + (((int64_t)b * t + i) * width + head) * d;
+        if (rope && which < 2) {
+          const int64_t row = (rope == 2) ? (int64_t)b * t + i : i;
+          for (int32_t c = 0; c < half; c++) {
+            const float cs = cos_t[row * half + c], sn = sin_t[row * half + c];
+            const float x1 = x[c], x2 = x[c + half];
+            dst[c] = round_bf16_f32(round_bf16_f32(x1 * cs) - round_bf16_f32(x2 * sn));
+            dst[c + half] = round_bf16_f32(round_bf16_f32(x1 * sn) + round_bf16_f32(x2 * cs));
+          }
+        } else {
+          memcpy(dst, x, sizeof(float) * (size_t)d);
+        }
+      }
+  free(x);
+  return 0;
+}
+
+/* The count of (query, key) pairs visible in a problem: the honest work
+ * measure the roofline uses (4 * d * heads * pairs flops). */
+int64_t svod_oracle_visible_pairs(int32_t batch, int32_t t, int32_t tk, int32_t causal, const int32_t *key_lens) {
+  int64_t pairs = 0;
+  for (int32_t b = 0; b < batch; b++) {
+    int32_t len = tk;
+    if (key_lens) {
+      len = key_lens[b];
+      if (len > tk) len = tk;
+      if (len < 0) len = 0;
+    }
+    for (int32_t i = 0; i < t; i++) {
+      int32_t n = len;
+      if (causal && i + 1 < n) n = i + 1;
+      pairs += n;
+    }
+  }
+  return pairs;
+}

@@ -1,0 +1,25 @@
+"""MI355X (gfx950) flash-attention forward and attention prologue behind the
+contract of Svod's `tk` op layer.
+
+The package is a thin host binding: ``svod_amd.ops`` mirrors
+``svod_tk::ops::{attention, heads}`` (same operand layouts, option names and
+error behaviour) over the C ABI of ``include/svodk.h``; the arithmetic lives in
+the HIP kernels under ``csrc/``.  PyTorch is used for device memory and streams
+only.
+"""
+from .ops import (  # noqa: F401
+    Attn,
+    Fallback,
+    GraphFallback,
+    KeyMask,
+    OpError,
+    Qkv,
+    attention,
+    chosen,
+    heads,
+    library_path,
+    load_library,
+    plan_attention,
+    plan_heads,
+    supported,
+)

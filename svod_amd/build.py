@@ -1,0 +1,59 @@
+"""Builds ``libsvodk_gfx950.so`` in-tree with hipcc, for gfx950 only.
+
+``python -m svod_amd.build`` compiles every source under ``csrc/``.  The
+library is never built implicitly at import: loading fails loudly when it is
+missing, so a stale or absent build cannot hide behind another code path.
+"""
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB = os.path.join(HERE, "libsvodk_gfx950.so")
+SOURCES = ["ops.cpp", "heads_kernel.hip", "attention_kernel.hip"]
+
+# Packed-FP32 VALU ops are switched off for device code; the host pass of hipcc
+# does not know the feature and says so, which is harmless.
+DEVICE_FLAGS = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+COMMON_FLAGS = ["-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-command-line-argument"]
+
+
+def hipcc() -> str:
+    for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and os.path.exists(cand):
+            return cand
+    raise RuntimeError("hipcc not found (looked at $HIPCC, PATH and /opt/rocm/bin)")
+
+
+def build(verbose: bool = False) -> str:
+    cc = hipcc()
+    objdir = os.path.join(HERE, "build")
+    os.makedirs(objdir, exist_ok=True)
+    objs = []
+    for src in SOURCES:
+        obj = os.path.join(objdir, os.path.splitext(src)[0] + ".o")
+        cmd = [cc, "-x", "hip", *DEVICE_FLAGS, *COMMON_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+        _run(cmd, verbose)
+        objs.append(obj)
+    _run([cc, *DEVICE_FLAGS, "-shared", "-fPIC", "-o", LIB, *objs], verbose)
+    return LIB
+
+
+def _run(cmd, verbose):
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    noise = ("packed-fp32-ops", "1 warning generated", "warnings generated")
+    err = "\n".join(l for l in proc.stderr.splitlines() if l.strip() and not any(n in l for n in noise))
+    if proc.returncode != 0:
+        raise RuntimeError(f"{' '.join(cmd)}\nfailed with:\n{proc.stderr}")
+    if verbose and err:
+        print(err, file=sys.stderr)
+
+
+if __name__ == "__main__":
+    print(build(verbose=True))

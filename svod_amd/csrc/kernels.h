@@ -1,0 +1,47 @@
+// Launchers of the gfx950 kernels; the op layer (ops.cpp) is their only caller.
+#pragma once
+#include <hip/hip_runtime_api.h>
+#include <stdint.h>
+
+namespace svodk {
+
+// The prologue: tk/src/kernels/heads.rs:40-125 (heads_body).
+struct HeadsArgs {
+  const void *qkv;  // [rows, (heads + 2*kv_heads) * d] bf16
+  const void *q_w;  // [d] or null
+  const void *k_w;  // [d] or null
+  const void *cos;  // [t | rows, d/2] or null
+  const void *sin;
+  void *q;  // [rows, heads, d]
+  void *k;  // [rows, kv_heads, d]
+  void *v;
+  int64_t rows;  // live batches * t
+  int32_t t, heads, kv_heads, d;
+  float eps;
+  int32_t rope;  // 0 none, 1 tables by position [t, d/2], 2 by token [rows, d/2]
+};
+hipError_t launch_heads(const HeadsArgs &a, hipStream_t stream);
+// Head sizes the prologue kernel is built for.
+bool heads_supports(int32_t d);
+
+// Flash attention forward: tk/src/kernels/attention.rs:466-924 (attention_body).
+struct AttnArgs {
+  const void *q;  // [batch, t, heads, d] bf16
+  const void *k;  // [batch, tk, kv_heads, d]
+  const void *v;
+  void *o;               // [batch, t, heads, d]
+  const void *key_lens;  // [batch] i32/i64 or null
+  const void *key_mask;  // [batch, tk] u8/i32 or null
+  int32_t lens_i64;      // key_lens holds 64-bit integers
+  int32_t mask_bytes;    // element size of key_mask: 1 or 4
+  int32_t batch;         // live batches
+  int32_t t, tk, heads, kv_heads, d;
+  int32_t causal;
+  float scale;
+};
+hipError_t launch_attention(const AttnArgs &a, hipStream_t stream);
+bool attention_supports(int32_t d);
+// Text of the tile configuration launch_attention picks for `a` (for chosen()).
+const char *attention_config(const AttnArgs &a);
+
+}  // namespace svodk

@@ -1,0 +1,491 @@
+// The op layer of the gfx950 library: what Svod's `svod_tk::ops::{attention, heads}`
+// do on the host before a kernel runs — validate, plan "kernel or graph", record
+// what was chosen, launch — restated in C++ behind the C ABI of include/svodk.h.
+//
+// Contract kept from the reference (tk/src/ops/mod.rs:1-4): an op launches a
+// kernel, or names why the caller's graph must run, or rejects what the graph
+// would also reject.  Validation comes first and never touches the device, so
+// it behaves the same on a machine without a GPU.
+#include <hip/hip_runtime_api.h>
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <string>
+
+#include "../../include/svodk.h"
+#include "kernels.h"
+
+namespace {
+
+// ---- per-thread records: ops::chosen (tk/src/ops/mod.rs:83-118) and the last error.
+thread_local std::string g_chosen;
+thread_local std::string g_error;
+
+const char *fallback_name(int why) {
+  switch (why) {
+    case SVODK_GRAPH_TARGET: return "Target";
+    case SVODK_GRAPH_DTYPE: return "Dtype";
+    case SVODK_GRAPH_SYMBOLIC: return "Symbolic";
+    case SVODK_GRAPH_SHAPE: return "Shape";
+    case SVODK_GRAPH_CONFIG: return "Config";
+    default: return "?";
+  }
+}
+
+// ran_graph (mod.rs:115-118).
+int ran_graph(const char *op, int why) {
+  g_chosen = std::string("Graph { op: \"") + op + "\", why: " + fallback_name(why) + " }";
+  return why;
+}
+
+// ran (mod.rs:110-113).
+void ran(const char *op, const char *family, const char *cfg) {
+  g_chosen = std::string("Kernel { op: \"") + op + "\", family: \"" + family + "\", cfg: \"" + cfg + "\" }";
+}
+
+int fail(int status, const char *fmt, ...) {
+  char buf[512];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof buf, fmt, ap);
+  va_end(ap);
+  g_error = buf;
+  return status;
+}
+
+const char *dtype_name(int32_t d) {
+  switch (d) {
+    case SVODK_BF16: return "BFloat16";
+    case SVODK_F16: return "Float16";
+    case SVODK_F32: return "Float32";
+    case SVODK_I32: return "Int32";
+    case SVODK_I64: return "Int64";
+    case SVODK_BOOL: return "Bool";
+    default: return "?";
+  }
+}
+
+size_t dtype_bytes(int32_t d) {
+  switch (d) {
+    case SVODK_BF16:
+    case SVODK_F16: return 2;
+    case SVODK_F32:
+    case SVODK_I32: return 4;
+    case SVODK_I64: return 8;
+    case SVODK_BOOL: return 1;
+    default: return 0;
+  }
+}
+
+std::string fmt_shape(const svodk_tensor *t) {
+  std::string s = "[";
+  for (int i = 0; i < t->rank; i++) {
+    if (i) s += ", ";
+    s += std::to_string((long long)t->shape[i]);
+  }
+  return s + "]";
+}
+
+bool well_formed(const svodk_tensor *t) {
+  if (t == nullptr || t->rank < 0 || t->rank > 4 || dtype_bytes(t->dtype) == 0) return false;
+  for (int i = 0; i < t->rank; i++)
+    if (t->shape[i] < 0) return false;
+  return true;
+}
+
+int64_t numel(const svodk_tensor *t) {
+  int64_t n = 1;
+  for (int i = 0; i < t->rank; i++) n *= t->shape[i];
+  return n;
+}
+
+bool same_shape(const svodk_tensor *a, const svodk_tensor *b) {
+  if (a->rank != b->rank) return false;
+  for (int i = 0; i < a->rank; i++)
+    if (a->shape[i] != b->shape[i]) return false;
+  return true;
+}
+
+bool is_int(int32_t d) { return d == SVODK_I32 || d == SVODK_I64; }
+
+// launch::aliasing (tk/src/launch.rs:227-246): no parameter the kernel writes
+// shares memory with another.  Here a parameter is a byte range.
+struct Span {
+  const char *name;
+  const void *data;
+  size_t bytes;
+  bool written;
+};
+
+int check_aliasing(const char *op, const Span *spans, int n) {
+  for (int i = 0; i < n; i++) {
+    for (int j = i + 1; j < n; j++) {
+      const Span &a = spans[i], &b = spans[j];
+      if (!(a.written || b.written) || a.data == nullptr || b.data == nullptr || a.bytes == 0 || b.bytes == 0) continue;
+      const char *a0 = (const char *)a.data, *b0 = (const char *)b.data;
+      if (a0 < b0 + b.bytes && b0 < a0 + a.bytes)
+        return fail(SVODK_ERR_LAUNCH, "%s: parameters %s and %s share memory", op, a.name, b.name);
+    }
+  }
+  return 0;
+}
+
+// ---- the target: ops::supported / planner (mod.rs:161-197), without the cost probes.
+// The library is built for gfx950 alone; any other device has no kernels.
+bool device_is_gfx950(int device) {
+  hipDeviceProp_t prop;
+  if (hipGetDeviceProperties(&prop, device) != hipSuccess) return false;
+  return std::strncmp(prop.gcnArchName, "gfx950", 6) == 0;
+}
+
+bool current_device_has_kernels() {
+  int device = -1;
+  if (hipGetDevice(&device) != hipSuccess || device < 0) {
+    (void)hipGetLastError();
+    return false;
+  }
+  static std::mutex lock;
+  static int known[64];  // 0 unknown, 1 yes, 2 no
+  std::lock_guard<std::mutex> guard(lock);
+  if (device >= 64) return device_is_gfx950(device);
+  if (known[device] == 0) known[device] = device_is_gfx950(device) ? 1 : 2;
+  return known[device] == 1;
+}
+
+// ---- shape gates (tk/src/ops/shape.rs).
+// gate (L92-99): a target with kernels, every operand the same 16-bit type the
+// target has a matrix core for.  This library's kernels are bf16.
+int gate(bool has_target, const int32_t *dtypes, int n) {
+  if (!has_target) return SVODK_GRAPH_TARGET;
+  if (n <= 0) return SVODK_GRAPH_DTYPE;
+  const int32_t first = dtypes[0];
+  if (!(first == SVODK_BF16 || first == SVODK_F16)) return SVODK_GRAPH_DTYPE;
+  for (int i = 0; i < n; i++)
+    if (dtypes[i] != first) return SVODK_GRAPH_DTYPE;
+  // f16 has a matrix core on gfx950 but no kernel in this library: "another
+  // type without a kernel on the target" (shape.rs:30-31).
+  if (first != SVODK_BF16) return SVODK_GRAPH_DTYPE;
+  return 0;
+}
+
+// shape::attention (L189-206).  attention_ranked lists configs for head sizes
+// that tile the matrix atom; here the candidates are the head sizes the HIP
+// kernel is instantiated for.
+int plan_attention(bool has_target, const int32_t *dtypes, int n, const int64_t *q, const int64_t *k, bool causal,
+                   bool bias) {
+  (void)causal;
+  (void)bias;
+  if (int why = gate(has_target, dtypes, n)) return why;
+  if (q == nullptr || k == nullptr) return SVODK_GRAPH_SYMBOLIC;
+  for (int i = 0; i < 4; i++)
+    if (q[i] == 0 || k[i] == 0) return SVODK_GRAPH_SHAPE;
+  if (q[3] > 0x7fffffff || !svodk::attention_supports((int32_t)q[3])) return SVODK_GRAPH_SHAPE;
+  return 0;
+}
+
+// shape::heads (L209-218) with heads_candidates (tk/src/ops/config/norm.rs:8-13):
+// rank 3, no empty dim, head size a power of two in 16..=256.
+int plan_heads(bool has_target, const int32_t *dtypes, int n, const int64_t *x, int rank, int32_t d) {
+  if (int why = gate(has_target, dtypes, n)) return why;
+  if (x == nullptr) return SVODK_GRAPH_SYMBOLIC;
+  if (rank != 3) return SVODK_GRAPH_SHAPE;
+  for (int i = 0; i < 3; i++)
+    if (x[i] == 0) return SVODK_GRAPH_SHAPE;
+  const bool pow2 = d > 0 && (d & (d - 1)) == 0;
+  if (!(pow2 && d >= 16 && d <= 256) || !svodk::heads_supports(d)) return SVODK_GRAPH_SHAPE;
+  return 0;
+}
+
+const char *OP_ATTN = "attention";
+const char *OP_HEADS = "heads";
+
+}  // namespace
+
+extern "C" {
+
+int svodk_abi_version(void) { return SVODK_ABI_VERSION; }
+
+const char *svodk_last_chosen(void) { return g_chosen.c_str(); }
+
+const char *svodk_last_error(void) { return g_error.c_str(); }
+
+const char *svodk_status_name(int status) {
+  switch (status) {
+    case SVODK_KERNEL: return "Kernel";
+    case SVODK_GRAPH_TARGET: return "Fallback::Target";
+    case SVODK_GRAPH_DTYPE: return "Fallback::Dtype";
+    case SVODK_GRAPH_SYMBOLIC: return "Fallback::Symbolic";
+    case SVODK_GRAPH_SHAPE: return "Fallback::Shape";
+    case SVODK_GRAPH_CONFIG: return "Fallback::Config";
+    case SVODK_ERR_SHAPE: return "Error::Shape";
+    case SVODK_ERR_DTYPE: return "Error::Dtype";
+    case SVODK_ERR_HEADS: return "Error::Heads";
+    case SVODK_ERR_LAUNCH: return "Error::Launch";
+    case SVODK_ERR_ARGUMENT: return "Error::Argument";
+    default: return "?";
+  }
+}
+
+int svodk_supported(void) { return current_device_has_kernels() ? 1 : 0; }
+
+int svodk_plan_attention(int32_t has_target, const int32_t *dtypes, int32_t n_dtypes, const int64_t *q_dims,
+                         const int64_t *k_dims, int32_t causal, int32_t bias) {
+  return plan_attention(has_target != 0, dtypes, n_dtypes, q_dims, k_dims, causal != 0, bias != 0);
+}
+
+int svodk_plan_heads(int32_t has_target, const int32_t *dtypes, int32_t n_dtypes, const int64_t *x_dims, int32_t x_rank,
+                     int32_t head_dim) {
+  return plan_heads(has_target != 0, dtypes, n_dtypes, x_dims, x_rank, head_dim);
+}
+
+// attend (tk/src/ops/attention.rs:126-303).
+int svodk_attention(const svodk_tensor *q, const svodk_tensor *k, const svodk_tensor *v, const svodk_attn *opts,
+                    const svodk_tensor *out, void *hip_stream) {
+  const char *op = OP_ATTN;
+  if (!well_formed(q) || !well_formed(k) || !well_formed(v) || !well_formed(out) || opts == nullptr)
+    return fail(SVODK_ERR_ARGUMENT, "%s: a null or malformed tensor descriptor", op);
+  // L131: q is [B, T, H, D].
+  if (q->rank != 4)
+    return fail(SVODK_ERR_SHAPE, "%s: q has shape %s, expected [B, T, H, D]", op, fmt_shape(q).c_str());
+  // L136-138: k is [B, Tk, H_kv, D]; v has k's shape.  (A cache with a row map
+  // relaxes the batch; a cache never takes a kernel here, but the check stands.)
+  const bool batch_fits = k->rank == 4 && (k->shape[0] == q->shape[0] || opts->has_cache);
+  if (!(k->rank == 4 && batch_fits && k->shape[3] == q->shape[3]))
+    return fail(SVODK_ERR_SHAPE, "%s: k has shape %s, expected [%lld, Tk, H_kv, %lld]", op, fmt_shape(k).c_str(),
+                (long long)q->shape[0], (long long)q->shape[3]);
+  if (!same_shape(v, k))
+    return fail(SVODK_ERR_SHAPE, "%s: v has shape %s, expected %s", op, fmt_shape(v).c_str(), fmt_shape(k).c_str());
+  // L139-141: k and v share q's type.
+  if (k->dtype != q->dtype)
+    return fail(SVODK_ERR_DTYPE, "%s: k is %s, the input is %s", op, dtype_name(k->dtype), dtype_name(q->dtype));
+  if (v->dtype != q->dtype)
+    return fail(SVODK_ERR_DTYPE, "%s: v is %s, the input is %s", op, dtype_name(v->dtype), dtype_name(q->dtype));
+  // L142-145: whole groups of query heads per KV head.
+  const int64_t heads = q->shape[2], kv_heads = k->shape[2];
+  if (!opts->has_cache && !(kv_heads > 0 && heads % kv_heads == 0))
+    return fail(SVODK_ERR_HEADS, "%s: %lld query heads are not a multiple of %lld key/value heads", op,
+                (long long)heads, (long long)kv_heads);
+  // L174-186: the key mask's shape.
+  const svodk_tensor *lens = nullptr, *bools = nullptr;
+  if (opts->key_kind == SVODK_KEYS_LENS) {
+    if (!well_formed(opts->keys)) return fail(SVODK_ERR_ARGUMENT, "%s: key lens descriptor missing", op);
+    if (!(opts->keys->rank == 1 && opts->keys->shape[0] == q->shape[0]))
+      return fail(SVODK_ERR_SHAPE, "%s: key lens has shape %s, expected [%lld]", op, fmt_shape(opts->keys).c_str(),
+                  (long long)q->shape[0]);
+    lens = opts->keys;
+  } else if (opts->key_kind == SVODK_KEYS_BOOL) {
+    if (!well_formed(opts->keys)) return fail(SVODK_ERR_ARGUMENT, "%s: key mask descriptor missing", op);
+    if (!(opts->keys->rank == 2 && opts->keys->shape[0] == q->shape[0] && opts->keys->shape[1] == k->shape[1]))
+      return fail(SVODK_ERR_SHAPE, "%s: key mask has shape %s, expected [%lld, %lld]", op,
+                  fmt_shape(opts->keys).c_str(), (long long)q->shape[0], (long long)k->shape[1]);
+    bools = opts->keys;
+  } else if (opts->key_kind != SVODK_KEYS_NONE) {
+    return fail(SVODK_ERR_ARGUMENT, "%s: unknown key mask kind %d", op, opts->key_kind);
+  }
+  // L187-190: segment starts are [B, T].
+  if (opts->seg_start != nullptr) {
+    if (!well_formed(opts->seg_start)) return fail(SVODK_ERR_ARGUMENT, "%s: seg start descriptor malformed", op);
+    if (!(opts->seg_start->rank == 2 && opts->seg_start->shape[0] == q->shape[0] &&
+          opts->seg_start->shape[1] == q->shape[1]))
+      return fail(SVODK_ERR_SHAPE, "%s: seg start has shape %s, expected [%lld, %lld]", op,
+                  fmt_shape(opts->seg_start).c_str(), (long long)q->shape[0], (long long)q->shape[1]);
+  }
+  // L193-203: a bias is [B | 1, H, T, Tk].
+  if (opts->bias != nullptr) {
+    if (!well_formed(opts->bias)) return fail(SVODK_ERR_ARGUMENT, "%s: bias descriptor malformed", op);
+    const svodk_tensor *bt = opts->bias;
+    const bool fits = bt->rank == 4 && (bt->shape[0] == q->shape[0] || bt->shape[0] == 1) && bt->shape[1] == heads &&
+                      bt->shape[2] == q->shape[1] && bt->shape[3] == k->shape[1];
+    if (!fits)
+      return fail(SVODK_ERR_SHAPE, "%s: bias has shape %s, expected [%lld | 1, %lld, %lld, %lld]", op,
+                  fmt_shape(bt).c_str(), (long long)q->shape[0], (long long)heads, (long long)q->shape[1],
+                  (long long)k->shape[1]);
+  }
+  // The output the reference op allocates itself (tk/src/ops/mod.rs:423-429):
+  // here the caller's, so its shape and type are checked like an operand's.
+  if (!same_shape(out, q))
+    return fail(SVODK_ERR_SHAPE, "%s: out has shape %s, expected %s", op, fmt_shape(out).c_str(),
+                fmt_shape(q).c_str());
+  if (out->dtype != q->dtype)
+    return fail(SVODK_ERR_DTYPE, "%s: out is %s, the input is %s", op, dtype_name(out->dtype), dtype_name(q->dtype));
+  if (lens != nullptr && !is_int(lens->dtype))
+    return fail(SVODK_ERR_DTYPE, "%s: key lens is %s, the input is an integer type", op, dtype_name(lens->dtype));
+  if (bools != nullptr && !(bools->dtype == SVODK_BOOL || bools->dtype == SVODK_I32))
+    return fail(SVODK_ERR_DTYPE, "%s: key mask is %s, the input is Bool or Int32", op, dtype_name(bools->dtype));
+  const int64_t cap = q->shape[0];
+  if (opts->batch_live > cap)
+    return fail(SVODK_ERR_SHAPE, "%s: live batch %d exceeds the capacity %lld", op, opts->batch_live, (long long)cap);
+
+  // L205-208: the plan.  A chunk mask plans as a causal one.
+  int32_t dtypes[4] = {q->dtype, k->dtype, v->dtype, opts->bias ? opts->bias->dtype : 0};
+  const int why = plan_attention(current_device_has_kernels(), dtypes, opts->bias ? 4 : 3, q->shape, k->shape,
+                                 opts->causal || opts->has_chunk, opts->bias != nullptr);
+  if (why != 0) return ran_graph(op, why);
+  // Options the reference's kernel holds and this library's does not: no
+  // config here holds them (the reference's own use of Fallback::Config, L210-214).
+  if (opts->has_window || opts->has_chunk || opts->seg_start != nullptr || opts->has_cache || opts->bias != nullptr ||
+      opts->splits > 1)
+    return ran_graph(op, SVODK_GRAPH_CONFIG);
+  const int64_t t = q->shape[1], tk = k->shape[1], d = q->shape[3];
+  if (t > 0x7fffffff || tk > 0x7fffffff || heads > 0x7fffffff || cap > 0x7fffffff)
+    return ran_graph(op, SVODK_GRAPH_SHAPE);
+
+  Span spans[6] = {{"q", q->data, (size_t)numel(q) * 2, false},
+                   {"k", k->data, (size_t)numel(k) * 2, false},
+                   {"v", v->data, (size_t)numel(v) * 2, false},
+                   {"o", out->data, (size_t)numel(out) * 2, true},
+                   {"key_lens", lens ? lens->data : nullptr, lens ? (size_t)numel(lens) * dtype_bytes(lens->dtype) : 0,
+                    false},
+                   {"key_mask", bools ? bools->data : nullptr,
+                    bools ? (size_t)numel(bools) * dtype_bytes(bools->dtype) : 0, false}};
+  if (q->data == nullptr || k->data == nullptr || v->data == nullptr || out->data == nullptr ||
+      (lens && lens->data == nullptr) || (bools && bools->data == nullptr))
+    return fail(SVODK_ERR_ARGUMENT, "%s: a null device pointer", op);
+  if (int rc = check_aliasing(op, spans, 6)) return rc;
+
+  svodk::AttnArgs a{};
+  a.q = q->data;
+  a.k = k->data;
+  a.v = v->data;
+  a.o = out->data;
+  a.key_lens = lens ? lens->data : nullptr;
+  a.key_mask = bools ? bools->data : nullptr;
+  a.lens_i64 = lens && lens->dtype == SVODK_I64;
+  a.mask_bytes = bools ? (int32_t)dtype_bytes(bools->dtype) : 0;
+  a.batch = opts->batch_live > 0 ? opts->batch_live : (int32_t)cap;
+  a.t = (int32_t)t;
+  a.tk = (int32_t)tk;
+  a.heads = (int32_t)heads;
+  a.kv_heads = (int32_t)kv_heads;
+  a.d = (int32_t)d;
+  a.causal = opts->causal != 0;
+  // L230: the default scale is 1/sqrt(D) in f32.
+  a.scale = opts->has_scale ? opts->scale : 1.0f / std::sqrt((float)d);
+  ran(op, "flash_attention", svodk::attention_config(a));
+  const hipError_t e = svodk::launch_attention(a, (hipStream_t)hip_stream);
+  if (e != hipSuccess) return fail(SVODK_ERR_LAUNCH, "%s: %s", op, hipGetErrorString(e));
+  return SVODK_KERNEL;
+}
+
+// heads (tk/src/ops/heads.rs:37-102).
+int svodk_heads(const svodk_tensor *qkv, const svodk_qkv *opts, const svodk_tensor *q, const svodk_tensor *k,
+                const svodk_tensor *v, void *hip_stream) {
+  const char *op = OP_HEADS;
+  if (!well_formed(qkv) || !well_formed(q) || !well_formed(k) || !well_formed(v) || opts == nullptr)
+    return fail(SVODK_ERR_ARGUMENT, "%s: a null or malformed tensor descriptor", op);
+  const int64_t heads = opts->heads, kv_heads = opts->kv_heads, d = opts->head_dim;
+  // L44: whole groups of query heads per KV head.
+  if (!(kv_heads > 0 && heads >= 0 && heads % kv_heads == 0))
+    return fail(SVODK_ERR_HEADS, "%s: %lld query heads are not a multiple of %lld key/value heads", op,
+                (long long)heads, (long long)kv_heads);
+  if (d <= 0) return fail(SVODK_ERR_ARGUMENT, "%s: head_dim %lld", op, (long long)d);
+  const int64_t slots = heads + 2 * kv_heads;
+  // L45-47: qkv is [B, T, slots*d].
+  if (!(qkv->rank == 3 && qkv->shape[2] == slots * d))
+    return fail(SVODK_ERR_SHAPE, "%s: qkv has shape %s, expected [B, T, %lld\xc2\xb7%lld]", op, fmt_shape(qkv).c_str(),
+                (long long)slots, (long long)d);
+  // L48-53: the norm weights are [d].
+  const svodk_tensor *norms[2] = {opts->q_norm, opts->k_norm};
+  const char *norm_names[2] = {"q norm", "k norm"};
+  for (int i = 0; i < 2; i++) {
+    if (norms[i] == nullptr) continue;
+    if (!well_formed(norms[i])) return fail(SVODK_ERR_ARGUMENT, "%s: %s descriptor malformed", op, norm_names[i]);
+    if (!(norms[i]->rank == 1 && norms[i]->shape[0] == d))
+      return fail(SVODK_ERR_SHAPE, "%s: %s has shape %s, expected [%lld]", op, norm_names[i],
+                  fmt_shape(norms[i]).c_str(), (long long)d);
+  }
+  // L54-63: tables are [1, T, 1, d/2] by position or [B, T, 1, d/2] by token.
+  if ((opts->cos == nullptr) != (opts->sin == nullptr))
+    return fail(SVODK_ERR_ARGUMENT, "%s: cos and sin come together", op);
+  bool per_batch = false;
+  if (opts->cos != nullptr) {
+    const svodk_tensor *c = opts->cos, *s = opts->sin;
+    if (!well_formed(c) || !well_formed(s)) return fail(SVODK_ERR_ARGUMENT, "%s: rope descriptor malformed", op);
+    const bool tail = c->rank == 4 && c->shape[1] == qkv->shape[1] && c->shape[2] == 1 && c->shape[3] == d / 2;
+    const bool fits = tail && (c->shape[0] == 1 || c->shape[0] == qkv->shape[0]);
+    if (!fits)
+      return fail(SVODK_ERR_SHAPE, "%s: cos has shape %s, expected [1, %lld, 1, %lld] or [%lld, %lld, 1, %lld]", op,
+                  fmt_shape(c).c_str(), (long long)qkv->shape[1], (long long)(d / 2), (long long)qkv->shape[0],
+                  (long long)qkv->shape[1], (long long)(d / 2));
+    if (!same_shape(s, c))
+      return fail(SVODK_ERR_SHAPE, "%s: sin has shape %s, expected %s", op, fmt_shape(s).c_str(),
+                  fmt_shape(c).c_str());
+    // L80: by token when the leading dim is not the constant 1.
+    per_batch = c->shape[0] != 1;
+  }
+  // The outputs the reference op allocates itself (L89-91), here the caller's.
+  const int64_t want_q[4] = {qkv->shape[0], qkv->shape[1], heads, d};
+  const int64_t want_kv[4] = {qkv->shape[0], qkv->shape[1], kv_heads, d};
+  const svodk_tensor *outs[3] = {q, k, v};
+  const char *out_names[3] = {"q", "k", "v"};
+  for (int i = 0; i < 3; i++) {
+    const int64_t *want = i == 0 ? want_q : want_kv;
+    bool fits = outs[i]->rank == 4;
+    for (int j = 0; fits && j < 4; j++) fits = outs[i]->shape[j] == want[j];
+    if (!fits)
+      return fail(SVODK_ERR_SHAPE, "%s: %s has shape %s, expected [%lld, %lld, %lld, %lld]", op, out_names[i],
+                  fmt_shape(outs[i]).c_str(), (long long)want[0], (long long)want[1], (long long)want[2],
+                  (long long)want[3]);
+    if (outs[i]->dtype != qkv->dtype)
+      return fail(SVODK_ERR_DTYPE, "%s: %s is %s, the input is %s", op, out_names[i], dtype_name(outs[i]->dtype),
+                  dtype_name(qkv->dtype));
+  }
+  const int64_t cap = qkv->shape[0];
+  if (opts->batch_live > cap)
+    return fail(SVODK_ERR_SHAPE, "%s: live batch %d exceeds the capacity %lld", op, opts->batch_live, (long long)cap);
+
+  // L65-72: a weight or table off the stream dtype keeps the graph.
+  int32_t dtypes[5];
+  int n = 0;
+  dtypes[n++] = qkv->dtype;
+  if (opts->q_norm) dtypes[n++] = opts->q_norm->dtype;
+  if (opts->k_norm) dtypes[n++] = opts->k_norm->dtype;
+  if (opts->cos) dtypes[n++] = opts->cos->dtype;
+  if (opts->sin) dtypes[n++] = opts->sin->dtype;
+  const int why = plan_heads(current_device_has_kernels(), dtypes, n, qkv->shape, qkv->rank, (int32_t)d);
+  if (why != 0) return ran_graph(op, why);
+  const int64_t t = qkv->shape[1];
+  if (t > 0x7fffffff || heads > 0x7fff || kv_heads > 0x7fff) return ran_graph(op, SVODK_GRAPH_SHAPE);
+
+  const size_t table_bytes = opts->cos ? (size_t)numel(opts->cos) * 2 : 0;
+  Span spans[8] = {{"qkv", qkv->data, (size_t)numel(qkv) * 2, false},
+                   {"q_w", opts->q_norm ? opts->q_norm->data : nullptr, (size_t)d * 2, false},
+                   {"k_w", opts->k_norm ? opts->k_norm->data : nullptr, (size_t)d * 2, false},
+                   {"cos", opts->cos ? opts->cos->data : nullptr, table_bytes, false},
+                   {"sin", opts->sin ? opts->sin->data : nullptr, table_bytes, false},
+                   {"q", q->data, (size_t)numel(q) * 2, true},
+                   {"k", k->data, (size_t)numel(k) * 2, true},
+                   {"v", v->data, (size_t)numel(v) * 2, true}};
+  if (qkv->data == nullptr || q->data == nullptr || k->data == nullptr || v->data == nullptr ||
+      (opts->q_norm && opts->q_norm->data == nullptr) || (opts->k_norm && opts->k_norm->data == nullptr) ||
+      (opts->cos && (opts->cos->data == nullptr || opts->sin->data == nullptr)))
+    return fail(SVODK_ERR_ARGUMENT, "%s: a null device pointer", op);
+  if (int rc = check_aliasing(op, spans, 8)) return rc;
+
+  svodk::HeadsArgs a{};
+  a.qkv = qkv->data;
+  a.q_w = opts->q_norm ? opts->q_norm->data : nullptr;
+  a.k_w = opts->k_norm ? opts->k_norm->data : nullptr;
+  a.cos = opts->cos ? opts->cos->data : nullptr;
+  a.sin = opts->sin ? opts->sin->data : nullptr;
+  a.q = q->data;
+  a.k = k->data;
+  a.v = v->data;
+  const int64_t live = opts->batch_live > 0 ? opts->batch_live : cap;
+  a.rows = live * t;
+  a.t = (int32_t)t;
+  a.heads = (int32_t)heads;
+  a.kv_heads = (int32_t)kv_heads;
+  a.d = (int32_t)d;
+  a.eps = (float)opts->eps;
+  a.rope = opts->cos ? (per_batch ? 2 : 1) : 0;
+  ran(op, "heads", "NormCfg { lanes_per_head: d/16, block: 256 }");
+  const hipError_t e = svodk::launch_heads(a, (hipStream_t)hip_stream);
+  if (e != hipSuccess) return fail(SVODK_ERR_LAUNCH, "%s: %s", op, hipGetErrorString(e));
+  return SVODK_KERNEL;
+}
+
+}  // extern "C"

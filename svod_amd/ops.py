@@ -1,0 +1,303 @@
+"""Host mirror of ``svod_tk::ops::{attention, heads}`` over the C ABI.
+
+Reference: ``tk/src/ops/attention.rs:100`` (``attention``), ``tk/src/ops/heads.rs:37``
+(``heads``), ``tk/src/ops/mod.rs:83-118`` (``chosen``), ``:164`` (``supported``).
+
+The reference op "always returns a Tensor": where no kernel applies it builds
+the equivalent graph itself.  That graph is Svod's, not this library's, so here
+the same outcome is reported instead of computed: :class:`GraphFallback` carries
+the reference's ``Fallback`` reason and the caller runs its own graph.  Nothing
+in this module computes attention on the host.
+"""
+from __future__ import annotations
+
+import ctypes
+import enum
+import os
+from dataclasses import dataclass
+from typing import Optional, Tuple
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_NAME = "libsvodk_gfx950.so"
+
+
+def library_path() -> str:
+    return os.path.join(_HERE, _LIB_NAME)
+
+
+class _Tensor(ctypes.Structure):
+    _fields_ = [("data", ctypes.c_void_p), ("dtype", ctypes.c_int32), ("rank", ctypes.c_int32),
+                ("shape", ctypes.c_int64 * 4)]
+
+
+class _Attn(ctypes.Structure):
+    _fields_ = [
+        ("causal", ctypes.c_int32), ("key_kind", ctypes.c_int32), ("keys", ctypes.POINTER(_Tensor)),
+        ("has_window", ctypes.c_int32), ("window_left", ctypes.c_int64), ("window_right", ctypes.c_int64),
+        ("has_chunk", ctypes.c_int32), ("chunk_size", ctypes.c_int64), ("chunk_has_left", ctypes.c_int32),
+        ("chunk_left", ctypes.c_int64), ("chunk_right", ctypes.c_int64),
+        ("seg_start", ctypes.POINTER(_Tensor)), ("has_cache", ctypes.c_int32), ("bias", ctypes.POINTER(_Tensor)),
+        ("splits", ctypes.c_int32), ("has_scale", ctypes.c_int32), ("scale", ctypes.c_float),
+        ("batch_live", ctypes.c_int32),
+    ]
+
+
+class _Qkv(ctypes.Structure):
+    _fields_ = [
+        ("heads", ctypes.c_int32), ("kv_heads", ctypes.c_int32), ("head_dim", ctypes.c_int32),
+        ("q_norm", ctypes.POINTER(_Tensor)), ("k_norm", ctypes.POINTER(_Tensor)), ("eps", ctypes.c_double),
+        ("cos", ctypes.POINTER(_Tensor)), ("sin", ctypes.POINTER(_Tensor)), ("batch_live", ctypes.c_int32),
+    ]
+
+
+_lib: Optional[ctypes.CDLL] = None
+
+
+def load_library() -> ctypes.CDLL:
+    """The shared library, loaded once.  Missing library = hard error: there is
+    no other implementation behind these ops."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    path = library_path()
+    if not os.path.exists(path):
+        raise ImportError(
+            f"{path} is missing: build it with `python -m svod_amd.build` (hipcc, gfx950). "
+            "svod_amd has no fallback implementation.")
+    lib = ctypes.CDLL(path)
+    tp = ctypes.POINTER(_Tensor)
+    lib.svodk_attention.restype = ctypes.c_int
+    lib.svodk_attention.argtypes = [tp, tp, tp, ctypes.POINTER(_Attn), tp, ctypes.c_void_p]
+    lib.svodk_heads.restype = ctypes.c_int
+    lib.svodk_heads.argtypes = [tp, ctypes.POINTER(_Qkv), tp, tp, tp, ctypes.c_void_p]
+    i32p, i64p = ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int64)
+    lib.svodk_plan_attention.restype = ctypes.c_int
+    lib.svodk_plan_attention.argtypes = [ctypes.c_int32, i32p, ctypes.c_int32, i64p, i64p, ctypes.c_int32, ctypes.c_int32]
+    lib.svodk_plan_heads.restype = ctypes.c_int
+    lib.svodk_plan_heads.argtypes = [ctypes.c_int32, i32p, ctypes.c_int32, i64p, ctypes.c_int32, ctypes.c_int32]
+    lib.svodk_supported.restype = ctypes.c_int
+    lib.svodk_last_chosen.restype = ctypes.c_char_p
+    lib.svodk_last_error.restype = ctypes.c_char_p
+    lib.svodk_status_name.restype = ctypes.c_char_p
+    lib.svodk_status_name.argtypes = [ctypes.c_int]
+    lib.svodk_abi_version.restype = ctypes.c_int
+    _lib = lib
+    return lib
+
+
+class Fallback(enum.IntEnum):
+    """``Fallback`` of tk/src/ops/shape.rs:26-39."""
+
+    Target = 1
+    Dtype = 2
+    Symbolic = 3
+    Shape = 4
+    Config = 5
+
+
+class GraphFallback(Exception):
+    """The op's ``Plan::Graph(why)`` outcome: no kernel applies, the caller's graph runs."""
+
+    def __init__(self, op: str, why: Fallback):
+        super().__init__(f"{op}: no kernel applies ({why.name}); run the graph op")
+        self.op, self.why = op, why
+
+
+class OpError(Exception):
+    """``ops::Error`` of tk/src/ops/mod.rs:132-157; ``kind`` is the variant's name."""
+
+    def __init__(self, kind: str, message: str):
+        super().__init__(message)
+        self.kind = kind
+
+
+_ERR_KIND = {-1: "Shape", -2: "Dtype", -3: "Heads", -4: "Launch", -5: "Argument"}
+
+_DTYPES = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2, torch.int32: 3, torch.int64: 4, torch.bool: 5}
+
+
+def _desc(t: torch.Tensor) -> _Tensor:
+    if t.dtype not in _DTYPES:
+        raise OpError("Dtype", f"unsupported element type {t.dtype}")
+    if t.dim() > 4:
+        raise OpError("Shape", f"rank {t.dim()} tensor")
+    if not t.is_contiguous():
+        raise OpError("Argument", "operands must be dense row-major (call .contiguous())")
+    d = _Tensor()
+    d.data = t.data_ptr()
+    d.dtype = _DTYPES[t.dtype]
+    d.rank = t.dim()
+    for i, s in enumerate(t.shape):
+        d.shape[i] = s
+    return d
+
+
+def _ref(keep: list, t: Optional[torch.Tensor]):
+    if t is None:
+        return ctypes.POINTER(_Tensor)()
+    d = _desc(t)
+    keep.append(d)
+    return ctypes.pointer(d)
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream if t.is_cuda else 0
+
+
+def _finish(op: str, status: int):
+    if status == 0:
+        return
+    if status > 0:
+        raise GraphFallback(op, Fallback(status))
+    raise OpError(_ERR_KIND.get(status, "?"), load_library().svodk_last_error().decode())
+
+
+@dataclass(frozen=True)
+class KeyMask:
+    """``KeyMask`` of tk/src/ops/attention.rs:29-37."""
+
+    kind: int = 0
+    tensor: Optional[torch.Tensor] = None
+
+    @staticmethod
+    def none() -> "KeyMask":
+        return KeyMask(0, None)
+
+    @staticmethod
+    def lens(lens: torch.Tensor) -> "KeyMask":
+        """``[B]`` integer valid-key counts: keys at and past ``lens[b]`` are masked."""
+        return KeyMask(1, lens)
+
+    @staticmethod
+    def bool(mask: torch.Tensor) -> "KeyMask":
+        """``[B, Tk]`` bool (or int32) mask, true (nonzero) where the key is attended."""
+        return KeyMask(2, mask)
+
+
+@dataclass
+class Attn:
+    """``Attn`` of tk/src/ops/attention.rs:60-86.  ``batch_live`` stands for a bound
+    batch variable (``Batch::Var``): only the first ``batch_live`` batches run."""
+
+    causal: bool = False
+    keys: KeyMask = KeyMask()
+    window: Optional[Tuple[int, int]] = None
+    chunk: Optional[Tuple[int, Optional[int], int]] = None  # (size, left, right)
+    seg_start: Optional[torch.Tensor] = None
+    cache: bool = False
+    splits: Optional[int] = None
+    scale: Optional[float] = None
+    bias: Optional[torch.Tensor] = None
+    batch_live: Optional[int] = None
+
+
+@dataclass
+class Qkv:
+    """``Qkv`` of tk/src/ops/heads.rs:19-31."""
+
+    heads: int
+    kv_heads: int
+    head_dim: int
+    q_norm: Optional[torch.Tensor] = None
+    k_norm: Optional[torch.Tensor] = None
+    eps: float = 1e-6
+    rope: Optional[Tuple[torch.Tensor, torch.Tensor]] = None
+    batch_live: Optional[int] = None
+
+
+def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, opts: Optional[Attn] = None,
+              out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``softmax(q·kᵀ·scale)·v`` over ``q [B,T,H,D]`` and ``k``/``v [B,Tk,H_kv,D]``;
+    returns ``[B,T,H,D]`` (tk/src/ops/attention.rs:98-103).  Enqueued on the
+    current stream of ``q``'s device; returns without synchronising."""
+    opts = opts or Attn()
+    lib = load_library()
+    if out is None:
+        # The op allocates its output at capacity (tk/src/ops/mod.rs:423-429).
+        out = torch.empty_like(q)
+    keep: list = []
+    a = _Attn()
+    a.causal = int(opts.causal)
+    a.key_kind = opts.keys.kind
+    a.keys = _ref(keep, opts.keys.tensor)
+    if opts.window is not None:
+        a.has_window, a.window_left, a.window_right = 1, opts.window[0], opts.window[1]
+    if opts.chunk is not None:
+        size, left, right = opts.chunk
+        a.has_chunk, a.chunk_size, a.chunk_right = 1, size, right
+        a.chunk_has_left, a.chunk_left = (0, 0) if left is None else (1, left)
+    a.seg_start = _ref(keep, opts.seg_start)
+    a.has_cache = int(bool(opts.cache))
+    a.bias = _ref(keep, opts.bias)
+    a.splits = opts.splits or 0
+    if opts.scale is not None:
+        a.has_scale, a.scale = 1, float(opts.scale)
+    a.batch_live = opts.batch_live or 0
+    qd, kd, vd, od = _desc(q), _desc(k), _desc(v), _desc(out)
+    status = lib.svodk_attention(ctypes.byref(qd), ctypes.byref(kd), ctypes.byref(vd), ctypes.byref(a),
+                                 ctypes.byref(od), ctypes.c_void_p(_stream(q)))
+    _finish("attention", status)
+    return out
+
+
+def heads(qkv: torch.Tensor, opts: Qkv, out: Optional[Tuple[torch.Tensor, torch.Tensor, torch.Tensor]] = None):
+    """``qkv [B,T,(heads+2·kv_heads)·head_dim]`` → ``(q [B,T,heads,D], k, v [B,T,kv_heads,D])``
+    (tk/src/ops/heads.rs:35-37)."""
+    lib = load_library()
+    if qkv.dim() == 3 and out is None:
+        b, t = qkv.shape[0], qkv.shape[1]
+        mk = lambda n: torch.empty((b, t, n, opts.head_dim), dtype=qkv.dtype, device=qkv.device)
+        out = (mk(opts.heads), mk(opts.kv_heads), mk(opts.kv_heads))
+    elif out is None:
+        # Let the library word the shape error; the outputs are never touched.
+        e = torch.empty((0, 0, 0, 0), dtype=qkv.dtype, device=qkv.device)
+        out = (e, e, e)
+    keep: list = []
+    o = _Qkv()
+    o.heads, o.kv_heads, o.head_dim = opts.heads, opts.kv_heads, opts.head_dim
+    o.q_norm, o.k_norm = _ref(keep, opts.q_norm), _ref(keep, opts.k_norm)
+    o.eps = float(opts.eps)
+    cos, sin = opts.rope if opts.rope is not None else (None, None)
+    o.cos, o.sin = _ref(keep, cos), _ref(keep, sin)
+    o.batch_live = opts.batch_live or 0
+    xd, qd, kd, vd = _desc(qkv), _desc(out[0]), _desc(out[1]), _desc(out[2])
+    status = lib.svodk_heads(ctypes.byref(xd), ctypes.byref(o), ctypes.byref(qd), ctypes.byref(kd), ctypes.byref(vd),
+                             ctypes.c_void_p(_stream(qkv)))
+    _finish("heads", status)
+    return out
+
+
+def chosen() -> str:
+    """What the last op on this thread ran (tk/src/ops/mod.rs:83-108)."""
+    return load_library().svodk_last_chosen().decode()
+
+
+def supported() -> bool:
+    """Whether the current device has kernels (tk/src/ops/mod.rs:164-166)."""
+    return bool(load_library().svodk_supported())
+
+
+def _plan(status: int) -> Optional[Fallback]:
+    return None if status == 0 else Fallback(status)
+
+
+def plan_attention(has_target: bool, dtypes, q_dims, k_dims, causal=False, bias=False) -> Optional[Fallback]:
+    """``shape::attention`` (tk/src/ops/shape.rs:189-206) as a pure function: ``None``
+    for ``Plan::Kernel``, else the ``Fallback``.  ``q_dims``/``k_dims`` ``None`` =
+    a symbolic dim past the batch."""
+    lib = load_library()
+    dt = (ctypes.c_int32 * len(dtypes))(*[_DTYPES[d] for d in dtypes])
+    qd = (ctypes.c_int64 * 4)(*q_dims) if q_dims is not None else None
+    kd = (ctypes.c_int64 * 4)(*k_dims) if k_dims is not None else None
+    return _plan(lib.svodk_plan_attention(int(has_target), dt, len(dtypes), qd, kd, int(causal), int(bias)))
+
+
+def plan_heads(has_target: bool, dtypes, x_dims, head_dim: int) -> Optional[Fallback]:
+    """``shape::heads`` (tk/src/ops/shape.rs:209-218) as a pure function."""
+    lib = load_library()
+    dt = (ctypes.c_int32 * len(dtypes))(*[_DTYPES[d] for d in dtypes])
+    xd = (ctypes.c_int64 * len(x_dims))(*x_dims) if x_dims is not None else None
+    return _plan(lib.svodk_plan_heads(int(has_target), dt, len(dtypes), xd, len(x_dims) if x_dims is not None else 0,
+                                      head_dim))

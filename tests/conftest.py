@@ -1,0 +1,26 @@
+import os
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with `-m gpu` on the GPU box)")
+
+
+@pytest.fixture(scope="session")
+def device():
+    """cuda:0 on a box whose device has kernels; the GPU tests fail, not skip, when the
+    library is missing or does not recognise the device."""
+    import torch
+
+    import svod_amd
+
+    assert torch.cuda.is_available(), "the gpu-marked tests need a GPU"
+    svod_amd.load_library()
+    assert svod_amd.supported(), "the current device is not a gfx950 this library has kernels for"
+    return torch.device("cuda:0")

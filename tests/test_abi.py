@@ -1,0 +1,165 @@
+"""The C ABI without a GPU: the library loads, exports what include/svodk.h declares, validates
+arguments as the reference op layer does and plans "kernel or graph" as its shape gates do.
+No compute call is made here."""
+import os
+import re
+
+import pytest
+import torch
+
+import svod_amd
+from svod_amd import Attn, Fallback, GraphFallback, KeyMask, OpError, Qkv
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+BF16, F16, F32, I32 = torch.bfloat16, torch.float16, torch.float32, torch.int32
+
+
+def t(shape, dtype=BF16):
+    return torch.zeros(shape, dtype=dtype)
+
+
+def test_every_declared_symbol_is_exported():
+    header = open(os.path.join(ROOT, "include", "svodk.h")).read()
+    names = set(re.findall(r"\b(svodk_[a-z_]+)\s*\(", header))
+    assert {"svodk_attention", "svodk_heads", "svodk_supported", "svodk_last_chosen"} <= names
+    lib = svod_amd.load_library()
+    for n in sorted(names):
+        assert hasattr(lib, n), n
+    assert lib.svodk_abi_version() == 1
+
+
+def test_status_names():
+    lib = svod_amd.load_library()
+    assert lib.svodk_status_name(0) == b"Kernel"
+    assert lib.svodk_status_name(4) == b"Fallback::Shape"
+    assert lib.svodk_status_name(-3) == b"Error::Heads"
+
+
+# ---- shape gates: tk/src/test/unit/ops_plan.rs:1153-1175 (every_op_falls_back_alike)
+@pytest.mark.parametrize("has_target,dtypes,static_dims,why", [
+    (False, [BF16, BF16], True, Fallback.Target),
+    (True, [F32, F32], True, Fallback.Dtype),
+    (True, [BF16, F32], True, Fallback.Dtype),
+    (True, [I32, I32], True, Fallback.Dtype),
+    (True, [BF16, BF16], False, Fallback.Symbolic),
+], ids=["no target", "f32 keeps the graph", "mixed operand types", "integers", "symbolic past the batch"])
+def test_every_op_falls_back_alike(has_target, dtypes, static_dims, why):
+    q = [2, 128, 16, 64] if static_dims else None
+    x = [2, 128, 1024] if static_dims else None
+    assert svod_amd.plan_attention(has_target, dtypes, q, q) == why
+    assert svod_amd.plan_heads(has_target, dtypes, x, 64) == why
+
+
+# ---- ops_plan.rs:1241-1262 (attention_plans).  The reference plans d in {32, 48, 64, 128, 256}
+# and sends d = 40 to the graph; this library's kernel is built for d in {64, 128} and sends
+# the other head sizes to the graph with the same reason, Fallback::Shape.
+@pytest.mark.parametrize("d,want", [(64, None), (128, None), (40, Fallback.Shape), (48, Fallback.Shape),
+                                    (32, Fallback.Shape), (256, Fallback.Shape)])
+def test_attention_plans(d, want):
+    assert svod_amd.plan_attention(True, [BF16] * 3, [2, 100, 8, d], [2, 37, 2, d]) == want
+
+
+def test_an_empty_dim_keeps_the_graph():
+    assert svod_amd.plan_attention(True, [BF16] * 3, [0, 100, 8, 64], [0, 37, 2, 64]) == Fallback.Shape
+    assert svod_amd.plan_heads(True, [BF16], [2, 0, 768], 64) == Fallback.Shape
+
+
+def test_f16_has_no_kernel_here():
+    """The reference runs f16 on its kernels; this library is bf16 only and says Dtype."""
+    assert svod_amd.plan_attention(True, [F16] * 3, [2, 100, 8, 64], [2, 37, 2, 64]) == Fallback.Dtype
+
+
+# ---- ops_plan.rs:1465-1487 (heads_plan and friends)
+@pytest.mark.parametrize("d,want", [(64, None), (128, None), (16, None), (256, None), (48, Fallback.Shape),
+                                    (512, Fallback.Shape), (8, Fallback.Shape)])
+def test_heads_plan(d, want):
+    assert svod_amd.plan_heads(True, [BF16], [2, 100, 12 * d], d) == want
+
+
+def test_heads_keep_the_graph_for_a_weight_off_the_stream_dtype():
+    assert svod_amd.plan_heads(True, [BF16, F16], [2, 100, 12 * 64], 64) == Fallback.Dtype
+
+
+def test_heads_need_three_dims():
+    assert svod_amd.plan_heads(True, [BF16], [200, 12 * 64], 64) == Fallback.Shape
+
+
+# ---- argument errors: ops_plan.rs:1814-1879 and ops.rs:990-1002
+def kind_of(fn):
+    with pytest.raises(OpError) as e:
+        fn()
+    return e.value.kind, str(e.value)
+
+
+def test_attention_rejects_what_the_graph_would_reject():
+    q = t([2, 10, 6, 64])
+    kv = t([2, 12, 4, 64])
+    kind, msg = kind_of(lambda: svod_amd.attention(q, kv, kv))
+    assert kind == "Heads" and "6 query heads" in msg and "4 key/value heads" in msg
+    kv2 = t([2, 12, 2, 64])
+    kind, msg = kind_of(lambda: svod_amd.attention(q, kv2, t([2, 11, 2, 64])))
+    assert kind == "Shape" and msg.startswith("attention: v has shape")
+    short = t([2, 12, 2, 32])
+    kind, msg = kind_of(lambda: svod_amd.attention(q, short, short))
+    assert kind == "Shape" and msg.startswith("attention: k has shape")
+    kind, msg = kind_of(lambda: svod_amd.attention(q, kv2, kv2, Attn(keys=KeyMask.lens(t([2, 1], I32)))))
+    assert kind == "Shape" and "key lens" in msg
+    kind, msg = kind_of(lambda: svod_amd.attention(q, kv2, kv2, Attn(keys=KeyMask.bool(t([2, 10], torch.bool)))))
+    assert kind == "Shape" and "key mask" in msg
+    kind, msg = kind_of(lambda: svod_amd.attention(q, kv2, kv2, Attn(seg_start=t([2, 12], I32))))
+    assert kind == "Shape" and "seg start" in msg
+    kind, msg = kind_of(lambda: svod_amd.attention(t([2, 10, 64]), kv2, kv2))
+    assert kind == "Shape" and "q has shape" in msg
+    kind, msg = kind_of(lambda: svod_amd.attention(q, kv2.to(F16), kv2.to(F16)))
+    assert kind == "Dtype" and "k is Float16" in msg
+    for dims in ([2, 6, 10, 13], [3, 6, 10, 12], [2, 2, 10, 12], [2, 6, 12, 12]):
+        kind, msg = kind_of(lambda: svod_amd.attention(q, kv2, kv2, Attn(bias=t(dims))))
+        assert kind == "Shape" and "bias" in msg, dims
+
+
+@pytest.mark.parametrize("lens", [[1], [3], [2, 1]], ids=["one length for two rows", "three lengths", "a matrix"])
+def test_attention_rejects_key_lengths_off_the_batch(lens):
+    """ops.rs:993-1002."""
+    q, kv = t([2, 16, 4, 64]), t([2, 32, 4, 64])
+    kind, msg = kind_of(lambda: svod_amd.attention(q, kv, kv, Attn(keys=KeyMask.lens(t(lens, I32)))))
+    assert kind == "Shape" and "key lens" in msg
+
+
+def test_heads_reject_what_the_graph_would_reject():
+    x = t([2, 10, 8 * 64])
+    kind, msg = kind_of(lambda: svod_amd.heads(x, Qkv(4, 3, 64)))
+    assert kind == "Heads"
+    kind, msg = kind_of(lambda: svod_amd.heads(t([2, 10, 7 * 64]), Qkv(4, 2, 64)))
+    assert kind == "Shape" and "qkv has shape" in msg
+    kind, msg = kind_of(lambda: svod_amd.heads(x, Qkv(4, 2, 64, q_norm=t([32]))))
+    assert kind == "Shape" and "q norm" in msg
+    kind, msg = kind_of(lambda: svod_amd.heads(x, Qkv(4, 2, 64, rope=(t([1, 9, 1, 32]), t([1, 9, 1, 32])))))
+    assert kind == "Shape" and "cos has shape" in msg
+    kind, msg = kind_of(lambda: svod_amd.heads(x, Qkv(4, 2, 64, rope=(t([1, 10, 1, 32]), t([2, 10, 1, 32])))))
+    assert kind == "Shape" and "sin has shape" in msg
+
+
+# ---- the three outcomes without a device: validation passes, then the gate says Target
+def test_without_a_device_the_op_names_the_graph_and_records_it():
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present: the Target fallback is the no-device outcome")
+    q, kv = t([2, 16, 4, 64]), t([2, 32, 2, 64])
+    with pytest.raises(GraphFallback) as e:
+        svod_amd.attention(q, kv, kv, Attn(causal=True))
+    assert e.value.why == Fallback.Target
+    assert svod_amd.chosen() == 'Graph { op: "attention", why: Target }'
+    with pytest.raises(GraphFallback) as e:
+        svod_amd.heads(t([2, 10, 8 * 64]), Qkv(4, 2, 64))
+    assert e.value.why == Fallback.Target
+    assert svod_amd.chosen() == 'Graph { op: "heads", why: Target }'
+    assert svod_amd.supported() is False
+
+
+def test_a_missing_library_is_a_hard_error(monkeypatch, tmp_path):
+    """There is no implementation behind the ops other than the HIP library."""
+    import svod_amd.ops as ops
+
+    monkeypatch.setattr(ops, "_lib", None)
+    monkeypatch.setattr(ops, "_HERE", str(tmp_path))
+    with pytest.raises(ImportError, match="no fallback"):
+        ops.load_library()

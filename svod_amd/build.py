@@ -18,7 +18,10 @@ SOURCES = ["ops.cpp", "heads_kernel.hip", "attention_kernel.hip"]
 
 # Packed-FP32 VALU ops are switched off for device code; the host pass of hipcc
 # does not know the feature and says so, which is harmless.
-DEVICE_FLAGS = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+DEVICE_FLAGS = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+                # MFMA results stay in arch VGPRs: the softmax reads them and the rescale writes them
+                # every step, and the AGPR form pays a copy each way.
+                "-mllvm", "-amdgpu-mfma-vgpr-form"]
 COMMON_FLAGS = ["-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-command-line-argument"]
 
 

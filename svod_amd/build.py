@@ -22,6 +22,10 @@ DEVICE_FLAGS = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang"
                 # MFMA results stay in arch VGPRs: the softmax reads them and the rescale writes them
                 # every step, and the AGPR form pays a copy each way.
                 "-mllvm", "-amdgpu-mfma-vgpr-form"]
+# The attention kernel folds MFMA results with max(): without this every operand is first
+# quieted by a max(x, x) of its own (32 extra VALU ops a step).  Nothing in that kernel tests
+# for NaN, and infinities (the masks) stay honoured.
+EXTRA_FLAGS = {"attention_kernel.hip": ["-fno-honor-nans"]}
 COMMON_FLAGS = ["-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-command-line-argument"]
 
 
@@ -39,7 +43,9 @@ def build(verbose: bool = False) -> str:
     objs = []
     for src in SOURCES:
         obj = os.path.join(objdir, os.path.splitext(src)[0] + ".o")
-        cmd = [cc, "-x", "hip", *DEVICE_FLAGS, *COMMON_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+        cmd = [cc, "-x", "hip", *DEVICE_FLAGS, *COMMON_FLAGS, *EXTRA_FLAGS.get(src, []),
+               *os.environ.get("SVODK_CXXFLAGS", "").split(), "-c",
+               os.path.join(CSRC, src), "-o", obj]
         _run(cmd, verbose)
         objs.append(obj)
     _run([cc, *DEVICE_FLAGS, "-shared", "-fPIC", "-o", LIB, *objs], verbose)

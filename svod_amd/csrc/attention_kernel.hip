@@ -22,9 +22,14 @@
 // product as its B operand without leaving registers: B wants, per lane, 8
 // consecutive k-indices of column l%32, and the contraction index is ours to
 // order, so V^T's fragments are fetched in the key order P's registers have.
+//
+// The loop is software-pipelined by one key block inside each wave: while the
+// VALU turns S(j) into P(j), the matrix pipe computes S(j+1), then O += P(j) V(j).
+// On this part a 32x32x16 MFMA leaves room for about four simple VALU
+// instructions beside it, and one wave cannot issue faster than about one
+// instruction per five cycles, so the step's instructions are laid out as
+// "one MFMA, a share of the VALU work, the LDS reads two MFMAs ahead".
 #include <hip/hip_runtime.h>
-
-#include <type_traits>
 
 #include "kernels.h"
 
@@ -32,39 +37,42 @@ namespace svodk {
 namespace {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
-typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 typedef __attribute__((ext_vector_type(4))) short s16x4;
+typedef __attribute__((ext_vector_type(8))) short s16x8;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
-typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(2))) float f32x2;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+typedef __attribute__((ext_vector_type(4))) int i32x4;
 
 #define LDS_PTR(T) T __attribute__((address_space(3))) *
 
-constexpr int kBkv = 64;           // keys per ring slot
-constexpr int kWaveRows = 32;      // query rows a wave owns: the N of the MFMA atom
+constexpr int kBkv = 64;       // keys per ring slot
+constexpr int kWaveRows = 32;  // query rows a wave owns: the N of the MFMA atom
+constexpr int kXcds = 8;       // accelerator dies of an MI355X, each with its own L2
 constexpr float kLog2e = 1.44269504088896340736f;
 constexpr float kRescaleAbove = 8.0f;  // tk/src/kernels/attention.rs:379
 
-// A ring slot holds a [64 keys, D] tile of K and one of V, rows unpadded
-// (D*2 bytes), filled by buffer_load_dwordx4 ... lds: a wave instruction lands
-// 64 consecutive 16-byte chunks, so the only freedom is WHICH global chunk a
-// lane fetches.  Each row's chunks are therefore stored XOR-permuted, with a
-// permutation chosen per tile so that its read pattern touches every bank once:
+// A ring slot holds a [64 keys, D] tile, rows unpadded (D*2 bytes), filled by
+// buffer_load_dwordx4 ... lds: a wave instruction lands 64 consecutive 16-byte
+// chunks, so the only freedom is WHICH global chunk a lane fetches.  Each row's
+// chunks are therefore stored XOR-permuted, with a permutation chosen per tile
+// so that its read pattern touches every bank once:
 //   K is read one chunk per lane, 16 consecutive rows at the same logical chunk
 //     (ds_read_b128 serves 16 lanes a cycle): chunk ^ sK(row) with sK distinct
 //     over 16 rows modulo the 256-byte bank period;
 //   V is read transposed, 4 consecutive rows x 64 contiguous bytes per 32 lanes
 //     (ds_read_b64_tr_b16): the 64-byte group index ^ sV(row) with sV distinct
 //     over 4 rows modulo the period.
+// K runs one block ahead of V, so each has its own pair of slots:
+// LDS = [K slot 0][K slot 1][V slot 0][V slot 1].
 template <int D>
 struct Tile {
   static constexpr int kRowBytes = D * 2;
   static constexpr int kCpr = D / 8;  // 16-byte chunks per row
   static constexpr int kBytes = kBkv * kRowBytes;
-  static constexpr int kStage = 2 * kBytes;  // K then V
+  static constexpr int kLds = 4 * kBytes;
   static constexpr int kInstrs = kBytes / 1024;  // wave-wide 1 KiB fills per tile
   __device__ static constexpr int swz_k(int row) { return D == 64 ? ((row >> 1) & 7) : (row & 15); }
   // In units of 64-byte groups (4 chunks).
@@ -72,6 +80,10 @@ struct Tile {
 };
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+__device__ __forceinline__ float max3(float a, float b, float c) {
+  return __builtin_fmaxf(__builtin_fmaxf(a, b), c);
+}
 
 __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
   f32x2 f = {lo, hi};
@@ -92,46 +104,284 @@ __device__ __forceinline__ Pair both_halves(float x) {
   return {__uint_as_float(r[0]), __uint_as_float(r[1])};
 }
 
-// A raw buffer over `bytes` bytes at `base`: loads past the end return zero,
-// which is how rows at and past a batch's key length read (the bounded views
-// of tk/src/kernels/attention.rs:551-560).
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base, int64_t bytes) {
+// A raw buffer descriptor over `bytes` bytes at `base` (stride 0, 32-bit raw format): loads
+// past the end return zero, which is how rows at and past a batch's key length read (the
+// bounded views of tk/src/kernels/attention.rs:551-560).
+__device__ __forceinline__ i32x4 make_rsrc(const void *base, int64_t bytes) {
   const int64_t clamped = bytes < 0 ? 0 : (bytes > 0xffffffffLL ? 0xffffffffLL : bytes);
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)(uint32_t)clamped, 0x00020000);
+  const uint64_t addr = (uint64_t)(uintptr_t)base;
+  i32x4 r;
+  r[0] = (int)(uint32_t)addr;
+  r[1] = (int)(uint32_t)((addr >> 32) & 0xffffu);
+  r[2] = (int)(uint32_t)clamped;
+  r[3] = 0x00020000;
+  return r;
+}
+
+// Everything a wave carries through the key loop.
+template <int D, int NW>
+struct Wave {
+  static constexpr int KS = D / 16;  // k-steps of the score product
+  static constexpr int DB = D / 32;  // 32-row blocks of O^T
+  static constexpr int CH = Tile<D>::kInstrs / NW;  // fills per wave per tile
+  // block constants
+  const uint8_t *k_base, *v_base;
+  int64_t kv_bytes;  // bytes of this (batch, kv head)'s rows below the length
+  int kv_row_bytes;
+  int end;           // key blocks the query tile sees
+  int len, tk;
+  const void *key_mask;
+  int64_t mask_row;  // b * tk
+  int mask_bytes;
+  int lds0;          // LDS byte address of the ring
+  int wave, lane, g;
+  int wave_first_row, my_row;
+  bool positive;
+  float c_exp, unit, limit;
+  // per-lane addressing
+  int k_src[CH], v_src[CH];  // global byte offsets of this lane's chunk in each fill
+  int k_read[KS], v_read[DB];
+  // state
+  bf16x8 qf[KS];
+  f32x16 acc[DB];
+  float m_run, l_run;
+  int mask_next;
+};
+
+// The fills are issued as raw instructions: the compiler's wait-count pass treats an LDS fill
+// it knows about as aliasing every later LDS read and would park the wave on the NEXT tile's
+// fills in the middle of the current tile.  The kernel waits for them itself (vmcnt(0) before
+// the barrier that ends a step).  m0 carries the LDS address of a wave instruction's 1 KiB.
+template <int D, int NW>
+__device__ __forceinline__ void fill_tile(const Wave<D, NW> &w, const uint8_t *base, int blk, int lds_at,
+                                          const int (&src)[Wave<D, NW>::CH]) {
+  const int64_t off = (int64_t)blk * kBkv * w.kv_row_bytes;
+  const i32x4 r = make_rsrc(base + off, w.kv_bytes - off);
+#pragma unroll
+  for (int i = 0; i < Wave<D, NW>::CH; i++) {
+    const int j = w.wave + NW * i;
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                 :
+                 : "s"(lds_at + j * 1024), "v"(src[i]), "s"(r)
+                 : "memory");
+  }
+}
+template <int D, int NW>
+__device__ __forceinline__ void fill_k(const Wave<D, NW> &w, int blk, int slot) {
+  fill_tile<D, NW>(w, w.k_base, blk, w.lds0 + slot * Tile<D>::kBytes, w.k_src);
+}
+template <int D, int NW>
+__device__ __forceinline__ void fill_v(const Wave<D, NW> &w, int blk, int slot) {
+  fill_tile<D, NW>(w, w.v_base, blk, w.lds0 + (2 + slot) * Tile<D>::kBytes, w.v_src);
+}
+
+// A key mask row is read 64 keys (one per lane) a block, one block ahead: the load is issued
+// before that block's fills and is long back when the block's step needs it.
+template <int D, int NW>
+__device__ __forceinline__ int mask_lane(const Wave<D, NW> &w, int blk) {
+  const int key = blk * kBkv + w.lane;
+  if (w.key_mask == nullptr || key >= w.tk) return 0;
+  const int64_t at = w.mask_row + key;
+  return w.mask_bytes == 1 ? (int)((const uint8_t *)w.key_mask)[at] : ((const int *)w.key_mask)[at];
+}
+
+// S^T = K . Q^T of the key block in K slot `slot`.
+template <int D, int NW>
+__device__ __forceinline__ void scores(const Wave<D, NW> &w, const uint8_t *smem, int slot, f32x16 &s0, f32x16 &s1) {
+  using TL = Tile<D>;
+  const uint8_t *ks_ = smem + slot * TL::kBytes;
+  const f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+  s0 = zero;
+  s1 = zero;
+#pragma unroll
+  for (int ks = 0; ks < Wave<D, NW>::KS; ks++) {
+    const u32x4 a0 = *reinterpret_cast<const u32x4 *>(ks_ + w.k_read[ks]);
+    const u32x4 a1 = *reinterpret_cast<const u32x4 *>(ks_ + w.k_read[ks] + 32 * TL::kRowBytes);
+    s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a0), w.qf[ks], s0, 0, 0, 0);
+    s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a1), w.qf[ks], s1, 0, 0, 0);
+  }
+}
+
+// One step of the key loop for block `blk` (parity PAR = blk & 1: V(blk) is in V slot PAR,
+// K(blk+1) in K slot PAR^1).  (s0, s1) hold S(blk); with MORE, S(blk+1) goes to (n0, n1).
+template <int D, int NW, bool CAUSAL, int PAR, bool MORE>
+__device__ __forceinline__ void step(Wave<D, NW> &w, const uint8_t *smem, int blk, const f32x16 &s0,
+                                     const f32x16 &s1, f32x16 &n0, f32x16 &n1) {
+  using TL = Tile<D>;
+  constexpr int KS = Wave<D, NW>::KS, DB = Wave<D, NW>::DB;
+  const int k0 = blk * kBkv;
+
+  // ---- the wave-uniform part of the mask, and the next block's fills.
+  uint64_t kbits = ~0ull;
+  if (w.key_mask != nullptr) kbits = __builtin_amdgcn_ballot_w64(w.mask_next != 0);
+  if (blk + 1 < w.end) {
+    w.mask_next = mask_lane<D, NW>(w, blk + 1);
+    fill_v<D, NW>(w, blk + 1, PAR ^ 1);
+  }
+  if (blk + 2 < w.end) fill_k<D, NW>(w, blk + 2, PAR);
+  if (k0 + kBkv > w.len) kbits &= (w.len > k0) ? (~0ull >> (64 - (w.len - k0))) : 0ull;
+  const bool diagonal = CAUSAL && (k0 + kBkv - 1 > w.wave_first_row);
+
+  // ---- the scores as 32 scalars (sub-registers of the accumulators: no moves).
+  float sv[32];
+#pragma unroll
+  for (int i = 0; i < 16; i++) {
+    sv[i] = s0[i];
+    sv[16 + i] = s1[i];
+  }
+  if (!w.positive) {
+#pragma unroll
+    for (int i = 0; i < 32; i++) sv[i] *= w.c_exp;
+  }
+  // ---- masks (L641-697) as one 64-bit word per lane: bit j = key k0 + j is kept.  Only
+  // blocks a mask edge crosses pay for it.
+  if (kbits != ~0ull || diagonal) {
+    uint64_t mine = kbits;
+    if (diagonal) {
+      const int seen = w.my_row - k0 + 1;  // keys k0 .. my_row
+      mine &= seen >= 64 ? ~0ull : (seen <= 0 ? 0ull : (~0ull >> (64 - seen)));
+    }
+    mine >>= 4 * w.g;
+    const uint32_t lo = (uint32_t)mine, hi = (uint32_t)(mine >> 32);
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+      const int rel = 8 * (i / 4) + (i % 4);  // key k0 + 32kb + 4g + rel
+      sv[i] = ((lo >> rel) & 1u) ? sv[i] : -INFINITY;
+      sv[16 + i] = ((hi >> rel) & 1u) ? sv[16 + i] : -INFINITY;
+    }
+  }
+
+  // ---- row maximum: in-lane tree of three-way folds, then the other half-wave's.
+  float t8[8];
+#pragma unroll
+  for (int i = 0; i < 8; i++) t8[i] = max3(sv[2 * i], sv[2 * i + 1], __builtin_fmaxf(sv[16 + 2 * i], sv[17 + 2 * i]));
+  float bm = max3(max3(t8[0], t8[1], t8[2]), max3(t8[3], t8[4], t8[5]), __builtin_fmaxf(t8[6], t8[7]));
+  {
+    const Pair p = both_halves(bm);
+    bm = __builtin_fmaxf(p.a, p.b);
+  }
+
+  // ---- lazy rescale (L418-431).
+  const float m_max = __builtin_fmaxf(w.m_run, bm);
+  const bool grows = w.limit < (m_max - w.m_run);
+  const float m_new = grows ? m_max : w.m_run;
+  const float corr = fast_exp2((w.m_run - m_new) * w.unit);
+  const float m_exp = m_new * w.unit;
+  w.m_run = m_new;
+
+  // ---- O^T rescale, skipped by a wave whose rows all kept their maximum (L56-59).
+  if (__builtin_amdgcn_ballot_w64(corr != 1.0f) != 0) {
+#pragma unroll
+    for (int db = 0; db < DB; db++) w.acc[db] *= corr;
+  }
+
+  // ---- from here to the barrier is one scheduling region: the matrix pipe computes
+  // S(blk+1), then O += P V, while the VALU exponentiates.
+  if (MORE) scores<D, NW>(w, smem, PAR ^ 1, n0, n1);
+
+  // p = 2^(s*unit - m*unit), summed unrounded in four chains, then held as bf16 (L432-444).
+  float bs0 = 0.0f, bs1 = 0.0f, bs2 = 0.0f, bs3 = 0.0f;
+  uint32_t pk[16];
+#pragma unroll
+  for (int i = 0; i < 32; i += 4) {
+    const float p0 = fast_exp2(__builtin_fmaf(sv[i], w.unit, -m_exp));
+    const float p1 = fast_exp2(__builtin_fmaf(sv[i + 1], w.unit, -m_exp));
+    const float p2 = fast_exp2(__builtin_fmaf(sv[i + 2], w.unit, -m_exp));
+    const float p3 = fast_exp2(__builtin_fmaf(sv[i + 3], w.unit, -m_exp));
+    bs0 += p0;
+    bs1 += p1;
+    bs2 += p2;
+    bs3 += p3;
+    pk[i / 2] = pack2(p0, p1);
+    pk[i / 2 + 1] = pack2(p2, p3);
+  }
+  w.l_run = w.l_run * corr + ((bs0 + bs1) + (bs2 + bs3));
+
+  // O^T += V^T . P^T : chunk c = 16 keys (c = 2kb + tt), fragment registers 4c .. 4c+3.
+  const uint8_t *vs_ = smem + (2 + PAR) * TL::kBytes;
+#pragma unroll
+  for (int c = 0; c < 4; c++) {
+    const u32x4 pw = {pk[4 * c], pk[4 * c + 1], pk[4 * c + 2], pk[4 * c + 3]};
+    const bf16x8 pf = __builtin_bit_cast(bf16x8, pw);
+#pragma unroll
+    for (int db = 0; db < DB; db++) {
+      const uint8_t *at = vs_ + w.v_read[db] + 16 * c * TL::kRowBytes;
+      const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_PTR(s16x4))(at));
+      const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_PTR(s16x4))(at + 8 * TL::kRowBytes));
+      const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+      w.acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, both), pf, w.acc[db], 0, 0, 0);
+    }
+  }
+
+  // The layout of the region: LDS reads run two matrix instructions ahead of their use, and
+  // each matrix instruction is followed by its share of the VALU work.
+  constexpr int kMfma = (MORE ? 2 * KS : 0) + 4 * DB;
+  constexpr int kValu = 150 / kMfma + 1;
+  __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+  for (int i = 0; i < kMfma; i++) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);      // one MFMA
+    __builtin_amdgcn_sched_group_barrier(0x002, kValu, 0);  // VALU
+    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);      // LDS reads
+  }
+  __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the fills issued this step have landed
+  __syncthreads();
+}
+
+// A step of a wave with nothing to compute: fills and the barrier only.
+template <int D, int NW>
+__device__ __forceinline__ void idle_step(Wave<D, NW> &w, int blk) {
+  const int par = blk & 1;
+  if (blk + 1 < w.end) fill_v<D, NW>(w, blk + 1, par ^ 1);
+  if (blk + 2 < w.end) fill_k<D, NW>(w, blk + 2, par);
+  __builtin_amdgcn_s_waitcnt(0x0f70);
+  __syncthreads();
 }
 
 template <int D, int NW, bool CAUSAL>
-__global__ __launch_bounds__(NW * 64) void flash_fwd_kernel(
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) void flash_fwd_kernel(
     const uint16_t *__restrict__ q, const uint16_t *__restrict__ k, const uint16_t *__restrict__ v,
     uint16_t *__restrict__ o, const void *__restrict__ key_lens, const void *__restrict__ key_mask, int32_t lens_i64,
-    int32_t mask_bytes, int32_t t, int32_t tk, int32_t heads, int32_t kv_heads, int32_t nqt, float scale) {
+    int32_t mask_bytes, int32_t t, int32_t tk, int32_t heads, int32_t kv_heads, int32_t nqt, int32_t nbatch,
+    float scale) {
   // The body is device code only: the host pass needs the kernel's handle, not its
-  // instructions (and drops the whole instantiation over the LDS-fill builtins).
+  // instructions (and drops the whole instantiation over the LDS-fill instructions).
 #if defined(__HIP_DEVICE_COMPILE__)
   using TL = Tile<D>;
+  using W = Wave<D, NW>;
   constexpr int BQ = NW * kWaveRows;
-  constexpr int KS = D / 16;  // k-steps of the score product
-  constexpr int DB = D / 32;  // 32-row blocks of O^T
-  constexpr int CH = TL::kInstrs / NW;  // fills per wave per tile
+  constexpr int KS = W::KS, DB = W::DB, CH = W::CH;
   static_assert(TL::kInstrs % NW == 0, "the tile fills in whole wave instructions per wave");
 
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
 
+  W w;
   const int tid = __builtin_amdgcn_workitem_id_x();
-  const int lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int g = lane >> 5;   // half-wave: the k-chunk of MFMA operands
-  const int ln = lane & 31;  // the query column this lane owns
+  w.lane = tid & 63;
+  w.wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  w.g = w.lane >> 5;           // half-wave: the k-chunk of MFMA operands
+  const int ln = w.lane & 31;  // the query column this lane owns
 
-  // grid x = query tile fastest, then head, then batch (attention.rs:512,523).
-  const int bid = __builtin_amdgcn_workgroup_id_x();
-  const int order = bid % nqt;
-  const int h = (bid / nqt) % heads;
-  const int b = bid / (nqt * heads);
+  // A unit of work is one (batch, KV head): the query tiles of the heads that share its K and
+  // V.  Workgroups are dealt to the 8 XCDs round-robin, each XCD with its own L2, so the units
+  // are dealt to the XCDs round-robin too and a unit's workgroups all land on one XCD: they
+  // meet in one L2 instead of being spread over all eight.  (The reference's grid is query
+  // tile fastest, then head, then batch, attention.rs:512,523; the order within a unit is that.)
+  const int group = heads / kv_heads;
+  const int unit_size = group * nqt;
+  const int units = kv_heads * nbatch;
+  const int wg = __builtin_amdgcn_workgroup_id_x();
+  const int local = wg / kXcds;
+  const int unit = (local / unit_size) * kXcds + wg % kXcds;
+  if (unit >= units) return;
+  const int within = local % unit_size;
+  const int order = within % nqt;
+  const int kvh = unit % kv_heads;  // L548: query head h reads KV head h / (heads / kv_heads)
+  const int h = kvh * group + within / nqt;
+  const int b = unit / kv_heads;
   // Where later queries see more keys the last query blocks run first (L524-528).
   const int qt = CAUSAL ? (nqt - 1 - order) : order;
   const int q_off = qt * BQ;
-  const int kvh = h / (heads / kv_heads);  // L548
 
   // L533-536: len = min(key_lens[b], tk).
   int len = tk;
@@ -144,235 +394,119 @@ __global__ __launch_bounds__(NW * 64) void flash_fwd_kernel(
   int end = (tk + kBkv - 1) / kBkv;
   if (CAUSAL) end = min(end, (q_off + BQ + kBkv - 1) / kBkv);
   if (key_lens != nullptr) end = min(end, (len + kBkv - 1) / kBkv);
+  w.end = end;
+  w.len = len;
+  w.tk = tk;
+  w.key_mask = key_mask;
+  w.mask_row = (int64_t)b * tk;
+  w.mask_bytes = mask_bytes;
 
   const int64_t q_row_stride = (int64_t)heads * D;
-  const int kv_row_bytes = kv_heads * D * 2;
-  const uint8_t *k_base = (const uint8_t *)(k + ((int64_t)b * tk * kv_heads + kvh) * D);
-  const uint8_t *v_base = (const uint8_t *)(v + ((int64_t)b * tk * kv_heads + kvh) * D);
-  // Bytes of this (batch, kv head)'s rows below the length, measured from its first row.
-  const int64_t kv_bytes = len > 0 ? (int64_t)(len - 1) * kv_row_bytes + D * 2 : 0;
+  w.kv_row_bytes = kv_heads * D * 2;
+  w.k_base = (const uint8_t *)(k + ((int64_t)b * tk * kv_heads + kvh) * D);
+  w.v_base = (const uint8_t *)(v + ((int64_t)b * tk * kv_heads + kvh) * D);
+  w.kv_bytes = len > 0 ? (int64_t)(len - 1) * w.kv_row_bytes + D * 2 : 0;
+  w.lds0 = (int)(uintptr_t)(LDS_PTR(uint8_t))(smem);
 
   // ---- Q fragments: B operand of the score product, resident for the block.
-  const int wave_first_row = q_off + wave * kWaveRows;
-  const int my_row = wave_first_row + ln;
-  bf16x8 qf[KS];
+  w.wave_first_row = q_off + w.wave * kWaveRows;
+  w.my_row = w.wave_first_row + ln;
   {
-    const uint16_t *q_ptr = q + ((int64_t)b * t + my_row) * q_row_stride + (int64_t)h * D + g * 8;
+    const uint16_t *q_ptr = q + ((int64_t)b * t + w.my_row) * q_row_stride + (int64_t)h * D + w.g * 8;
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
-      u32x4 w = {0, 0, 0, 0};
-      if (my_row < t) w = *reinterpret_cast<const u32x4 *>(q_ptr + ks * 16);
-      qf[ks] = __builtin_bit_cast(bf16x8, w);
+      u32x4 x = {0, 0, 0, 0};
+      if (w.my_row < t) x = *reinterpret_cast<const u32x4 *>(q_ptr + ks * 16);
+      w.qf[ks] = __builtin_bit_cast(bf16x8, x);
     }
   }
 
-  // ---- ring fill: this wave's share of a tile, CH wave-wide 1 KiB fills of K and of V.
-  // Fill j lands on rows [j*rows_per, ...): lane i at physical chunk i % kCpr of row i / kCpr.
+  // ---- this wave's share of a tile fill: CH wave-wide 1 KiB instructions.  Fill j lands on
+  // rows [j*rows_per, ...): lane i at physical chunk i % kCpr of row i / kCpr.
   constexpr int kRowsPer = 64 / TL::kCpr;
-  int k_src[CH], v_src[CH];
 #pragma unroll
   for (int i = 0; i < CH; i++) {
-    const int j = wave + NW * i;
-    const int row = j * kRowsPer + lane / TL::kCpr;
-    const int pc = lane % TL::kCpr;
-    k_src[i] = row * kv_row_bytes + ((pc ^ TL::swz_k(row)) << 4);
-    v_src[i] = row * kv_row_bytes + ((pc ^ (TL::swz_v(row) << 2)) << 4);
+    const int j = w.wave + NW * i;
+    const int row = j * kRowsPer + w.lane / TL::kCpr;
+    const int pc = w.lane % TL::kCpr;
+    w.k_src[i] = row * w.kv_row_bytes + ((pc ^ TL::swz_k(row)) << 4);
+    w.v_src[i] = row * w.kv_row_bytes + ((pc ^ (TL::swz_v(row) << 2)) << 4);
   }
-  auto fill = [&](int blk, int stage) {
-    const int64_t off = (int64_t)blk * kBkv * kv_row_bytes;
-    const __amdgpu_buffer_rsrc_t kr = make_rsrc(k_base + off, kv_bytes - off);
-    const __amdgpu_buffer_rsrc_t vr = make_rsrc(v_base + off, kv_bytes - off);
-    uint8_t *ks = smem + stage * TL::kStage;
-#pragma unroll
-    for (int i = 0; i < CH; i++) {
-      const int j = wave + NW * i;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, (LDS_PTR(void))(ks + j * 1024), 16, k_src[i], 0, 0, 0);
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, (LDS_PTR(void))(ks + TL::kBytes + j * 1024), 16, v_src[i], 0, 0, 0);
-    }
-  };
-
   // ---- per-lane LDS offsets of the operand reads.
   // K fragment (kb, ks): row 32kb + ln, logical chunk 2ks + g.
-  int k_read[KS];
 #pragma unroll
-  for (int ks = 0; ks < KS; ks++) k_read[ks] = ln * TL::kRowBytes + (((2 * ks + g) ^ TL::swz_k(ln)) << 4);
-  // V^T fragment (kb, tt, half, db): lanes 4j..4j+3 of a 16-lane group supply row j
-  // (four 4-element runs), lane i of the group receives column i of those 4 rows.
-  const int vq = (lane & 15) >> 2;                        // row within the group of 4
-  const int vc = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);  // chunk within the 64-byte group
-  int v_read[DB];
+  for (int ks = 0; ks < KS; ks++) w.k_read[ks] = ln * TL::kRowBytes + (((2 * ks + w.g) ^ TL::swz_k(ln)) << 4);
+  // V^T fragment: lanes 4j..4j+3 of a 16-lane group supply row j (four 4-element runs),
+  // lane i of the group receives column i of those 4 rows.
+  const int vq = (w.lane & 15) >> 2;                             // row within the group of 4
+  const int vc = 2 * ((w.lane >> 4) & 1) + ((w.lane & 3) >> 1);  // chunk within the 64-byte group
 #pragma unroll
   for (int db = 0; db < DB; db++)
-    v_read[db] = (4 * g + vq) * TL::kRowBytes + ((db ^ TL::swz_v(vq)) << 6) + (vc << 4) + ((lane & 1) << 3);
+    w.v_read[db] = (4 * w.g + vq) * TL::kRowBytes + ((db ^ TL::swz_v(vq)) << 6) + (vc << 4) + ((w.lane & 1) << 3);
 
-  // ---- online softmax state.  m in RAW score units (raw_max form).
-  const bool positive = scale > 0.0f;
-  const float c_exp = scale * kLog2e;  // L619
-  // With a non-positive scale the maximum does not commute with it: the scores
-  // are scaled first and m lives in the exponent's units (L365-370).
-  const float unit = positive ? c_exp : 1.0f;
-  const float limit = kRescaleAbove / unit;
-  float m_run = -1e30f, l_run = 0.0f;
-  f32x16 acc[DB];
+  // ---- online softmax state.  m in RAW score units (raw_max form) when the scale is positive;
+  // otherwise the maximum does not commute with it: the scores are scaled first and m lives
+  // in the exponent's units (L365-370).
+  w.positive = scale > 0.0f;
+  w.c_exp = scale * kLog2e;  // L619
+  w.unit = w.positive ? w.c_exp : 1.0f;
+  w.limit = kRescaleAbove / w.unit;
+  w.m_run = -1e30f;
+  w.l_run = 0.0f;
+  const f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-  for (int db = 0; db < DB; db++)
-#pragma unroll
-    for (int i = 0; i < 16; i++) acc[db][i] = 0.0f;
+  for (int db = 0; db < DB; db++) w.acc[db] = zero;
 
-  if (end > 0) fill(0, 0);
-  __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's fills have landed
+  // ---- prologue: K(0), V(0), K(1) in flight, then the first block's scores.
+  w.mask_next = mask_lane<D, NW>(w, 0);
+  if (end > 0) {
+    fill_k<D, NW>(w, 0, 0);
+    fill_v<D, NW>(w, 0, 0);
+  }
+  if (end > 1) fill_k<D, NW>(w, 1, 1);
+  // A wait the compiler knows of: it covers the Q loads too, so that no wait of its own for
+  // them lands inside the loop, where it would also wait out the fills in flight.
+  __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
   __syncthreads();
 
-  auto step = [&](int blk, auto stage_c) {
-    constexpr int stage = decltype(stage_c)::value;
-    const int k0 = blk * kBkv;
-    if (blk + 1 < end) fill(blk + 1, stage ^ 1);
+  // A causal wave past its last visible key has nothing to add from a block: it only keeps
+  // filling and meeting the barriers.  Blocks [0, my_end) are this wave's.
+  int my_end = end;
+  if (CAUSAL) my_end = min(end, (w.wave_first_row + kWaveRows - 1) / kBkv + 1);
 
-    const uint8_t *ks_ = smem + stage * TL::kStage;
-    const uint8_t *vs_ = ks_ + TL::kBytes;
-    // A causal wave past its last visible key has nothing to add from this block.
-    const bool idle = CAUSAL && k0 > wave_first_row + kWaveRows - 1;
-    if (!idle) {
-      // ---- S^T = K . Q^T
-      f32x16 s[2];
-#pragma unroll
-      for (int kb = 0; kb < 2; kb++) {
-#pragma unroll
-        for (int i = 0; i < 16; i++) s[kb][i] = 0.0f;
-#pragma unroll
-        for (int ks = 0; ks < KS; ks++) {
-          const u32x4 w = *reinterpret_cast<const u32x4 *>(ks_ + k_read[ks] + kb * 32 * TL::kRowBytes);
-          s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, w), qf[ks], s[kb], 0, 0, 0);
-        }
-      }
-      if (!positive) {
-#pragma unroll
-        for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-          for (int i = 0; i < 16; i++) s[kb][i] *= c_exp;
-      }
-
-      // ---- masks (L641-697) as one 64-bit word per lane: bit j = key k0 + j is kept.
-      // The length and the key mask give a wave-uniform word; causality a per-lane one.
-      uint64_t kbits = ~0ull;
-      if (key_mask != nullptr) {
-        const int key = k0 + lane;
-        bool vis = false;
-        if (key < tk) {
-          const int64_t at = (int64_t)b * tk + key;
-          vis = mask_bytes == 1 ? ((const uint8_t *)key_mask)[at] != 0 : ((const int *)key_mask)[at] != 0;
-        }
-        kbits = __builtin_amdgcn_ballot_w64(vis);
-      }
-      if (k0 + kBkv > len) kbits &= (len > k0) ? (~0ull >> (64 - (len - k0))) : 0ull;
-      const bool diagonal = CAUSAL && (k0 + kBkv - 1 > wave_first_row);
-      if (kbits != ~0ull || diagonal) {
-        uint64_t mine = kbits;
-        if (diagonal) {
-          const int seen = my_row - k0 + 1;  // keys k0 .. my_row
-          mine &= seen >= 64 ? ~0ull : (seen <= 0 ? 0ull : (~0ull >> (64 - seen)));
-        }
-        mine >>= 4 * g;
-#pragma unroll
-        for (int kb = 0; kb < 2; kb++) {
-          const uint32_t word = kb ? (uint32_t)(mine >> 32) : (uint32_t)mine;
-#pragma unroll
-          for (int i = 0; i < 16; i++) {
-            const int rel = 8 * (i / 4) + (i % 4);  // key k0 + 32kb + 4g + rel
-            s[kb][i] = ((word >> rel) & 1u) ? s[kb][i] : -INFINITY;
-          }
-        }
-      }
-
-      // ---- row maximum: in-lane tree, then the other half-wave's.
-      float t8[8];
-#pragma unroll
-      for (int i = 0; i < 8; i++) t8[i] = fmaxf(fmaxf(s[0][2 * i], s[0][2 * i + 1]), fmaxf(s[1][2 * i], s[1][2 * i + 1]));
-      float bm = fmaxf(fmaxf(fmaxf(t8[0], t8[1]), fmaxf(t8[2], t8[3])), fmaxf(fmaxf(t8[4], t8[5]), fmaxf(t8[6], t8[7])));
-      {
-        const Pair p = both_halves(bm);
-        bm = fmaxf(p.a, p.b);
-      }
-
-      // ---- lazy rescale (L418-431).
-      const float m_max = fmaxf(m_run, bm);
-      const bool grows = limit < (m_max - m_run);
-      const float m_new = grows ? m_max : m_run;
-      const float corr = fast_exp2((m_run - m_new) * unit);
-      const float m_exp = m_new * unit;
-      m_run = m_new;
-
-      // ---- p = 2^(s*unit - m*unit), held as bf16 (L432-435); the row sum adds the
-      // probabilities as held, two per v_dot2 (the `truncate_p` form's rule, L436-444,
-      // applied to the rounded values), in four independent chains.
-      float bs[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-      uint32_t pk[2][8];
-      const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
-#pragma unroll
-      for (int kb = 0; kb < 2; kb++) {
-#pragma unroll
-        for (int i = 0; i < 16; i += 2) {
-          const float p0 = fast_exp2(__builtin_fmaf(s[kb][i], unit, -m_exp));
-          const float p1 = fast_exp2(__builtin_fmaf(s[kb][i + 1], unit, -m_exp));
-          const uint32_t w = pack2(p0, p1);
-          pk[kb][i / 2] = w;
-          bs[(i / 2) & 3] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, w), ones, bs[(i / 2) & 3], false);
-        }
-      }
-      l_run = l_run * corr + ((bs[0] + bs[1]) + (bs[2] + bs[3]));
-
-      // ---- O^T rescale, skipped by a wave whose rows all kept their maximum (L56-59).
-      if (__builtin_amdgcn_ballot_w64(corr != 1.0f) != 0) {
-#pragma unroll
-        for (int db = 0; db < DB; db++)
-#pragma unroll
-          for (int i = 0; i < 16; i++) acc[db][i] *= corr;
-      }
-
-      // ---- O^T += V^T . P^T
-#pragma unroll
-      for (int kb = 0; kb < 2; kb++) {
-#pragma unroll
-        for (int tt = 0; tt < 2; tt++) {
-          u32x4 pw = {pk[kb][4 * tt], pk[kb][4 * tt + 1], pk[kb][4 * tt + 2], pk[kb][4 * tt + 3]};
-          const bf16x8 pf = __builtin_bit_cast(bf16x8, pw);
-#pragma unroll
-          for (int db = 0; db < DB; db++) {
-            const uint8_t *at = vs_ + v_read[db] + (32 * kb + 16 * tt) * TL::kRowBytes;
-            const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_PTR(s16x4))(at));
-            const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_PTR(s16x4))(at + 8 * TL::kRowBytes));
-            typedef __attribute__((ext_vector_type(8))) short s16x8;
-            const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-            acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, both), pf, acc[db], 0, 0, 0);
-          }
-        }
-      }
-    }
-    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the next tile's fills have landed
-    __syncthreads();
-  };
+  f32x16 a0 = zero, a1 = zero, b0 = zero, b1 = zero;
+  if (my_end > 0) scores<D, NW>(w, smem, 0, a0, a1);
 
   int blk = 0;
-  for (; blk + 2 <= end; blk += 2) {
-    step(blk, std::integral_constant<int, 0>{});
-    step(blk + 1, std::integral_constant<int, 1>{});
+  for (; blk + 2 < my_end; blk += 2) {
+    step<D, NW, CAUSAL, 0, true>(w, smem, blk, a0, a1, b0, b1);
+    step<D, NW, CAUSAL, 1, true>(w, smem, blk + 1, b0, b1, a0, a1);
   }
-  if (blk < end) step(blk, std::integral_constant<int, 0>{});
+  // One or two blocks of this wave are left; S(blk) is in (a0, a1).
+  if (blk + 2 == my_end) {
+    step<D, NW, CAUSAL, 0, true>(w, smem, blk, a0, a1, b0, b1);
+    step<D, NW, CAUSAL, 1, false>(w, smem, blk + 1, b0, b1, a0, a1);
+    blk += 2;
+  } else if (blk + 1 == my_end) {
+    step<D, NW, CAUSAL, 0, false>(w, smem, blk, a0, a1, b0, b1);
+    blk += 1;
+  }
+  for (; blk < end; blk++) idle_step<D, NW>(w, blk);
 
   // ---- out = o / (l == 0 ? 1 : l), bounded store (L892-898, L974-980).
-  const Pair lp = both_halves(l_run);
+  const Pair lp = both_halves(w.l_run);
   const float l_tot = lp.a + lp.b;
   const float inv = 1.0f / (l_tot == 0.0f ? 1.0f : l_tot);
-  if (my_row < t) {
-    uint16_t *o_ptr = o + ((int64_t)b * t + my_row) * q_row_stride + (int64_t)h * D + 4 * g;
+  if (w.my_row < t) {
+    uint16_t *o_ptr = o + ((int64_t)b * t + w.my_row) * q_row_stride + (int64_t)h * D + 4 * w.g;
 #pragma unroll
     for (int db = 0; db < DB; db++) {
 #pragma unroll
       for (int c = 0; c < 4; c++) {
-        u32x2 w;
-        w[0] = pack2(acc[db][4 * c] * inv, acc[db][4 * c + 1] * inv);
-        w[1] = pack2(acc[db][4 * c + 2] * inv, acc[db][4 * c + 3] * inv);
-        *reinterpret_cast<u32x2 *>(o_ptr + 32 * db + 8 * c) = w;
+        u32x2 x;
+        x[0] = pack2(w.acc[db][4 * c] * inv, w.acc[db][4 * c + 1] * inv);
+        x[1] = pack2(w.acc[db][4 * c + 2] * inv, w.acc[db][4 * c + 3] * inv);
+        *reinterpret_cast<u32x2 *>(o_ptr + 32 * db + 8 * c) = x;
       }
     }
   }
@@ -386,8 +520,8 @@ hipError_t launch(const AttnArgs &a, hipStream_t stream) {
   const int nqt = (a.t + BQ - 1) / BQ;
   const int64_t blocks = (int64_t)nqt * a.heads * a.batch;
   if (blocks == 0) return hipSuccess;
-  if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;
-  constexpr int smem = 2 * TL::kStage;
+  if (blocks > 0x7ffffff0LL) return hipErrorInvalidConfiguration;
+  constexpr int smem = TL::kLds;
   // The fills address a (batch, kv head)'s rows with 32-bit byte offsets.
   if ((int64_t)a.tk * a.kv_heads * a.d * 2 > 0x7fffffffLL) return hipErrorInvalidValue;
   auto kernel = flash_fwd_kernel<D, NW, CAUSAL>;
@@ -398,9 +532,15 @@ hipError_t launch(const AttnArgs &a, hipStream_t stream) {
     if (e != hipSuccess) return e;
     configured = true;
   }
-  hipLaunchKernelGGL(kernel, dim3((uint32_t)blocks), dim3(NW * 64), smem, stream, (const uint16_t *)a.q,
+  // Units of work (batch, KV head) are dealt over the XCDs in whole rounds; the workgroups of
+  // a round's missing units exit at once.
+  const int64_t unit_size = (int64_t)(a.heads / a.kv_heads) * nqt;
+  const int64_t units = (int64_t)a.kv_heads * a.batch;
+  const int64_t grid = (units + kXcds - 1) / kXcds * kXcds * unit_size;
+  if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
+  hipLaunchKernelGGL(kernel, dim3((uint32_t)grid), dim3(NW * 64), smem, stream, (const uint16_t *)a.q,
                      (const uint16_t *)a.k, (const uint16_t *)a.v, (uint16_t *)a.o, a.key_lens, a.key_mask, a.lens_i64,
-                     a.mask_bytes, a.t, a.tk, a.heads, a.kv_heads, nqt, a.scale);
+                     a.mask_bytes, a.t, a.tk, a.heads, a.kv_heads, nqt, a.batch, a.scale);
   return hipGetLastError();
 }
 

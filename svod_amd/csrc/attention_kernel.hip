@@ -24,7 +24,7 @@
 // order, so V^T's fragments are fetched in the key order P's registers have.
 //
 // The loop is software-pipelined by one key block inside each wave: while the
-// VALU turns S(j) into P(j), the matrix pipe computes S(j+1), then O += P(j) V(j).
+// VALU turns S(j) into P(j), the matrix pipe computes S(j+1) and O += P(j) V(j).
 // On this part a 32x32x16 MFMA leaves room for about four simple VALU
 // instructions beside it, and one wave cannot issue faster than about one
 // instruction per five cycles, so the step's instructions are laid out as
@@ -185,14 +185,14 @@ __device__ __forceinline__ int mask_lane(const Wave<D, NW> &w, int blk) {
   return w.mask_bytes == 1 ? (int)((const uint8_t *)w.key_mask)[at] : ((const int *)w.key_mask)[at];
 }
 
-// S^T = K . Q^T of the key block in K slot `slot`.
+// S^T = K . Q^T of the key block in K slot `slot`, as 32 scalars: sv[16kb + i] is the score of
+// key 32kb + 8(i/4) + 4g + i%4 (sub-registers of the two accumulators: no moves).
 template <int D, int NW>
-__device__ __forceinline__ void scores(const Wave<D, NW> &w, const uint8_t *smem, int slot, f32x16 &s0, f32x16 &s1) {
+__device__ __forceinline__ void scores(const Wave<D, NW> &w, const uint8_t *smem, int slot, float (&sv)[32]) {
   using TL = Tile<D>;
   const uint8_t *ks_ = smem + slot * TL::kBytes;
   const f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-  s0 = zero;
-  s1 = zero;
+  f32x16 s0 = zero, s1 = zero;
 #pragma unroll
   for (int ks = 0; ks < Wave<D, NW>::KS; ks++) {
     const u32x4 a0 = *reinterpret_cast<const u32x4 *>(ks_ + w.k_read[ks]);
@@ -200,129 +200,209 @@ __device__ __forceinline__ void scores(const Wave<D, NW> &w, const uint8_t *smem
     s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a0), w.qf[ks], s0, 0, 0, 0);
     s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a1), w.qf[ks], s1, 0, 0, 0);
   }
-}
-
-// One step of the key loop for block `blk` (parity PAR = blk & 1: V(blk) is in V slot PAR,
-// K(blk+1) in K slot PAR^1).  (s0, s1) hold S(blk); with MORE, S(blk+1) goes to (n0, n1).
-template <int D, int NW, bool CAUSAL, int PAR, bool MORE>
-__device__ __forceinline__ void step(Wave<D, NW> &w, const uint8_t *smem, int blk, const f32x16 &s0,
-                                     const f32x16 &s1, f32x16 &n0, f32x16 &n1) {
-  using TL = Tile<D>;
-  constexpr int KS = Wave<D, NW>::KS, DB = Wave<D, NW>::DB;
-  const int k0 = blk * kBkv;
-
-  // ---- the wave-uniform part of the mask, and the next block's fills.
-  uint64_t kbits = ~0ull;
-  if (w.key_mask != nullptr) kbits = __builtin_amdgcn_ballot_w64(w.mask_next != 0);
-  if (blk + 1 < w.end) {
-    w.mask_next = mask_lane<D, NW>(w, blk + 1);
-    fill_v<D, NW>(w, blk + 1, PAR ^ 1);
-  }
-  if (blk + 2 < w.end) fill_k<D, NW>(w, blk + 2, PAR);
-  if (k0 + kBkv > w.len) kbits &= (w.len > k0) ? (~0ull >> (64 - (w.len - k0))) : 0ull;
-  const bool diagonal = CAUSAL && (k0 + kBkv - 1 > w.wave_first_row);
-
-  // ---- the scores as 32 scalars (sub-registers of the accumulators: no moves).
-  float sv[32];
 #pragma unroll
   for (int i = 0; i < 16; i++) {
     sv[i] = s0[i];
     sv[16 + i] = s1[i];
   }
-  if (!w.positive) {
-#pragma unroll
-    for (int i = 0; i < 32; i++) sv[i] *= w.c_exp;
+}
+
+// The wave-uniform part of block `blk`'s mask: bit j = key 64 blk + j is below the length and
+// kept by the key mask (`word` is this lane's key-mask element of the block).
+template <int D, int NW>
+__device__ __forceinline__ uint64_t uniform_bits(const Wave<D, NW> &w, int blk, int word) {
+  const int k0 = blk * kBkv;
+  uint64_t kbits = ~0ull;
+  if (w.key_mask != nullptr) kbits = __builtin_amdgcn_ballot_w64(word != 0);
+  if (k0 + kBkv > w.len) kbits &= (w.len > k0) ? (~0ull >> (64 - (w.len - k0))) : 0ull;
+  return kbits;
+}
+
+// Whether a mask edge crosses block `blk` for this wave (L698-733).
+template <int D, int NW, bool CAUSAL>
+__device__ __forceinline__ bool on_edge(const Wave<D, NW> &w, int blk, uint64_t kbits) {
+  return kbits != ~0ull || (CAUSAL && (blk * kBkv + kBkv - 1 > w.wave_first_row));
+}
+
+// Scales (a non-positive scale only) and masks (L641-697) the scores of block `blk`: hidden
+// scores become -inf.  `kbits` is the uniform word; causality adds a per-lane one.
+template <int D, int NW, bool CAUSAL>
+__device__ __forceinline__ void mask_scores(const Wave<D, NW> &w, int blk, uint64_t kbits, float (&sv)[32]) {
+  const int k0 = blk * kBkv;
+  uint64_t mine = kbits;
+  if (CAUSAL && (k0 + kBkv - 1 > w.wave_first_row)) {
+    const int seen = w.my_row - k0 + 1;  // keys k0 .. my_row
+    mine &= seen >= 64 ? ~0ull : (seen <= 0 ? 0ull : (~0ull >> (64 - seen)));
   }
-  // ---- masks (L641-697) as one 64-bit word per lane: bit j = key k0 + j is kept.  Only
-  // blocks a mask edge crosses pay for it.
-  if (kbits != ~0ull || diagonal) {
-    uint64_t mine = kbits;
-    if (diagonal) {
-      const int seen = w.my_row - k0 + 1;  // keys k0 .. my_row
-      mine &= seen >= 64 ? ~0ull : (seen <= 0 ? 0ull : (~0ull >> (64 - seen)));
-    }
-    mine >>= 4 * w.g;
-    const uint32_t lo = (uint32_t)mine, hi = (uint32_t)(mine >> 32);
+  mine >>= 4 * w.g;
+  const uint32_t lo = (uint32_t)mine, hi = (uint32_t)(mine >> 32);
 #pragma unroll
-    for (int i = 0; i < 16; i++) {
-      const int rel = 8 * (i / 4) + (i % 4);  // key k0 + 32kb + 4g + rel
-      sv[i] = ((lo >> rel) & 1u) ? sv[i] : -INFINITY;
-      sv[16 + i] = ((hi >> rel) & 1u) ? sv[16 + i] : -INFINITY;
-    }
+  for (int i = 0; i < 16; i++) {
+    const int rel = 8 * (i / 4) + (i % 4);  // key k0 + 32kb + 4g + rel
+    sv[i] = ((lo >> rel) & 1u) ? sv[i] : -INFINITY;
+    sv[16 + i] = ((hi >> rel) & 1u) ? sv[16 + i] : -INFINITY;
   }
+}
 
-  // ---- row maximum: in-lane tree of three-way folds, then the other half-wave's.
-  float t8[8];
+// The row maximum of a block's scores: in-lane tree of three-way folds, then the other
+// half-wave's.
+__device__ __forceinline__ float row_max(const float (&sv)[32]) {
+  float t[11];
 #pragma unroll
-  for (int i = 0; i < 8; i++) t8[i] = max3(sv[2 * i], sv[2 * i + 1], __builtin_fmaxf(sv[16 + 2 * i], sv[17 + 2 * i]));
-  float bm = max3(max3(t8[0], t8[1], t8[2]), max3(t8[3], t8[4], t8[5]), __builtin_fmaxf(t8[6], t8[7]));
-  {
-    const Pair p = both_halves(bm);
-    bm = __builtin_fmaxf(p.a, p.b);
-  }
+  for (int i = 0; i < 10; i++) t[i] = max3(sv[3 * i], sv[3 * i + 1], sv[3 * i + 2]);
+  t[10] = __builtin_fmaxf(sv[30], sv[31]);
+  const float u0 = max3(t[0], t[1], t[2]), u1 = max3(t[3], t[4], t[5]), u2 = max3(t[6], t[7], t[8]);
+  const float bm = max3(max3(u0, u1, u2), t[9], t[10]);
+  const Pair p = both_halves(bm);
+  return __builtin_fmaxf(p.a, p.b);
+}
 
-  // ---- lazy rescale (L418-431).
-  const float m_max = __builtin_fmaxf(w.m_run, bm);
-  const bool grows = w.limit < (m_max - w.m_run);
-  const float m_new = grows ? m_max : w.m_run;
-  const float corr = fast_exp2((w.m_run - m_new) * w.unit);
-  const float m_exp = m_new * w.unit;
-  w.m_run = m_new;
-
-  // ---- O^T rescale, skipped by a wave whose rows all kept their maximum (L56-59).
-  if (__builtin_amdgcn_ballot_w64(corr != 1.0f) != 0) {
+// Half a block's probabilities: p = 2^(s*unit - m*unit) for 16 scores, summed unrounded in
+// four chains, then held as bf16 (L432-444).
+__device__ __forceinline__ void probabilities(const float *sv, float unit, float m_exp, float (&bs)[4],
+                                              uint32_t *pk) {
 #pragma unroll
-    for (int db = 0; db < DB; db++) w.acc[db] *= corr;
-  }
-
-  // ---- from here to the barrier is one scheduling region: the matrix pipe computes
-  // S(blk+1), then O += P V, while the VALU exponentiates.
-  if (MORE) scores<D, NW>(w, smem, PAR ^ 1, n0, n1);
-
-  // p = 2^(s*unit - m*unit), summed unrounded in four chains, then held as bf16 (L432-444).
-  float bs0 = 0.0f, bs1 = 0.0f, bs2 = 0.0f, bs3 = 0.0f;
-  uint32_t pk[16];
-#pragma unroll
-  for (int i = 0; i < 32; i += 4) {
-    const float p0 = fast_exp2(__builtin_fmaf(sv[i], w.unit, -m_exp));
-    const float p1 = fast_exp2(__builtin_fmaf(sv[i + 1], w.unit, -m_exp));
-    const float p2 = fast_exp2(__builtin_fmaf(sv[i + 2], w.unit, -m_exp));
-    const float p3 = fast_exp2(__builtin_fmaf(sv[i + 3], w.unit, -m_exp));
-    bs0 += p0;
-    bs1 += p1;
-    bs2 += p2;
-    bs3 += p3;
+  for (int i = 0; i < 16; i += 4) {
+    const float p0 = fast_exp2(__builtin_fmaf(sv[i], unit, -m_exp));
+    const float p1 = fast_exp2(__builtin_fmaf(sv[i + 1], unit, -m_exp));
+    const float p2 = fast_exp2(__builtin_fmaf(sv[i + 2], unit, -m_exp));
+    const float p3 = fast_exp2(__builtin_fmaf(sv[i + 3], unit, -m_exp));
+    bs[0] += p0;
+    bs[1] += p1;
+    bs[2] += p2;
+    bs[3] += p3;
     pk[i / 2] = pack2(p0, p1);
     pk[i / 2 + 1] = pack2(p2, p3);
   }
-  w.l_run = w.l_run * corr + ((bs0 + bs1) + (bs2 + bs3));
+}
 
-  // O^T += V^T . P^T : chunk c = 16 keys (c = 2kb + tt), fragment registers 4c .. 4c+3.
-  const uint8_t *vs_ = smem + (2 + PAR) * TL::kBytes;
+// O^T += V^T . P^T over 32 keys (half a block): chunks c of 16 keys, fragment registers 4c..4c+3.
+template <int D, int NW>
+__device__ __forceinline__ void accumulate(Wave<D, NW> &w, const uint8_t *vs_, int half, const uint32_t *pk) {
+  using TL = Tile<D>;
 #pragma unroll
-  for (int c = 0; c < 4; c++) {
+  for (int c = 0; c < 2; c++) {
     const u32x4 pw = {pk[4 * c], pk[4 * c + 1], pk[4 * c + 2], pk[4 * c + 3]};
     const bf16x8 pf = __builtin_bit_cast(bf16x8, pw);
 #pragma unroll
-    for (int db = 0; db < DB; db++) {
-      const uint8_t *at = vs_ + w.v_read[db] + 16 * c * TL::kRowBytes;
+    for (int db = 0; db < Wave<D, NW>::DB; db++) {
+      const uint8_t *at = vs_ + w.v_read[db] + (32 * half + 16 * c) * TL::kRowBytes;
       const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_PTR(s16x4))(at));
       const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_PTR(s16x4))(at + 8 * TL::kRowBytes));
       const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
       w.acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, both), pf, w.acc[db], 0, 0, 0);
     }
   }
+}
 
-  // The layout of the region: LDS reads run two matrix instructions ahead of their use, and
-  // each matrix instruction is followed by its share of the VALU work.
-  constexpr int kMfma = (MORE ? 2 * KS : 0) + 4 * DB;
-  constexpr int kValu = 150 / kMfma + 1;
+// The running maximum's update for a block whose row maximum is `bm`: the lazy rescale of
+// L418-431, and the O^T rescale that a wave skips when all its rows kept their maximum
+// (L56-59).  Returns the exponent's offset m*unit; `corr` is the correction of l.
+template <int D, int NW>
+__device__ __forceinline__ float adopt_maximum(Wave<D, NW> &w, float bm, float &corr) {
+  const float m_max = __builtin_fmaxf(w.m_run, bm);
+  const bool grows = w.limit < (m_max - w.m_run);
+  const float m_new = grows ? m_max : w.m_run;
+  corr = fast_exp2((w.m_run - m_new) * w.unit);
+  w.m_run = m_new;
+  if (__builtin_amdgcn_ballot_w64(corr != 1.0f) != 0) {
+#pragma unroll
+    for (int db = 0; db < Wave<D, NW>::DB; db++) w.acc[db] *= corr;
+  }
+  return m_new * w.unit;
+}
+
+// The hot step: block `blk` (parity PAR = blk & 1: V(blk) in V slot PAR, K(blk+1) in K slot
+// PAR^1) when block blk+1 is this wave's too, no mask edge crosses it and the scale is
+// positive.  `sv` holds S(blk) and `bm` its row maximum; S(blk+1) goes to `nv`, its maximum to
+// `bm`.  From the rescale to the barrier it is one scheduling region in which the matrix pipe
+// never waits for the VALU's whole job: S(blk+1) beside the first half's exponentials,
+// O += P V of the first half beside the second half's exponentials, O += P V of the second
+// half beside the row maximum of S(blk+1).
+template <int D, int NW, int PAR>
+__device__ __forceinline__ void hot_step(Wave<D, NW> &w, const uint8_t *smem, int blk, const float (&sv)[32],
+                                         float (&nv)[32], float &bm) {
+  using TL = Tile<D>;
+  constexpr int KS = Wave<D, NW>::KS, DB = Wave<D, NW>::DB;
+  fill_v<D, NW>(w, blk + 1, PAR ^ 1);
+  if (blk + 2 < w.end) {
+    w.mask_next = mask_lane<D, NW>(w, blk + 2);
+    fill_k<D, NW>(w, blk + 2, PAR);
+  }
+  float corr;
+  const float m_exp = adopt_maximum<D, NW>(w, bm, corr);
+
+  const uint8_t *vs_ = smem + (2 + PAR) * TL::kBytes;
+  float bs[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  uint32_t pk[16];
+  scores<D, NW>(w, smem, PAR ^ 1, nv);
+  probabilities(sv, w.unit, m_exp, bs, pk);
+  accumulate<D, NW>(w, vs_, 0, pk);
+  probabilities(sv + 16, w.unit, m_exp, bs, pk + 8);
+  accumulate<D, NW>(w, vs_, 1, pk + 8);
+  bm = row_max(nv);
+  w.l_run = w.l_run * corr + ((bs[0] + bs[1]) + (bs[2] + bs[3]));
+  // The layout of the region.  LDS reads run two matrix instructions ahead of their use.
+  constexpr int kA = 56 / (2 * KS) + 1;  // VALU beside each score MFMA: the first half's p
+  constexpr int kB = 56 / (2 * DB) + 1;  // beside each MFMA of the first half's P V: the second half's p
+  constexpr int kC = 28 / (2 * DB) + 1;  // beside each MFMA of the second half's P V: the row maximum
   __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
 #pragma unroll
-  for (int i = 0; i < kMfma; i++) {
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);      // one MFMA
-    __builtin_amdgcn_sched_group_barrier(0x002, kValu, 0);  // VALU
-    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);      // LDS reads
+  for (int i = 0; i < 2 * KS; i++) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    __builtin_amdgcn_sched_group_barrier(0x002, kA, 0);
+    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+  }
+#pragma unroll
+  for (int i = 0; i < 2 * DB; i++) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    __builtin_amdgcn_sched_group_barrier(0x002, kB, 0);
+    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+  }
+#pragma unroll
+  for (int i = 0; i < 2 * DB; i++) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    __builtin_amdgcn_sched_group_barrier(0x002, kC, 0);
+    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+  }
+  __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the fills issued this step have landed
+  __syncthreads();
+}
+
+// The general step, for the blocks at the edges: any block, a next block or none, masks, any
+// scale.  Slots are picked at run time.  `sv` holds the masked S(blk) and `bm` its row maximum;
+// on exit they hold block blk+1's (when this wave has one).
+template <int D, int NW, bool CAUSAL>
+__device__ __forceinline__ void edge_step(Wave<D, NW> &w, const uint8_t *smem, int blk, int my_end, float (&sv)[32],
+                                          float &bm) {
+  using TL = Tile<D>;
+  const int par = blk & 1;
+  const bool more = blk + 1 < my_end;
+  const uint64_t kbits_next = uniform_bits<D, NW>(w, blk + 1, w.mask_next);
+  if (blk + 1 < w.end) fill_v<D, NW>(w, blk + 1, par ^ 1);
+  if (blk + 2 < w.end) {
+    w.mask_next = mask_lane<D, NW>(w, blk + 2);
+    fill_k<D, NW>(w, blk + 2, par);
+  }
+  float corr;
+  const float m_exp = adopt_maximum<D, NW>(w, bm, corr);
+
+  const uint8_t *vs_ = smem + (2 + par) * TL::kBytes;
+  float bs[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  uint32_t pk[16];
+  probabilities(sv, w.unit, m_exp, bs, pk);
+  probabilities(sv + 16, w.unit, m_exp, bs, pk + 8);
+  accumulate<D, NW>(w, vs_, 0, pk);
+  accumulate<D, NW>(w, vs_, 1, pk + 8);
+  w.l_run = w.l_run * corr + ((bs[0] + bs[1]) + (bs[2] + bs[3]));
+  if (more) {
+    scores<D, NW>(w, smem, par ^ 1, sv);
+    if (!w.positive) {
+#pragma unroll
+      for (int i = 0; i < 32; i++) sv[i] *= w.c_exp;
+    }
+    if (on_edge<D, NW, CAUSAL>(w, blk + 1, kbits_next)) mask_scores<D, NW, CAUSAL>(w, blk + 1, kbits_next, sv);
+    bm = row_max(sv);
   }
   __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the fills issued this step have landed
   __syncthreads();
@@ -457,8 +537,10 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
 #pragma unroll
   for (int db = 0; db < DB; db++) w.acc[db] = zero;
 
-  // ---- prologue: K(0), V(0), K(1) in flight, then the first block's scores.
-  w.mask_next = mask_lane<D, NW>(w, 0);
+  // ---- prologue: K(0), V(0), K(1) in flight, then the first block's scores, masked, and
+  // their row maximum.  Key-mask words are read two blocks ahead of their use.
+  const int word0 = mask_lane<D, NW>(w, 0);
+  w.mask_next = mask_lane<D, NW>(w, 1);
   if (end > 0) {
     fill_k<D, NW>(w, 0, 0);
     fill_v<D, NW>(w, 0, 0);
@@ -474,23 +556,35 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
   int my_end = end;
   if (CAUSAL) my_end = min(end, (w.wave_first_row + kWaveRows - 1) / kBkv + 1);
 
-  f32x16 a0 = zero, a1 = zero, b0 = zero, b1 = zero;
-  if (my_end > 0) scores<D, NW>(w, smem, 0, a0, a1);
+  float sv[32], nv[32];  // S of the current and of the next block, swapping roles each hot step
+  float bm = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < 32; i++) sv[i] = nv[i] = 0.0f;
+  if (my_end > 0) {
+    scores<D, NW>(w, smem, 0, sv);
+    if (!w.positive) {
+#pragma unroll
+      for (int i = 0; i < 32; i++) sv[i] *= w.c_exp;
+    }
+    const uint64_t kbits0 = uniform_bits<D, NW>(w, 0, word0);
+    if (on_edge<D, NW, CAUSAL>(w, 0, kbits0)) mask_scores<D, NW, CAUSAL>(w, 0, kbits0, sv);
+    bm = row_max(sv);
+  }
 
+  // Blocks [0, full) are crossed by no mask edge for this wave: they lie below the length and,
+  // for a causal wave, below its first row's diagonal.  A key mask puts every block on the
+  // edge path.  Step j is hot when block j+1 is such a block.
+  int full = 0;
+  if (w.positive && key_mask == nullptr) {
+    full = min(my_end, len / kBkv);
+    if (CAUSAL) full = min(full, (w.wave_first_row + 1) / kBkv);
+  }
   int blk = 0;
-  for (; blk + 2 < my_end; blk += 2) {
-    step<D, NW, CAUSAL, 0, true>(w, smem, blk, a0, a1, b0, b1);
-    step<D, NW, CAUSAL, 1, true>(w, smem, blk + 1, b0, b1, a0, a1);
+  for (; blk + 2 < full; blk += 2) {
+    hot_step<D, NW, 0>(w, smem, blk, sv, nv, bm);
+    hot_step<D, NW, 1>(w, smem, blk + 1, nv, sv, bm);
   }
-  // One or two blocks of this wave are left; S(blk) is in (a0, a1).
-  if (blk + 2 == my_end) {
-    step<D, NW, CAUSAL, 0, true>(w, smem, blk, a0, a1, b0, b1);
-    step<D, NW, CAUSAL, 1, false>(w, smem, blk + 1, b0, b1, a0, a1);
-    blk += 2;
-  } else if (blk + 1 == my_end) {
-    step<D, NW, CAUSAL, 0, false>(w, smem, blk, a0, a1, b0, b1);
-    blk += 1;
-  }
+  for (; blk < my_end; blk++) edge_step<D, NW, CAUSAL>(w, smem, blk, my_end, sv, bm);
   for (; blk < end; blk++) idle_step<D, NW>(w, blk);
 
   // ---- out = o / (l == 0 ? 1 : l), bounded store (L892-898, L974-980).

@@ -25,7 +25,7 @@ DEVICE_FLAGS = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang"
 # The attention kernel folds MFMA results with max(): without this every operand is first
 # quieted by a max(x, x) of its own (32 extra VALU ops a step).  Nothing in that kernel tests
 # for NaN, and infinities (the masks) stay honoured.
-EXTRA_FLAGS = {"attention_kernel.hip": ["-fno-honor-nans"]}
+EXTRA_FLAGS = {"attention_kernel.hip": ["-fno-honor-nans", "-mllvm", "-amdgpu-kernarg-preload-count=16"]}
 COMMON_FLAGS = ["-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-command-line-argument"]
 
 

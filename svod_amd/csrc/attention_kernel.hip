@@ -312,59 +312,127 @@ __device__ __forceinline__ float adopt_maximum(Wave<D, NW> &w, float bm, float &
   return m_new * w.unit;
 }
 
+// Keeps the computation of `x` where the source has it: instruction selection is otherwise free
+// to let arithmetic without side effects drift past the fences between slots.
+__device__ __forceinline__ void pin(float &x) { asm volatile("" : "+v"(x)); }
+
+// One unit of the exponentials: two scores to two probabilities (p = 2^(s*unit - m*unit)),
+// each added unrounded to a row-sum chain, the pair held as bf16 (L432-444).
+__device__ __forceinline__ uint32_t p_unit(float s_a, float s_b, float unit, float m_exp, float &sum_a, float &sum_b) {
+  const float pa = fast_exp2(__builtin_fmaf(s_a, unit, -m_exp));
+  const float pb = fast_exp2(__builtin_fmaf(s_b, unit, -m_exp));
+  sum_a += pa;
+  sum_b += pb;
+  return pack2(pa, pb);
+}
+
 // The hot step: block `blk` (parity PAR = blk & 1: V(blk) in V slot PAR, K(blk+1) in K slot
 // PAR^1) when block blk+1 is this wave's too, no mask edge crosses it and the scale is
 // positive.  `sv` holds S(blk) and `bm` its row maximum; S(blk+1) goes to `nv`, its maximum to
-// `bm`.  From the rescale to the barrier it is one scheduling region in which the matrix pipe
-// never waits for the VALU's whole job: S(blk+1) beside the first half's exponentials,
-// O += P V of the first half beside the second half's exponentials, O += P V of the second
-// half beside the row maximum of S(blk+1).
+// `bm`.
+//
+// The step is written as a sequence of slots, one matrix instruction each, fenced so that the
+// compiler keeps their order: the LDS fragment a matrix instruction reads was requested four
+// slots earlier, and each slot carries its share of the VALU work, so that the matrix pipe
+// never waits for the VALU's whole job.  2 KS slots compute S(blk+1) beside the exponentials
+// of keys 0..31; 2 DB slots add P V of keys 0..31 beside the exponentials of keys 32..63;
+// 2 DB slots add P V of keys 32..63 beside the row maximum of S(blk+1).
 template <int D, int NW, int PAR>
 __device__ __forceinline__ void hot_step(Wave<D, NW> &w, const uint8_t *smem, int blk, const float (&sv)[32],
                                          float (&nv)[32], float &bm) {
   using TL = Tile<D>;
   constexpr int KS = Wave<D, NW>::KS, DB = Wave<D, NW>::DB;
+  constexpr int NQK = 2 * KS;  // score slots
+  constexpr int NPV = 4 * DB;  // P V slots, half of them per 32 keys
+  const uint8_t *ks_ = smem + (PAR ^ 1) * TL::kBytes;
+  const uint8_t *vs_ = smem + (2 + PAR) * TL::kBytes;
+  // Score fragment f: key half kb = f & 1, k-step ks = f >> 1.
+  auto k_frag = [&](int f) -> u32x4 {
+    return *reinterpret_cast<const u32x4 *>(ks_ + w.k_read[f >> 1] + (f & 1) * 32 * TL::kRowBytes);
+  };
+  // P V fragment j: 16-key chunk c = j / DB (0..3), d-block db = j % DB.
+  auto v_frag = [&](int j) -> s16x8 {
+    const uint8_t *at = vs_ + w.v_read[j % DB] + 16 * (j / DB) * TL::kRowBytes;
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_PTR(s16x4))(at));
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_PTR(s16x4))(at + 8 * TL::kRowBytes));
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  };
+
+  u32x4 kf[4];
+#pragma unroll
+  for (int f = 0; f < 4; f++) kf[f] = k_frag(f);
   fill_v<D, NW>(w, blk + 1, PAR ^ 1);
-  if (blk + 2 < w.end) {
-    w.mask_next = mask_lane<D, NW>(w, blk + 2);
-    fill_k<D, NW>(w, blk + 2, PAR);
-  }
+  if (blk + 2 < w.end) fill_k<D, NW>(w, blk + 2, PAR);
+  w.mask_next = 0;  // hot steps run without a key mask only
   float corr;
   const float m_exp = adopt_maximum<D, NW>(w, bm, corr);
+  __builtin_amdgcn_sched_barrier(0);
 
-  const uint8_t *vs_ = smem + (2 + PAR) * TL::kBytes;
   float bs[4] = {0.0f, 0.0f, 0.0f, 0.0f};
   uint32_t pk[16];
-  scores<D, NW>(w, smem, PAR ^ 1, nv);
-  probabilities(sv, w.unit, m_exp, bs, pk);
-  accumulate<D, NW>(w, vs_, 0, pk);
-  probabilities(sv + 16, w.unit, m_exp, bs, pk + 8);
-  accumulate<D, NW>(w, vs_, 1, pk + 8);
-  bm = row_max(nv);
+  s16x8 vf[4];
+  const f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+  f32x16 s0 = zero, s1 = zero;
+  // ---- S(blk+1) beside the probabilities of keys 0..31 (8 units over NQK slots).
+#pragma unroll
+  for (int i = 0; i < NQK; i++) {
+    const bf16x8 a = __builtin_bit_cast(bf16x8, kf[i & 3]);
+    if (i & 1)
+      s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, w.qf[i >> 1], s1, 0, 0, 0);
+    else
+      s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, w.qf[i >> 1], s0, 0, 0, 0);
+    if (i + 4 < NQK)
+      kf[i & 3] = k_frag(i + 4);
+    else
+      vf[(i + 4 - NQK) & 3] = v_frag(i + 4 - NQK);
+#pragma unroll
+    for (int u = 8 * i / NQK; u < 8 * (i + 1) / NQK; u++)
+      pk[u] = p_unit(sv[2 * u], sv[2 * u + 1], w.unit, m_exp, bs[(2 * u) & 3], bs[(2 * u + 1) & 3]);
+    if (8 * i / NQK < 8 * (i + 1) / NQK) {
+#pragma unroll
+      for (int x = 0; x < 4; x++) pin(bs[x]);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+#pragma unroll
+  for (int i = 0; i < 16; i++) {
+    nv[i] = s0[i];
+    nv[16 + i] = s1[i];
+  }
+  // ---- O += P V of keys 0..31 beside the probabilities of keys 32..63, then O += P V of keys
+  // 32..63 beside the row maximum of S(blk+1).
+  float t[11];
+#pragma unroll
+  for (int j = 0; j < NPV; j++) {
+    const int c = j / DB;
+    const u32x4 pw = {pk[4 * c], pk[4 * c + 1], pk[4 * c + 2], pk[4 * c + 3]};
+    w.acc[j % DB] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vf[j & 3]),
+                                                           __builtin_bit_cast(bf16x8, pw), w.acc[j % DB], 0, 0, 0);
+    if (j + 4 < NPV) vf[j & 3] = v_frag(j + 4);
+    if (j < NPV / 2) {
+#pragma unroll
+      for (int u = 8 + 16 * j / NPV; u < 8 + 16 * (j + 1) / NPV; u++)
+        pk[u] = p_unit(sv[2 * u], sv[2 * u + 1], w.unit, m_exp, bs[(2 * u) & 3], bs[(2 * u + 1) & 3]);
+#pragma unroll
+      for (int x = 0; x < 4; x++) pin(bs[x]);
+    } else {
+      // The row maximum's first level, ten three-way folds and one two-way, over these slots.
+      const int jj = j - NPV / 2;
+#pragma unroll
+      for (int x = 11 * jj / (NPV / 2); x < 11 * (jj + 1) / (NPV / 2); x++)
+      {
+        t[x] = x < 10 ? max3(nv[3 * x], nv[3 * x + 1], nv[3 * x + 2]) : __builtin_fmaxf(nv[30], nv[31]);
+        pin(t[x]);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  {
+    const float u0 = max3(t[0], t[1], t[2]), u1 = max3(t[3], t[4], t[5]), u2 = max3(t[6], t[7], t[8]);
+    const Pair p = both_halves(max3(max3(u0, u1, u2), t[9], t[10]));
+    bm = __builtin_fmaxf(p.a, p.b);
+  }
   w.l_run = w.l_run * corr + ((bs[0] + bs[1]) + (bs[2] + bs[3]));
-  // The layout of the region.  LDS reads run two matrix instructions ahead of their use.
-  constexpr int kA = 56 / (2 * KS) + 1;  // VALU beside each score MFMA: the first half's p
-  constexpr int kB = 56 / (2 * DB) + 1;  // beside each MFMA of the first half's P V: the second half's p
-  constexpr int kC = 28 / (2 * DB) + 1;  // beside each MFMA of the second half's P V: the row maximum
-  __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
-#pragma unroll
-  for (int i = 0; i < 2 * KS; i++) {
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-    __builtin_amdgcn_sched_group_barrier(0x002, kA, 0);
-    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-  }
-#pragma unroll
-  for (int i = 0; i < 2 * DB; i++) {
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-    __builtin_amdgcn_sched_group_barrier(0x002, kB, 0);
-    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-  }
-#pragma unroll
-  for (int i = 0; i < 2 * DB; i++) {
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-    __builtin_amdgcn_sched_group_barrier(0x002, kC, 0);
-    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-  }
   __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the fills issued this step have landed
   __syncthreads();
 }
@@ -418,15 +486,39 @@ __device__ __forceinline__ void idle_step(Wave<D, NW> &w, int blk) {
   __syncthreads();
 }
 
+// n / d for n < 2^32 with rcp = floor(2^32 / d) (2^32 - 1 for d = 1) from the host: the
+// estimate is the quotient or one less.
+__device__ __forceinline__ uint32_t div_by(uint32_t n, uint32_t d, uint32_t rcp) {
+  const uint32_t q = __umulhi(n, rcp);
+  return n - q * d >= d ? q + 1 : q;
+}
+
+// Launch geometry the host works out once: sizes and their reciprocals for div_by.
+struct Geometry {
+  uint32_t unit_size, unit_rcp;  // workgroups of a (batch, KV head): group * nqt
+  uint32_t nqt, nqt_rcp;         // query tiles
+  uint32_t kv_heads, kvh_rcp;
+  uint32_t group;                // heads / kv_heads
+  uint32_t units;                // kv_heads * batch
+};
+
 template <int D, int NW, bool CAUSAL>
-__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) void flash_fwd_kernel(
-    const uint16_t *__restrict__ q, const uint16_t *__restrict__ k, const uint16_t *__restrict__ v,
-    uint16_t *__restrict__ o, const void *__restrict__ key_lens, const void *__restrict__ key_mask, int32_t lens_i64,
-    int32_t mask_bytes, int32_t t, int32_t tk, int32_t heads, int32_t kv_heads, int32_t nqt, int32_t nbatch,
-    float scale) {
+__global__ __launch_bounds__(NW * 64, D == 64 ? 3 : 2) void flash_fwd_kernel(
+    uint32_t unit_size, uint32_t unit_rcp, uint32_t nqt_u, uint32_t nqt_rcp, uint32_t kvh_u, uint32_t kvh_rcp,
+    uint32_t units, uint32_t heads_group, const void *__restrict__ key_lens, const uint16_t *__restrict__ q, int32_t t,
+    uint32_t tk_lens64, const uint16_t *__restrict__ k, const uint16_t *__restrict__ v,
+    uint16_t *__restrict__ o, const void *__restrict__ key_mask, int32_t mask_bytes, float scale) {
   // The body is device code only: the host pass needs the kernel's handle, not its
   // instructions (and drops the whole instantiation over the LDS-fill instructions).
 #if defined(__HIP_DEVICE_COMPILE__)
+  // The first 14 dwords of the arguments (up to tk_lens64) arrive in registers with the wave
+  // (kernarg preload, scalars and pointers only): they are what the workgroup's coordinates,
+  // its length and the Q loads need, so none of those waits for an argument load.  Two of them
+  // are packed to fit: heads | group << 16, and tk | (key_lens is 64-bit) << 31.
+  const Geometry geo = {unit_size, unit_rcp, nqt_u, nqt_rcp, kvh_u, kvh_rcp, heads_group >> 16, units};
+  const int heads = (int)(heads_group & 0xffffu);
+  const int tk = (int)(tk_lens64 & 0x7fffffffu);
+  const bool lens_i64 = (tk_lens64 >> 31) != 0;
   using TL = Tile<D>;
   using W = Wave<D, NW>;
   constexpr int BQ = NW * kWaveRows;
@@ -435,6 +527,28 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
 
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
 
+  // A unit of work is one (batch, KV head): the query tiles of the heads that share its K and
+  // V.  Workgroups are dealt to the 8 XCDs round-robin, each XCD with its own L2, so the units
+  // are dealt to the XCDs round-robin too and a unit's workgroups all land on one XCD: they
+  // meet in one L2 instead of being spread over all eight.  (The reference's grid is query
+  // tile fastest, then head, then batch, attention.rs:512,523; the order within a unit is that.)
+  const uint32_t wg = __builtin_amdgcn_workgroup_id_x();
+  const uint32_t local = wg / kXcds;
+  const uint32_t round = div_by(local, geo.unit_size, geo.unit_rcp);
+  const uint32_t unit = round * kXcds + wg % kXcds;
+  if (unit >= geo.units) return;
+  const uint32_t within = local - round * geo.unit_size;
+  const uint32_t head_in_group = div_by(within, geo.nqt, geo.nqt_rcp);
+  const int order = (int)(within - head_in_group * geo.nqt);
+  const int b = (int)div_by(unit, geo.kv_heads, geo.kvh_rcp);
+  const int kvh = (int)(unit - (uint32_t)b * geo.kv_heads);  // L548: query head h reads KV head h / (heads / kv_heads)
+  const int h = kvh * (int)geo.group + (int)head_in_group;
+  const int kv_heads = (int)geo.kv_heads;
+  const int nqt = (int)geo.nqt;
+  // Where later queries see more keys the last query blocks run first (L524-528).
+  const int qt = CAUSAL ? (nqt - 1 - order) : order;
+  const int q_off = qt * BQ;
+
   W w;
   const int tid = __builtin_amdgcn_workitem_id_x();
   w.lane = tid & 63;
@@ -442,52 +556,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
   w.g = w.lane >> 5;           // half-wave: the k-chunk of MFMA operands
   const int ln = w.lane & 31;  // the query column this lane owns
 
-  // A unit of work is one (batch, KV head): the query tiles of the heads that share its K and
-  // V.  Workgroups are dealt to the 8 XCDs round-robin, each XCD with its own L2, so the units
-  // are dealt to the XCDs round-robin too and a unit's workgroups all land on one XCD: they
-  // meet in one L2 instead of being spread over all eight.  (The reference's grid is query
-  // tile fastest, then head, then batch, attention.rs:512,523; the order within a unit is that.)
-  const int group = heads / kv_heads;
-  const int unit_size = group * nqt;
-  const int units = kv_heads * nbatch;
-  const int wg = __builtin_amdgcn_workgroup_id_x();
-  const int local = wg / kXcds;
-  const int unit = (local / unit_size) * kXcds + wg % kXcds;
-  if (unit >= units) return;
-  const int within = local % unit_size;
-  const int order = within % nqt;
-  const int kvh = unit % kv_heads;  // L548: query head h reads KV head h / (heads / kv_heads)
-  const int h = kvh * group + within / nqt;
-  const int b = unit / kv_heads;
-  // Where later queries see more keys the last query blocks run first (L524-528).
-  const int qt = CAUSAL ? (nqt - 1 - order) : order;
-  const int q_off = qt * BQ;
-
-  // L533-536: len = min(key_lens[b], tk).
-  int len = tk;
-  if (key_lens != nullptr) {
-    long long n = lens_i64 ? ((const long long *)key_lens)[b] : (long long)((const int *)key_lens)[b];
-    n = n < 0 ? 0 : n;
-    len = n < (long long)tk ? (int)n : tk;
-  }
-  // L596-608: key blocks some query of the tile sees.
-  int end = (tk + kBkv - 1) / kBkv;
-  if (CAUSAL) end = min(end, (q_off + BQ + kBkv - 1) / kBkv);
-  if (key_lens != nullptr) end = min(end, (len + kBkv - 1) / kBkv);
-  w.end = end;
-  w.len = len;
-  w.tk = tk;
-  w.key_mask = key_mask;
-  w.mask_row = (int64_t)b * tk;
-  w.mask_bytes = mask_bytes;
-
   const int64_t q_row_stride = (int64_t)heads * D;
-  w.kv_row_bytes = kv_heads * D * 2;
-  w.k_base = (const uint8_t *)(k + ((int64_t)b * tk * kv_heads + kvh) * D);
-  w.v_base = (const uint8_t *)(v + ((int64_t)b * tk * kv_heads + kvh) * D);
-  w.kv_bytes = len > 0 ? (int64_t)(len - 1) * w.kv_row_bytes + D * 2 : 0;
-  w.lds0 = (int)(uintptr_t)(LDS_PTR(uint8_t))(smem);
-
   // ---- Q fragments: B operand of the score product, resident for the block.
   w.wave_first_row = q_off + w.wave * kWaveRows;
   w.my_row = w.wave_first_row + ln;
@@ -501,6 +570,31 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
     }
   }
 
+  // L533-536: len = min(key_lens[b], tk).
+  int len = tk;
+  if (key_lens != nullptr) {
+    long long n = lens_i64 ? ((const long long *)key_lens)[b] : (long long)((const int *)key_lens)[b];
+    n = n < 0 ? 0 : n;
+    len = n < (long long)tk ? (int)n : tk;
+  }
+
+  // L596-608: key blocks some query of the tile sees.
+  int end = (tk + kBkv - 1) / kBkv;
+  if (CAUSAL) end = min(end, (q_off + BQ + kBkv - 1) / kBkv);
+  if (key_lens != nullptr) end = min(end, (len + kBkv - 1) / kBkv);
+  w.end = end;
+  w.len = len;
+  w.tk = tk;
+  w.key_mask = key_mask;
+  w.mask_row = (int64_t)b * tk;
+  w.mask_bytes = mask_bytes;
+
+  w.kv_row_bytes = kv_heads * D * 2;
+  w.k_base = (const uint8_t *)(k + ((int64_t)b * tk * kv_heads + kvh) * D);
+  w.v_base = (const uint8_t *)(v + ((int64_t)b * tk * kv_heads + kvh) * D);
+  w.kv_bytes = len > 0 ? (int64_t)(len - 1) * w.kv_row_bytes + D * 2 : 0;
+  w.lds0 = (int)(uintptr_t)(LDS_PTR(uint8_t))(smem);
+
   // ---- this wave's share of a tile fill: CH wave-wide 1 KiB instructions.  Fill j lands on
   // rows [j*rows_per, ...): lane i at physical chunk i % kCpr of row i / kCpr.
   constexpr int kRowsPer = 64 / TL::kCpr;
@@ -512,6 +606,16 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
     w.k_src[i] = row * w.kv_row_bytes + ((pc ^ TL::swz_k(row)) << 4);
     w.v_src[i] = row * w.kv_row_bytes + ((pc ^ (TL::swz_v(row) << 2)) << 4);
   }
+  // ---- K(0), V(0), K(1) go first: everything below runs in the shadow of their flight.
+  if (end > 0) {
+    fill_k<D, NW>(w, 0, 0);
+    fill_v<D, NW>(w, 0, 0);
+  }
+  if (end > 1) fill_k<D, NW>(w, 1, 1);
+  // Key-mask words are read two blocks ahead of their use.
+  const int word0 = mask_lane<D, NW>(w, 0);
+  w.mask_next = mask_lane<D, NW>(w, 1);
+
   // ---- per-lane LDS offsets of the operand reads.
   // K fragment (kb, ks): row 32kb + ln, logical chunk 2ks + g.
 #pragma unroll
@@ -537,20 +641,12 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) vo
 #pragma unroll
   for (int db = 0; db < DB; db++) w.acc[db] = zero;
 
-  // ---- prologue: K(0), V(0), K(1) in flight, then the first block's scores, masked, and
-  // their row maximum.  Key-mask words are read two blocks ahead of their use.
-  const int word0 = mask_lane<D, NW>(w, 0);
-  w.mask_next = mask_lane<D, NW>(w, 1);
-  if (end > 0) {
-    fill_k<D, NW>(w, 0, 0);
-    fill_v<D, NW>(w, 0, 0);
-  }
-  if (end > 1) fill_k<D, NW>(w, 1, 1);
   // A wait the compiler knows of: it covers the Q loads too, so that no wait of its own for
   // them lands inside the loop, where it would also wait out the fills in flight.
   __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
   __syncthreads();
 
+  // ---- the first block's scores, masked, and their row maximum.
   // A causal wave past its last visible key has nothing to add from a block: it only keeps
   // filling and meeting the barriers.  Blocks [0, my_end) are this wave's.
   int my_end = end;
@@ -632,9 +728,23 @@ hipError_t launch(const AttnArgs &a, hipStream_t stream) {
   const int64_t units = (int64_t)a.kv_heads * a.batch;
   const int64_t grid = (units + kXcds - 1) / kXcds * kXcds * unit_size;
   if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
-  hipLaunchKernelGGL(kernel, dim3((uint32_t)grid), dim3(NW * 64), smem, stream, (const uint16_t *)a.q,
-                     (const uint16_t *)a.k, (const uint16_t *)a.v, (uint16_t *)a.o, a.key_lens, a.key_mask, a.lens_i64,
-                     a.mask_bytes, a.t, a.tk, a.heads, a.kv_heads, nqt, a.batch, a.scale);
+  auto rcp = [](uint32_t d) { return d == 1 ? 0xffffffffu : (uint32_t)((1ull << 32) / d); };
+  Geometry geo;
+  geo.unit_size = (uint32_t)unit_size;
+  geo.unit_rcp = rcp(geo.unit_size);
+  geo.nqt = (uint32_t)nqt;
+  geo.nqt_rcp = rcp(geo.nqt);
+  geo.kv_heads = (uint32_t)a.kv_heads;
+  geo.kvh_rcp = rcp(geo.kv_heads);
+  geo.group = (uint32_t)(a.heads / a.kv_heads);
+  geo.units = (uint32_t)units;
+  if (a.heads > 0xffff) return hipErrorInvalidConfiguration;  // heads and group share an argument
+  const uint32_t heads_group = (uint32_t)a.heads | geo.group << 16;
+  const uint32_t tk_lens64 = (uint32_t)a.tk | (a.lens_i64 ? 0x80000000u : 0u);
+  hipLaunchKernelGGL(kernel, dim3((uint32_t)grid), dim3(NW * 64), smem, stream, geo.unit_size, geo.unit_rcp, geo.nqt,
+                     geo.nqt_rcp, geo.kv_heads, geo.kvh_rcp, geo.units, heads_group, a.key_lens,
+                     (const uint16_t *)a.q, a.t, tk_lens64, (const uint16_t *)a.k,
+                     (const uint16_t *)a.v, (uint16_t *)a.o, a.key_mask, a.mask_bytes, a.scale);
   return hipGetLastError();
 }
 

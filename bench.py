@@ -25,6 +25,11 @@ import time
 
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of
+# this file, each scaled by what the counter reads for a 256 MiB device copy (x2.000 and x1.000);
+# the summaries are under profiles/.  Counters cannot be read from inside a timed run.
+HBM_TRAFFIC_BYTES = {"bge_m3": 110.29e6, "qwen3_attention": 176.86e6, "qwen3_prologue": 271.07e6,
+                     "whisper": 245.93e6, "long": 125.28e6}
 
 
 def parse():
@@ -33,8 +38,14 @@ def parse():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="bge_m3",
-                    choices=["bge_m3", "bge_m3_bool", "qwen3_attention", "qwen3_prologue", "whisper", "long"])
+                    choices=["bge_m3", "bge_m3_bool", "qwen3_attention", "qwen3_prologue", "whisper", "long",
+                             "hbm_copy"],
+                    help="hbm_copy is a plain 256 MiB device copy: the known-size kernel the HBM counters "
+                         "(FETCH_SIZE, WRITE_SIZE) are calibrated on")
     ap.add_argument("--layers", type=int, default=24, help="calls per step for the bge_m3 workloads")
+    ap.add_argument("--calls", type=int, default=16,
+                    help="calls per step for the other workloads, rotating over 4 copies of the operands so that "
+                         "none is served from the Infinity Cache")
     ap.add_argument("--no-graph", action="store_true", help="enqueue eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="rough budget of the CPU baseline sample")
@@ -80,11 +91,22 @@ def main():
             args.layers, " (KeyMask::Bool)" if args.workload == "bge_m3_bool" else " (KeyMask::Lens)")
         cpu_sample = ("attention", w0)
         kernel_name = "flash_fwd_kernel<64>"
+    elif args.workload == "hbm_copy":
+        srcs = [torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255) for _ in range(2)]
+        dsts = [torch.empty_like(x) for x in srcs]
+        for i in range(args.calls):
+            calls.append(lambda i=i: dsts[i % 2].copy_(srcs[i % 2]))
+        bytes_min = 2 * srcs[0].numel()
+        workload = "plain device copy of 256 MiB (torch copy_), counter calibration"
+        kernel_name, bound = "torch elementwise copy", "hbm"
     elif args.workload == "qwen3_prologue":
         p = W.config3_prologue(device=dev)
-        outs = tuple(torch.empty((8, 2048, n, 128), dtype=torch.bfloat16, device=dev) for n in (16, 8, 8))
         opts = Qkv(p.heads, p.kv_heads, p.head_dim, p.q_w, p.k_w, p.eps, (p.cos, p.sin))
-        calls.append(lambda: svod_amd.heads(p.qkv, opts, out=outs))
+        ins = [p.qkv] + [p.qkv.clone() for _ in range(3)]
+        outs = [tuple(torch.empty((8, 2048, n, 128), dtype=torch.bfloat16, device=dev) for n in (16, 8, 8))
+                for _ in range(4)]
+        for i in range(args.calls):
+            calls.append(lambda i=i: svod_amd.heads(ins[i % 4], opts, out=outs[i % 4]))
         bytes_min = p.min_bytes()
         workload = "Qwen3-Embedding prologue bf16 qkv[8,2048,4096] -> q,k,v (RMSNorm eps 1e-6 + RoPE theta 1e6)"
         cpu_sample = ("heads", p)
@@ -105,8 +127,11 @@ def main():
             workload = "long-context pair attention bf16 B2 H16 D64 S8192, lens {8192, 5000}"
             kernel_name = "flash_fwd_kernel<64>"
         keys = KeyMask.lens(w.key_lens) if w.key_lens is not None else KeyMask.none()
-        out = torch.empty_like(w.q)
-        calls.append(lambda: svod_amd.attention(w.q, w.k, w.v, Attn(causal=w.causal, keys=keys, scale=w.scale), out=out))
+        ins = [(w.q, w.k, w.v)] + [(w.q.clone(), w.k.clone(), w.v.clone()) for _ in range(3)]
+        outs = [torch.empty_like(w.q) for _ in range(4)]
+        opts = Attn(causal=w.causal, keys=keys, scale=w.scale)
+        for i in range(args.calls):
+            calls.append(lambda i=i: svod_amd.attention(*ins[i % 4], opts, out=outs[i % 4]))
         flops_vis, flops_nom, bytes_min = w.visible_flops(), w.nominal_flops(), w.min_bytes()
         cpu_sample = ("attention", w)
 
@@ -169,7 +194,8 @@ def main():
         value = flops_vis * len(calls) / (ms_per_step * 1e-3) / 1e12
         achieved = flops_vis / (kernel_us * 1e-6) / 1e12
         roof = {"bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None, "kernel": kernel_name,
+                "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": HBM_TRAFFIC_BYTES.get(args.workload),
+                "traffic_unit": "bytes per launch", "kernel": kernel_name,
                 "kernel_us": round(kernel_us, 3), "flops_per_launch_visible": flops_vis,
                 "flops_per_launch_nominal": flops_nom,
                 "nominal_tflops": round(flops_nom / (kernel_us * 1e-6) / 1e12, 2),
@@ -179,7 +205,8 @@ def main():
         value = bytes_min * len(calls) / (ms_per_step * 1e-3) / 1e9
         achieved = bytes_min / (kernel_us * 1e-6) / 1e9
         roof = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None, "kernel": kernel_name,
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": HBM_TRAFFIC_BYTES.get(args.workload),
+                "traffic_unit": "bytes per launch", "kernel": kernel_name,
                 "kernel_us": round(kernel_us, 3), "bytes_per_launch": bytes_min}
         metric, unit = "attention prologue GB/s on 1 MI355X", "GB/s"
 

@@ -46,116 +46,165 @@ __device__ __forceinline__ void widen(const u32x4 &w, float (&x)[8]) {
   }
 }
 
-template <int D>
+// Rows and slots come from flat item numbers by division.  The 32-bit form divides with a
+// reciprocal from the host (rcp = floor(2^32 / d), 2^32 - 1 for d = 1: the estimate is the
+// quotient or one less); the 64-bit form is for tensors past 2^32 lanes.
+struct Div32 {
+  typedef uint32_t index;
+  uint32_t d, rcp;
+  __device__ __forceinline__ uint32_t quot(uint32_t n) const {
+    const uint32_t q = __umulhi(n, rcp);
+    return n - q * d >= d ? q + 1 : q;
+  }
+};
+struct Div64 {
+  typedef int64_t index;
+  int64_t d;
+  uint32_t unused;
+  __device__ __forceinline__ int64_t quot(int64_t n) const { return n / d; }
+};
+
+// A block owns kItems * kThreads consecutive lanes of the flat (row, slot, part) space, slots
+// fastest: thread i takes lanes i, i + kThreads, ...  All loads of a thread are issued before
+// any arithmetic.  One item per thread measured fastest on an MI355X (2 and 4 were 5 % and
+// 20 % slower: the many small waves keep more of HBM's channels busy than fewer long ones),
+// and every byte is touched once, so loads and stores are marked non-temporal.
+constexpr int kItems = 1;
+
+template <int D, typename Div>
 __global__ __launch_bounds__(kThreads) void heads_kernel(const uint16_t *__restrict__ qkv,
                                                          const uint16_t *__restrict__ q_w,
                                                          const uint16_t *__restrict__ k_w,
                                                          const uint16_t *__restrict__ cos_t,
                                                          const uint16_t *__restrict__ sin_t, uint16_t *__restrict__ q,
                                                          uint16_t *__restrict__ k, uint16_t *__restrict__ v,
-                                                         int64_t items, int32_t t, int32_t heads, int32_t kv_heads,
-                                                         float eps, int32_t rope) {
+                                                         int64_t items, Div by_slots, Div by_t, int32_t heads,
+                                                         int32_t kv_heads, float eps, int32_t rope) {
 #pragma clang fp contract(off)
+  typedef typename Div::index Index;
   constexpr int kHalf = D / 2;
   constexpr int kLanes = D / 16;  // lanes sharing one head slot
-  const int32_t slots = heads + 2 * kv_heads;
-  const int64_t gid = (int64_t)__builtin_amdgcn_workgroup_id_x() * kThreads + __builtin_amdgcn_workitem_id_x();
-  const int64_t item = gid / kLanes;  // (row, slot), slots fastest
-  const int32_t part = (int32_t)(gid % kLanes);
-  // Lanes of a slot always run together (kLanes divides 64 and the item count
-  // is rounded up per wave below), so the exchanges see their partners.
-  const bool live = item < items;
-  const int64_t row = live ? item / slots : 0;
-  const int32_t slot = live ? (int32_t)(item % slots) : 0;
+  static_assert(kThreads % kLanes == 0, "a thread keeps its part of the slot across its items");
+  const Index slots = (Index)by_slots.d;
+  const Index first = (Index)__builtin_amdgcn_workgroup_id_x() * (kThreads * kItems) + __builtin_amdgcn_workitem_id_x();
+  const int32_t part = (int32_t)(__builtin_amdgcn_workitem_id_x() % kLanes);
 
-  const uint16_t *src = qkv + (row * slots + slot) * D + part * 8;
-  u32x4 w1 = {0, 0, 0, 0}, w2 = {0, 0, 0, 0};
-  if (live) {
-    w1 = *reinterpret_cast<const u32x4 *>(src);
-    w2 = *reinterpret_cast<const u32x4 *>(src + kHalf);
-  }
-
-  const bool is_q = slot < heads;
-  const bool is_k = !is_q && slot < heads + kv_heads;
-  const uint16_t *weight = is_q ? q_w : (is_k ? k_w : nullptr);
-  const bool rotate = rope != 0 && (is_q || is_k);
-
-  uint16_t *dst;
-  if (is_q)
-    dst = q + (row * heads + slot) * D;
-  else if (is_k)
-    dst = k + (row * kv_heads + (slot - heads)) * D;
-  else
-    dst = v + (row * kv_heads + (slot - heads - kv_heads)) * D;
-  dst += part * 8;
-
-  // Slots are uniform across the lanes of a slot, not across the wave: the
-  // exchanges below run for every lane, the arithmetic is selected per lane.
-  float y1[8], y2[8];
-  widen(w1, y1);
-  widen(w2, y2);
-  float sum = 0.0f;
+  // Lanes of a slot always run together (kLanes divides 64), so the exchanges see their partners.
+  bool live[kItems];
+  Index row[kItems];
+  int32_t slot[kItems];
+  u32x4 w1[kItems], w2[kItems];
 #pragma unroll
-  for (int i = 0; i < 8; i++) sum += y1[i] * y1[i] + y2[i] * y2[i];
-#pragma unroll
-  for (int m = 1; m < kLanes; m <<= 1) sum += __shfl_xor(sum, m, 64);
-
-  if (weight != nullptr) {
-    const float inv = __builtin_amdgcn_rsqf(sum * (1.0f / (float)D) + eps);
-    const u32x4 g1 = *reinterpret_cast<const u32x4 *>(weight + part * 8);
-    const u32x4 g2 = *reinterpret_cast<const u32x4 *>(weight + kHalf + part * 8);
-    float a1[8], a2[8];
-    widen(g1, a1);
-    widen(g2, a2);
-#pragma unroll
-    for (int i = 0; i < 8; i++) {
-      y1[i] = (y1[i] * inv) * a1[i];
-      y2[i] = (y2[i] * inv) * a2[i];
+  for (int u = 0; u < kItems; u++) {
+    const Index item = (first + (Index)u * kThreads) / kLanes;  // (row, slot), slots fastest
+    live[u] = (int64_t)item < items;
+    row[u] = live[u] ? by_slots.quot(item) : 0;
+    slot[u] = live[u] ? (int32_t)(item - row[u] * slots) : 0;
+    const uint16_t *src = qkv + ((int64_t)row[u] * slots + slot[u]) * D + part * 8;
+    w1[u] = w2[u] = u32x4{0, 0, 0, 0};
+    if (live[u]) {
+      w1[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src));
+      w2[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + kHalf));
     }
   }
-  if (rotate) {
-    const int64_t trow = (rope == 2) ? row : row % t;
-    const u32x4 cw = *reinterpret_cast<const u32x4 *>(cos_t + trow * kHalf + part * 8);
-    const u32x4 sw = *reinterpret_cast<const u32x4 *>(sin_t + trow * kHalf + part * 8);
-    float c[8], s[8];
-    widen(cw, c);
-    widen(sw, s);
+
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-      const float r1 = y1[i] * c[i] - y2[i] * s[i];
-      const float r2 = y1[i] * s[i] + y2[i] * c[i];
-      y1[i] = r1;
-      y2[i] = r2;
-    }
-  }
-  if (!live) return;
-  u32x4 o1, o2;
-  if (weight != nullptr || rotate) {
+  for (int u = 0; u < kItems; u++) {
+    const bool is_q = slot[u] < heads;
+    const bool is_k = !is_q && slot[u] < heads + kv_heads;
+    const uint16_t *weight = is_q ? q_w : (is_k ? k_w : nullptr);
+    const bool rotate = rope != 0 && (is_q || is_k);
+
+    uint16_t *dst;
+    if (is_q)
+      dst = q + ((int64_t)row[u] * heads + slot[u]) * D;
+    else if (is_k)
+      dst = k + ((int64_t)row[u] * kv_heads + (slot[u] - heads)) * D;
+    else
+      dst = v + ((int64_t)row[u] * kv_heads + (slot[u] - heads - kv_heads)) * D;
+    dst += part * 8;
+
+    // Slots are uniform across the lanes of a slot, not across the wave: the
+    // exchanges below run for every lane, the arithmetic is selected per lane.
+    float y1[8], y2[8];
+    widen(w1[u], y1);
+    widen(w2[u], y2);
+    float sum = 0.0f;
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-      o1[i] = pack_bf16(y1[2 * i], y1[2 * i + 1]);
-      o2[i] = pack_bf16(y2[2 * i], y2[2 * i + 1]);
+    for (int i = 0; i < 8; i++) sum += y1[i] * y1[i] + y2[i] * y2[i];
+#pragma unroll
+    for (int m = 1; m < kLanes; m <<= 1) sum += __shfl_xor(sum, m, 64);
+
+    if (weight != nullptr) {
+      const float inv = __builtin_amdgcn_rsqf(sum * (1.0f / (float)D) + eps);
+      const u32x4 g1 = *reinterpret_cast<const u32x4 *>(weight + part * 8);
+      const u32x4 g2 = *reinterpret_cast<const u32x4 *>(weight + kHalf + part * 8);
+      float a1[8], a2[8];
+      widen(g1, a1);
+      widen(g2, a2);
+#pragma unroll
+      for (int i = 0; i < 8; i++) {
+        y1[i] = (y1[i] * inv) * a1[i];
+        y2[i] = (y2[i] * inv) * a2[i];
+      }
     }
-  } else {
-    o1 = w1;  // untouched slots (v, or q/k with neither norm nor rope) keep their bits
-    o2 = w2;
+    if (rotate) {
+      const Index trow = (rope == 2) ? row[u] : row[u] - by_t.quot(row[u]) * (Index)by_t.d;
+      const u32x4 cw = *reinterpret_cast<const u32x4 *>(cos_t + (int64_t)trow * kHalf + part * 8);
+      const u32x4 sw = *reinterpret_cast<const u32x4 *>(sin_t + (int64_t)trow * kHalf + part * 8);
+      float c[8], s[8];
+      widen(cw, c);
+      widen(sw, s);
+#pragma unroll
+      for (int i = 0; i < 8; i++) {
+        const float r1 = y1[i] * c[i] - y2[i] * s[i];
+        const float r2 = y1[i] * s[i] + y2[i] * c[i];
+        y1[i] = r1;
+        y2[i] = r2;
+      }
+    }
+    if (!live[u]) continue;
+    u32x4 o1, o2;
+    if (weight != nullptr || rotate) {
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        o1[i] = pack_bf16(y1[2 * i], y1[2 * i + 1]);
+        o2[i] = pack_bf16(y2[2 * i], y2[2 * i + 1]);
+      }
+    } else {
+      o1 = w1[u];  // untouched slots (v, or q/k with neither norm nor rope) keep their bits
+      o2 = w2[u];
+    }
+    __builtin_nontemporal_store(o1, reinterpret_cast<u32x4 *>(dst));
+    __builtin_nontemporal_store(o2, reinterpret_cast<u32x4 *>(dst + kHalf));
   }
-  *reinterpret_cast<u32x4 *>(dst) = o1;
-  *reinterpret_cast<u32x4 *>(dst + kHalf) = o2;
 }
 
 template <int D>
 hipError_t launch(const HeadsArgs &a, hipStream_t stream) {
   constexpr int kLanes = D / 16;
-  const int64_t items = a.rows * (a.heads + 2 * a.kv_heads);
+  const int64_t slots = a.heads + 2 * a.kv_heads;
+  const int64_t items = a.rows * slots;
   if (items == 0) return hipSuccess;
   const int64_t threads = items * kLanes;
-  const int64_t blocks = (threads + kThreads - 1) / kThreads;
+  const int64_t per_block = (int64_t)kThreads * kItems;
+  const int64_t blocks = (threads + per_block - 1) / per_block;
   if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;
-  hipLaunchKernelGGL(heads_kernel<D>, dim3((uint32_t)blocks), dim3(kThreads), 0, stream,
-                     (const uint16_t *)a.qkv, (const uint16_t *)a.q_w, (const uint16_t *)a.k_w,
-                     (const uint16_t *)a.cos, (const uint16_t *)a.sin, (uint16_t *)a.q, (uint16_t *)a.k,
-                     (uint16_t *)a.v, items, a.t, a.heads, a.kv_heads, a.eps, a.rope);
+  const int64_t t = a.t > 0 ? a.t : 1;
+  if (blocks * per_block < 0xffffffffLL) {
+    auto rcp = [](uint32_t d) { return d == 1 ? 0xffffffffu : (uint32_t)((1ull << 32) / d); };
+    const Div32 by_slots = {(uint32_t)slots, rcp((uint32_t)slots)}, by_t = {(uint32_t)t, rcp((uint32_t)t)};
+    hipLaunchKernelGGL((heads_kernel<D, Div32>), dim3((uint32_t)blocks), dim3(kThreads), 0, stream,
+                       (const uint16_t *)a.qkv, (const uint16_t *)a.q_w, (const uint16_t *)a.k_w,
+                       (const uint16_t *)a.cos, (const uint16_t *)a.sin, (uint16_t *)a.q, (uint16_t *)a.k,
+                       (uint16_t *)a.v, items, by_slots, by_t, a.heads, a.kv_heads, a.eps, a.rope);
+  } else {
+    const Div64 by_slots = {slots, 0}, by_t = {t, 0};
+    hipLaunchKernelGGL((heads_kernel<D, Div64>), dim3((uint32_t)blocks), dim3(kThreads), 0, stream,
+                       (const uint16_t *)a.qkv, (const uint16_t *)a.q_w, (const uint16_t *)a.k_w,
+                       (const uint16_t *)a.cos, (const uint16_t *)a.sin, (uint16_t *)a.q, (uint16_t *)a.k,
+                       (uint16_t *)a.v, items, by_slots, by_t, a.heads, a.kv_heads, a.eps, a.rope);
+  }
   return hipGetLastError();
 }
 

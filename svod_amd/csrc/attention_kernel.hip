@@ -666,6 +666,8 @@ __global__ __launch_bounds__(NW * 64, D == 64 ? 3 : 2) void flash_fwd_kernel(
     if (on_edge<D, NW, CAUSAL>(w, 0, kbits0)) mask_scores<D, NW, CAUSAL>(w, 0, kbits0, sv);
     bm = row_max(sv);
   }
+  // Step 0 refills the K slot those scores were read from: every wave has read it first.
+  __syncthreads();
 
   // Blocks [0, full) are crossed by no mask edge for this wave: they lie below the length and,
   // for a causal wave, below its first row's diagonal.  A key mask puts every block on the

@@ -23,7 +23,7 @@
 extern "C" {
 #endif
 
-#define SVODK_ABI_VERSION 1
+#define SVODK_ABI_VERSION 2
 
 /* Element types of a tensor descriptor. */
 typedef enum svodk_dtype {
@@ -74,8 +74,17 @@ typedef enum svodk_key_mask {
 /*
  * Attn of tk/src/ops/attention.rs:60-86.  Zero-initialise, then set fields.
  * Options this library has no kernel for (window, chunk, seg_start, cache,
- * bias, splits > 1) are still validated as the reference validates them and
- * then answered with SVODK_GRAPH_CONFIG.
+ * bias) are still validated as the reference validates them and then answered
+ * with SVODK_GRAPH_CONFIG.
+ *
+ * `splits` > 1 asks for key splits (tk/src/ops/attention.rs:79, 280-302): the
+ * count is capped at the number of 64-key blocks of Tk (split_ranked, :405-410);
+ * each split leaves a partial state in `workspace` and combine_splits
+ * (tk/src/kernels/attention.rs:984-1014) merges them into `out`.  The reference
+ * op allocates those partial tensors itself; this library allocates nothing,
+ * so the caller lends `workspace` (svodk_attention_workspace says how many
+ * bytes).  Without a large enough workspace a split call answers
+ * SVODK_GRAPH_CONFIG.
  */
 typedef struct svodk_attn {
   int32_t causal;
@@ -97,6 +106,8 @@ typedef struct svodk_attn {
    * batches, only the first `batch_live` are computed and written.
    * <= 0 means all of them. */
   int32_t batch_live;
+  void *workspace; /* device scratch for key splits, or NULL */
+  int64_t workspace_bytes;
 } svodk_attn;
 
 /* Qkv of tk/src/ops/heads.rs:19-31. */
@@ -118,6 +129,14 @@ typedef struct svodk_qkv {
  */
 int svodk_attention(const svodk_tensor *q, const svodk_tensor *k, const svodk_tensor *v, const svodk_attn *opts,
                     const svodk_tensor *out, void *hip_stream);
+
+/*
+ * Bytes of `workspace` svodk_attention needs for these operands and options:
+ * the f32 partial tensors o_part [splits, B, T, H, D], m_part and l_part
+ * [splits, B, T, H] of tk/src/ops/attention.rs:285-293, for the split count the
+ * call would run with; 0 when it would not split.  Pure, no device.
+ */
+int64_t svodk_attention_workspace(const svodk_tensor *q, const svodk_tensor *k, const svodk_attn *opts);
 
 /*
  * ops::heads (tk/src/ops/heads.rs:37-102).

@@ -75,6 +75,8 @@ def _declare(l: ctypes.CDLL) -> None:
     l.svod_oracle_attention_graph.argtypes = common + [_i32, _f32p, _f32p, _f32p, _f32p, _i32]
     l.svod_oracle_attention_flash.restype = ctypes.c_int
     l.svod_oracle_attention_flash.argtypes = common + [_i32, _i32, _i32, _f32p, _f32p, _f32p, _f32p, _i32]
+    l.svod_oracle_attention_flash_split.restype = ctypes.c_int
+    l.svod_oracle_attention_flash_split.argtypes = common + [_i32, _i32, _i32, _i32, _f32p, _f32p, _f32p, _f32p, _i32]
     heads = [_i32] * 5 + [_i32, _i32, ctypes.c_double, _i32] + [_f32p] * 5 + [_f32p] * 3
     for name in ("svod_oracle_heads_direct", "svod_oracle_heads_kernel", "svod_oracle_heads_graph"):
         getattr(l, name).restype = ctypes.c_int
@@ -195,12 +197,13 @@ def attention_graph(p: AttnProblem, threads: int = 8) -> np.ndarray:
     return out
 
 
-def attention_flash(p: AttnProblem, bq: int = 64, bkv: int = 64, threads: int = 8) -> np.ndarray:
-    """The tile program under the host interpreter (tk/src/kernels/attention.rs:381-450,466-924)."""
+def attention_flash(p: AttnProblem, bq: int = 64, bkv: int = 64, threads: int = 8, splits: int = 1) -> np.ndarray:
+    """The tile program under the host interpreter (tk/src/kernels/attention.rs:381-450,466-924);
+    with ``splits > 1`` its keys split and the partial states merged (L609-612, L899-921, L948-1014)."""
     q, k, v = _f32(p.q), _f32(p.k), _f32(p.v)
     out = np.zeros(q.shape, dtype=np.float32)
     args, _keep = p._common()
-    rc = lib().svod_oracle_attention_flash(*args, int(p.bf16), bq, bkv, _ptr(q, _f32p), _ptr(k, _f32p), _ptr(v, _f32p), _ptr(out, _f32p), threads)
+    rc = lib().svod_oracle_attention_flash_split(*args, int(p.bf16), bq, bkv, int(splits), _ptr(q, _f32p), _ptr(k, _f32p), _ptr(v, _f32p), _ptr(out, _f32p), threads)
     if rc:
         raise ValueError(f"oracle attention_flash rejected the problem (rc={rc})")
     return out

@@ -398,6 +398,7 @@ typedef struct {
   int32_t bq, bkv;
   const float *q, *k, *v;
   float *out;
+  int32_t splits; /* key splits: FaCfg::splits (tk/src/kernels/attention.rs:19-21) */
 } flash_ctx;
 
 static inline double r32(double x) { return (double)(float)x; }
@@ -423,6 +424,11 @@ static void flash_slice(const void *ctxp, int32_t b, int32_t h) {
   double *o = (double *)malloc(sizeof(double) * (size_t)bq * (size_t)d);
   double *s = (double *)malloc(sizeof(double) * (size_t)bq * (size_t)bkv);
   double *p16 = (double *)malloc(sizeof(double) * (size_t)bq * (size_t)bkv);
+  const int32_t splits = c->splits > 1 ? c->splits : 1;
+  /* The partial states of the splits: o_part, m_part, l_part (L487-492). */
+  double *pm = (double *)malloc(sizeof(double) * (size_t)splits * (size_t)bq);
+  double *pl = (double *)malloc(sizeof(double) * (size_t)splits * (size_t)bq);
+  double *po = (double *)malloc(sizeof(double) * (size_t)splits * (size_t)bq * (size_t)d);
   for (int32_t q_off = 0; q_off < t; q_off += bq) {
     /* L584-612: the key blocks some query of the tile sees. */
     int32_t first = 0, end = (tk + bkv - 1) / bkv;
@@ -442,12 +448,17 @@ static void flash_slice(const void *ctxp, int32_t b, int32_t h) {
       int32_t e = (len + bkv - 1) / bkv;
       if (e < end) end = e;
     }
+   for (int32_t split = 0; split < splits; split++) {
+    /* L609-612: a split takes an even share of the key blocks. */
+    const int32_t n_blocks = end - first;
+    const int32_t s_first = first + (int32_t)((int64_t)n_blocks * split / splits);
+    const int32_t s_end = first + (int32_t)((int64_t)n_blocks * (split + 1) / splits);
     for (int32_t r = 0; r < bq; r++) {
       m[r] = (double)(float)-1e30; /* L616 */
       l[r] = 0.0;
       for (int32_t dd = 0; dd < d; dd++) o[(int64_t)r * d + dd] = 0.0;
     }
-    for (int32_t blk = first; blk < end; blk++) {
+    for (int32_t blk = s_first; blk < s_end; blk++) {
       const int32_t k0 = blk * bkv;
       /* s = q . k^T, rows past t and keys past the view's bound read as zero. */
       for (int32_t r = 0; r < bq; r++) {
@@ -506,6 +517,28 @@ static void flash_slice(const void *ctxp, int32_t b, int32_t h) {
         }
       }
     }
+    memcpy(pm + (int64_t)split * bq, m, sizeof(double) * (size_t)bq);
+    memcpy(pl + (int64_t)split * bq, l, sizeof(double) * (size_t)bq);
+    memcpy(po + (int64_t)split * bq * d, o, sizeof(double) * (size_t)bq * (size_t)d);
+   }
+    if (splits > 1) {
+      /* merged() of L948-969 as combine_splits runs it (L984-1014), in f32: the largest
+       * maximum, each part rescaled to it, sums in split order. */
+      for (int32_t r = 0; r < bq; r++) {
+        double mm = pm[r];
+        for (int32_t sp = 1; sp < splits; sp++)
+          if (pm[(int64_t)sp * bq + r] > mm) mm = pm[(int64_t)sp * bq + r];
+        for (int32_t sp = 0; sp < splits; sp++) {
+          const double w = r32(exp2(r32(pm[(int64_t)sp * bq + r] - mm)));
+          const double lw = r32(pl[(int64_t)sp * bq + r] * w);
+          l[r] = sp == 0 ? lw : r32(l[r] + lw);
+          for (int32_t dd = 0; dd < d; dd++) {
+            const double ow = r32(po[((int64_t)sp * bq + r) * d + dd] * w);
+            o[(int64_t)r * d + dd] = sp == 0 ? ow : r32(o[(int64_t)r * d + dd] + ow);
+          }
+        }
+      }
+    }
     /* L974-980 normalized, cast, bounded store. */
     for (int32_t r = 0; r < bq; r++) {
       const int32_t i = q_off + r;
@@ -523,6 +556,9 @@ static void flash_slice(const void *ctxp, int32_t b, int32_t h) {
   free(o);
   free(s);
   free(p16);
+  free(pm);
+  free(pl);
+  free(po);
 }
 
 int svod_oracle_attention_flash(int32_t batch, int32_t t, int32_t tk, int32_t heads, int32_t kv_heads, int32_t d,
@@ -532,10 +568,27 @@ int svod_oracle_attention_flash(int32_t batch, int32_t t, int32_t tk, int32_t he
                                 const float *v, float *out, int32_t threads) {
   flash_ctx c = {{batch, t, tk, heads, kv_heads, d, causal, window_left, window_right, scale, key_lens, key_mask,
                   mask_stride, bf16_stream},
-                 bq, bkv, q, k, v, out};
+                 bq, bkv, q, k, v, out, 1};
   int rc = check_problem(&c.p);
   if (rc) return rc;
   if (bq <= 0 || bkv <= 0) return -1;
+  run_slices(flash_slice, &c, batch, heads, threads);
+  return 0;
+}
+
+/* The same program with its keys split `splits` ways and the partial states merged
+ * (tk/src/kernels/attention.rs:487-492, 609-612, 899-921 and combine_splits, 948-1014). */
+int svod_oracle_attention_flash_split(int32_t batch, int32_t t, int32_t tk, int32_t heads, int32_t kv_heads, int32_t d,
+                                      int32_t causal, int32_t window_left, int32_t window_right, float scale,
+                                      const int32_t *key_lens, const int32_t *key_mask, int32_t mask_stride,
+                                      int32_t bf16_stream, int32_t bq, int32_t bkv, int32_t splits, const float *q,
+                                      const float *k, const float *v, float *out, int32_t threads) {
+  flash_ctx c = {{batch, t, tk, heads, kv_heads, d, causal, window_left, window_right, scale, key_lens, key_mask,
+                  mask_stride, bf16_stream},
+                 bq, bkv, q, k, v, out, splits};
+  int rc = check_problem(&c.p);
+  if (rc) return rc;
+  if (bq <= 0 || bkv <= 0 || splits <= 0) return -1;
   run_slices(flash_slice, &c, batch, heads, threads);
   return 0;
 }

@@ -42,6 +42,7 @@ typedef __attribute__((ext_vector_type(4))) short s16x4;
 typedef __attribute__((ext_vector_type(8))) short s16x8;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 typedef __attribute__((ext_vector_type(4))) int i32x4;
@@ -501,13 +502,19 @@ struct Geometry {
   uint32_t group;                // heads / kv_heads
   uint32_t units;                // kv_heads * batch
 };
+// The key splits of a launch that has them, and where their partial states go.
+struct Splits {
+  uint32_t count, rcp;
+  float *o_part, *m_part, *l_part;
+  uint32_t nbatch;
+};
 
-template <int D, int NW, bool CAUSAL>
+template <int D, int NW, bool CAUSAL, bool SPLIT>
 __global__ __launch_bounds__(NW * 64, D == 64 ? 3 : 2) void flash_fwd_kernel(
     uint32_t unit_size, uint32_t unit_rcp, uint32_t nqt_u, uint32_t nqt_rcp, uint32_t kvh_u, uint32_t kvh_rcp,
     uint32_t units, uint32_t heads_group, const void *__restrict__ key_lens, const uint16_t *__restrict__ q, int32_t t,
     uint32_t tk_lens64, const uint16_t *__restrict__ k, const uint16_t *__restrict__ v,
-    uint16_t *__restrict__ o, const void *__restrict__ key_mask, int32_t mask_bytes, float scale) {
+    uint16_t *__restrict__ o, const void *__restrict__ key_mask, int32_t mask_bytes, float scale, Splits sp) {
   // The body is device code only: the host pass needs the kernel's handle, not its
   // instructions (and drops the whole instantiation over the LDS-fill instructions).
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -544,9 +551,15 @@ __global__ __launch_bounds__(NW * 64, D == 64 ? 3 : 2) void flash_fwd_kernel(
   const int kvh = (int)(unit - (uint32_t)b * geo.kv_heads);  // L548: query head h reads KV head h / (heads / kv_heads)
   const int h = kvh * (int)geo.group + (int)head_in_group;
   const int kv_heads = (int)geo.kv_heads;
-  const int nqt = (int)geo.nqt;
+  // Grid x of the reference is order * splits + split (L523); geo.nqt counts those.
+  int split = 0, tile = order, nqt = (int)geo.nqt;
+  if (SPLIT) {
+    tile = (int)div_by((uint32_t)order, sp.count, sp.rcp);
+    split = order - tile * (int)sp.count;
+    nqt = (int)div_by(geo.nqt, sp.count, sp.rcp);
+  }
   // Where later queries see more keys the last query blocks run first (L524-528).
-  const int qt = CAUSAL ? (nqt - 1 - order) : order;
+  const int qt = CAUSAL ? (nqt - 1 - tile) : tile;
   const int q_off = qt * BQ;
 
   W w;
@@ -558,14 +571,13 @@ __global__ __launch_bounds__(NW * 64, D == 64 ? 3 : 2) void flash_fwd_kernel(
 
   const int64_t q_row_stride = (int64_t)heads * D;
   // ---- Q fragments: B operand of the score product, resident for the block.
-  w.wave_first_row = q_off + w.wave * kWaveRows;
-  w.my_row = w.wave_first_row + ln;
+  const int row = q_off + w.wave * kWaveRows + ln;  // this lane's query
   {
-    const uint16_t *q_ptr = q + ((int64_t)b * t + w.my_row) * q_row_stride + (int64_t)h * D + w.g * 8;
+    const uint16_t *q_ptr = q + ((int64_t)b * t + row) * q_row_stride + (int64_t)h * D + w.g * 8;
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
       u32x4 x = {0, 0, 0, 0};
-      if (w.my_row < t) x = *reinterpret_cast<const u32x4 *>(q_ptr + ks * 16);
+      if (row < t) x = *reinterpret_cast<const u32x4 *>(q_ptr + ks * 16);
       w.qf[ks] = __builtin_bit_cast(bf16x8, x);
     }
   }
@@ -582,16 +594,28 @@ __global__ __launch_bounds__(NW * 64, D == 64 ? 3 : 2) void flash_fwd_kernel(
   int end = (tk + kBkv - 1) / kBkv;
   if (CAUSAL) end = min(end, (q_off + BQ + kBkv - 1) / kBkv);
   if (key_lens != nullptr) end = min(end, (len + kBkv - 1) / kBkv);
+  // L609-612: a split takes an even share of those blocks.  From here on the kernel works in
+  // the split's own frame: keys, lengths and query rows count from the split's first key.
+  int first_key = 0;
+  if (SPLIT) {
+    const int s_first = (int)div_by((uint32_t)end * (uint32_t)split, sp.count, sp.rcp);
+    const int s_end = (int)div_by((uint32_t)end * (uint32_t)(split + 1), sp.count, sp.rcp);
+    first_key = s_first * kBkv;
+    end = s_end - s_first;
+    len = max(len - first_key, 0);
+  }
   w.end = end;
   w.len = len;
-  w.tk = tk;
+  w.tk = tk - first_key;
   w.key_mask = key_mask;
-  w.mask_row = (int64_t)b * tk;
+  w.mask_row = (int64_t)b * tk + first_key;
   w.mask_bytes = mask_bytes;
+  w.wave_first_row = q_off + w.wave * kWaveRows - first_key;
+  w.my_row = w.wave_first_row + ln;
 
   w.kv_row_bytes = kv_heads * D * 2;
-  w.k_base = (const uint8_t *)(k + ((int64_t)b * tk * kv_heads + kvh) * D);
-  w.v_base = (const uint8_t *)(v + ((int64_t)b * tk * kv_heads + kvh) * D);
+  w.k_base = (const uint8_t *)(k + (((int64_t)b * tk + first_key) * kv_heads + kvh) * D);
+  w.v_base = (const uint8_t *)(v + (((int64_t)b * tk + first_key) * kv_heads + kvh) * D);
   w.kv_bytes = len > 0 ? (int64_t)(len - 1) * w.kv_row_bytes + D * 2 : 0;
   w.lds0 = (int)(uintptr_t)(LDS_PTR(uint8_t))(smem);
 
@@ -650,7 +674,10 @@ __global__ __launch_bounds__(NW * 64, D == 64 ? 3 : 2) void flash_fwd_kernel(
   // A causal wave past its last visible key has nothing to add from a block: it only keeps
   // filling and meeting the barriers.  Blocks [0, my_end) are this wave's.
   int my_end = end;
-  if (CAUSAL) my_end = min(end, (w.wave_first_row + kWaveRows - 1) / kBkv + 1);
+  if (CAUSAL) {
+    const int last_row = w.wave_first_row + kWaveRows - 1;  // negative: the split lies past every row's diagonal
+    my_end = min(end, last_row < 0 ? 0 : last_row / kBkv + 1);
+  }
 
   float sv[32], nv[32];  // S of the current and of the next block, swapping roles each hot step
   float bm = -INFINITY;
@@ -685,12 +712,33 @@ __global__ __launch_bounds__(NW * 64, D == 64 ? 3 : 2) void flash_fwd_kernel(
   for (; blk < my_end; blk++) edge_step<D, NW, CAUSAL>(w, smem, blk, my_end, sv, bm);
   for (; blk < end; blk++) idle_step<D, NW>(w, blk);
 
-  // ---- out = o / (l == 0 ? 1 : l), bounded store (L892-898, L974-980).
   const Pair lp = both_halves(w.l_run);
   const float l_tot = lp.a + lp.b;
+  if (SPLIT) {
+    // ---- the split's partial state (L899-921): the accumulator as it stands, the maximum in
+    // the exponent's units (L848-853) and the sum.
+    if (row < t) {
+      const int64_t at = (((int64_t)split * sp.nbatch + b) * t + row) * heads + h;
+      if (w.g == 0) {
+        sp.m_part[at] = w.positive ? w.m_run * w.c_exp : w.m_run;
+        sp.l_part[at] = l_tot;
+      }
+      float *o_ptr = sp.o_part + at * D + 4 * w.g;
+#pragma unroll
+      for (int db = 0; db < DB; db++) {
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+          const f32x4 x = {w.acc[db][4 * c], w.acc[db][4 * c + 1], w.acc[db][4 * c + 2], w.acc[db][4 * c + 3]};
+          *reinterpret_cast<f32x4 *>(o_ptr + 32 * db + 8 * c) = x;
+        }
+      }
+    }
+    return;
+  }
+  // ---- out = o / (l == 0 ? 1 : l), bounded store (L892-898, L974-980).
   const float inv = 1.0f / (l_tot == 0.0f ? 1.0f : l_tot);
-  if (w.my_row < t) {
-    uint16_t *o_ptr = o + ((int64_t)b * t + w.my_row) * q_row_stride + (int64_t)h * D + 4 * w.g;
+  if (row < t) {
+    uint16_t *o_ptr = o + ((int64_t)b * t + row) * q_row_stride + (int64_t)h * D + 4 * w.g;
 #pragma unroll
     for (int db = 0; db < DB; db++) {
 #pragma unroll
@@ -705,18 +753,19 @@ __global__ __launch_bounds__(NW * 64, D == 64 ? 3 : 2) void flash_fwd_kernel(
 #endif  // __HIP_DEVICE_COMPILE__
 }
 
-template <int D, int NW, bool CAUSAL>
+template <int D, int NW, bool CAUSAL, bool SPLIT>
 hipError_t launch(const AttnArgs &a, hipStream_t stream) {
   using TL = Tile<D>;
   constexpr int BQ = NW * kWaveRows;
-  const int nqt = (a.t + BQ - 1) / BQ;
+  const int splits = SPLIT ? a.splits : 1;
+  const int nqt = (a.t + BQ - 1) / BQ * splits;  // grid x: query tile * splits + split (L512, L523)
   const int64_t blocks = (int64_t)nqt * a.heads * a.batch;
   if (blocks == 0) return hipSuccess;
   if (blocks > 0x7ffffff0LL) return hipErrorInvalidConfiguration;
   constexpr int smem = TL::kLds;
   // The fills address a (batch, kv head)'s rows with 32-bit byte offsets.
   if ((int64_t)a.tk * a.kv_heads * a.d * 2 > 0x7fffffffLL) return hipErrorInvalidValue;
-  auto kernel = flash_fwd_kernel<D, NW, CAUSAL>;
+  auto kernel = flash_fwd_kernel<D, NW, CAUSAL, SPLIT>;
   static bool configured = false;  // one attribute call per instantiation
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
@@ -743,16 +792,25 @@ hipError_t launch(const AttnArgs &a, hipStream_t stream) {
   if (a.heads > 0xffff) return hipErrorInvalidConfiguration;  // heads and group share an argument
   const uint32_t heads_group = (uint32_t)a.heads | geo.group << 16;
   const uint32_t tk_lens64 = (uint32_t)a.tk | (a.lens_i64 ? 0x80000000u : 0u);
+  Splits sp;
+  sp.count = (uint32_t)splits;
+  sp.rcp = rcp(sp.count);
+  sp.o_part = a.o_part;
+  sp.m_part = a.m_part;
+  sp.l_part = a.l_part;
+  sp.nbatch = (uint32_t)a.batch;
+  if (splits > 1 && (a.o_part == nullptr || a.m_part == nullptr || a.l_part == nullptr)) return hipErrorInvalidValue;
   hipLaunchKernelGGL(kernel, dim3((uint32_t)grid), dim3(NW * 64), smem, stream, geo.unit_size, geo.unit_rcp, geo.nqt,
                      geo.nqt_rcp, geo.kv_heads, geo.kvh_rcp, geo.units, heads_group, a.key_lens,
                      (const uint16_t *)a.q, a.t, tk_lens64, (const uint16_t *)a.k,
-                     (const uint16_t *)a.v, (uint16_t *)a.o, a.key_mask, a.mask_bytes, a.scale);
+                     (const uint16_t *)a.v, (uint16_t *)a.o, a.key_mask, a.mask_bytes, a.scale, sp);
   return hipGetLastError();
 }
 
 template <int D>
 hipError_t launch_d(const AttnArgs &a, hipStream_t stream) {
-  return a.causal ? launch<D, 4, true>(a, stream) : launch<D, 4, false>(a, stream);
+  if (a.splits > 1) return a.causal ? launch<D, 4, true, true>(a, stream) : launch<D, 4, false, true>(a, stream);
+  return a.causal ? launch<D, 4, true, false>(a, stream) : launch<D, 4, false, false>(a, stream);
 }
 
 }  // namespace

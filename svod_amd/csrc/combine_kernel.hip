@@ -1,0 +1,82 @@
+// combine_splits for gfx950: the partial online-softmax states the attention kernel's key
+// splits leave are merged into the output (tk/src/kernels/attention.rs:948-1014):
+//   m = max_s m_s ;  w_s = 2^(m_s - m) ;  l = sum_s l_s w_s ;  o = sum_s o_s w_s
+//   out = o / (l == 0 ? 1 : l), a row no key reached coming out as zeros (L971-980).
+// Sums run in split order, one op at a time in f32, as the reference's tile program does.
+//
+// The kernel is HBM-bound (every partial is read once): a row of d floats is shared by d/4
+// lanes, each reading one 128-bit chunk per split and writing 8 bytes of bf16.
+#include <hip/hip_runtime.h>
+
+#include "kernels.h"
+
+namespace svodk {
+namespace {
+
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+
+constexpr int kThreads = 256;
+
+__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+  f32x2 f = {lo, hi};
+  bf16x2 b = __builtin_convertvector(f, bf16x2);  // round to nearest even
+  return __builtin_bit_cast(uint32_t, b);
+}
+
+template <int D>
+__global__ __launch_bounds__(kThreads) void combine_kernel(const float *__restrict__ o_part,
+                                                           const float *__restrict__ m_part,
+                                                           const float *__restrict__ l_part, uint16_t *__restrict__ o,
+                                                           int64_t rows, int32_t splits) {
+#pragma clang fp contract(off)
+  constexpr int kLanes = D / 4;  // lanes sharing a row
+  const int64_t gid = (int64_t)__builtin_amdgcn_workgroup_id_x() * kThreads + __builtin_amdgcn_workitem_id_x();
+  const int64_t row = gid / kLanes;
+  const int part = (int)(gid % kLanes);
+  if (row >= rows) return;
+  float m = m_part[row];
+  for (int s = 1; s < splits; s++) m = __builtin_fmaxf(m, m_part[(int64_t)s * rows + row]);
+  float l = 0.0f;
+  f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+  for (int s = 0; s < splits; s++) {
+    const int64_t at = (int64_t)s * rows + row;
+    const float w = __builtin_amdgcn_exp2f(m_part[at] - m);
+    const float lw = l_part[at] * w;
+    const f32x4 x = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(o_part + at * D) + part);
+    const f32x4 ow = x * w;
+    l = s == 0 ? lw : l + lw;
+    acc = s == 0 ? ow : acc + ow;
+  }
+  const float ll = l == 0.0f ? 1.0f : l;
+  u32x2 out;
+  out[0] = pack2(acc[0] / ll, acc[1] / ll);
+  out[1] = pack2(acc[2] / ll, acc[3] / ll);
+  *(reinterpret_cast<u32x2 *>(o + row * D) + part) = out;
+}
+
+template <int D>
+hipError_t launch(const CombineArgs &a, hipStream_t stream) {
+  const int64_t threads = a.rows * (D / 4);
+  if (threads == 0) return hipSuccess;
+  const int64_t blocks = (threads + kThreads - 1) / kThreads;
+  if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;
+  hipLaunchKernelGGL(combine_kernel<D>, dim3((uint32_t)blocks), dim3(kThreads), 0, stream, a.o_part, a.m_part,
+                     a.l_part, (uint16_t *)a.o, a.rows, a.splits);
+  return hipGetLastError();
+}
+
+}  // namespace
+
+hipError_t launch_combine(const CombineArgs &a, hipStream_t stream) {
+  if (a.splits < 1) return hipErrorInvalidValue;
+  switch (a.d) {
+    case 64: return launch<64>(a, stream);
+    case 128: return launch<128>(a, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+}  // namespace svodk

@@ -38,8 +38,22 @@ struct AttnArgs {
   int32_t t, tk, heads, kv_heads, d;
   int32_t causal;
   float scale;
+  // Key splits (FaCfg::splits, tk/src/kernels/attention.rs:19-21, 487-492): with splits > 1 each
+  // split writes its partial state instead of `o`: o_part [splits, batch, t, heads, d],
+  // m_part and l_part [splits, batch, t, heads], all f32; launch_combine merges them.
+  int32_t splits;
+  float *o_part, *m_part, *l_part;
 };
 hipError_t launch_attention(const AttnArgs &a, hipStream_t stream);
+
+// combine_splits: tk/src/kernels/attention.rs:948-1014.
+struct CombineArgs {
+  const float *o_part, *m_part, *l_part;
+  void *o;       // [rows, d] bf16
+  int64_t rows;  // batch * t * heads
+  int32_t d, splits;
+};
+hipError_t launch_combine(const CombineArgs &a, hipStream_t stream);
 bool attention_supports(int32_t d);
 // Text of the tile configuration launch_attention picks for `a` (for chosen()).
 const char *attention_config(const AttnArgs &a);

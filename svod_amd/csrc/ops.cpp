@@ -241,6 +241,14 @@ int svodk_plan_heads(int32_t has_target, const int32_t *dtypes, int32_t n_dtypes
   return plan_heads(has_target != 0, dtypes, n_dtypes, x_dims, x_rank, head_dim);
 }
 
+// split_ranked of tk/src/ops/attention.rs:405-410 for this library's one tile shape: a named
+// count is capped at the 64-key blocks of tk; none, or one, leaves the keys unsplit.
+static int split_count(int32_t asked, int64_t tk) {
+  const int64_t most = tk > 0 ? (tk + 63) / 64 : 1;
+  if (asked <= 1) return 1;
+  return (int)(asked < most ? asked : most);
+}
+
 // attend (tk/src/ops/attention.rs:126-303).
 int svodk_attention(const svodk_tensor *q, const svodk_tensor *k, const svodk_tensor *v, const svodk_attn *opts,
                     const svodk_tensor *out, void *hip_stream) {
@@ -326,8 +334,7 @@ int svodk_attention(const svodk_tensor *q, const svodk_tensor *k, const svodk_te
   if (why != 0) return ran_graph(op, why);
   // Options the reference's kernel holds and this library's does not: no
   // config here holds them (the reference's own use of Fallback::Config, L210-214).
-  if (opts->has_window || opts->has_chunk || opts->seg_start != nullptr || opts->has_cache || opts->bias != nullptr ||
-      opts->splits > 1)
+  if (opts->has_window || opts->has_chunk || opts->seg_start != nullptr || opts->has_cache || opts->bias != nullptr)
     return ran_graph(op, SVODK_GRAPH_CONFIG);
   const int64_t t = q->shape[1], tk = k->shape[1], d = q->shape[3];
   if (t > 0x7fffffff || tk > 0x7fffffff || heads > 0x7fffffff || cap > 0x7fffffff)
@@ -364,10 +371,48 @@ int svodk_attention(const svodk_tensor *q, const svodk_tensor *k, const svodk_te
   a.causal = opts->causal != 0;
   // L230: the default scale is 1/sqrt(D) in f32.
   a.scale = opts->has_scale ? opts->scale : 1.0f / std::sqrt((float)d);
+  // L280-302: key splits.  The partial tensors live in the caller's workspace.
+  a.splits = split_count(opts->splits, tk);
+  if (a.splits > 1) {
+    const int64_t rows = (int64_t)a.batch * t * heads;
+    const int64_t need = (int64_t)a.splits * rows * (d + 2) * 4;
+    if (opts->workspace == nullptr || opts->workspace_bytes < need) return ran_graph(op, SVODK_GRAPH_CONFIG);
+    Span ws[2] = {{"workspace", opts->workspace, (size_t)need, true}, {"o", out->data, (size_t)numel(out) * 2, true}};
+    if (int rc = check_aliasing(op, ws, 2)) return rc;
+    for (int i = 0; i < 3; i++) {
+      Span pair[2] = {{"workspace", opts->workspace, (size_t)need, true}, spans[i]};
+      if (int rc = check_aliasing(op, pair, 2)) return rc;
+    }
+    a.o_part = (float *)opts->workspace;
+    a.m_part = a.o_part + (int64_t)a.splits * rows * d;
+    a.l_part = a.m_part + (int64_t)a.splits * rows;
+  }
   ran(op, "flash_attention", svodk::attention_config(a));
-  const hipError_t e = svodk::launch_attention(a, (hipStream_t)hip_stream);
+  hipError_t e = svodk::launch_attention(a, (hipStream_t)hip_stream);
   if (e != hipSuccess) return fail(SVODK_ERR_LAUNCH, "%s: %s", op, hipGetErrorString(e));
+  if (a.splits > 1) {
+    svodk::CombineArgs c{};
+    c.o_part = a.o_part;
+    c.m_part = a.m_part;
+    c.l_part = a.l_part;
+    c.o = out->data;
+    c.rows = (int64_t)a.batch * t * heads;
+    c.d = a.d;
+    c.splits = a.splits;
+    ran(op, "combine_splits", "NormCfg { br: 4 }");
+    e = svodk::launch_combine(c, (hipStream_t)hip_stream);
+    if (e != hipSuccess) return fail(SVODK_ERR_LAUNCH, "%s: %s", op, hipGetErrorString(e));
+  }
   return SVODK_KERNEL;
+}
+
+// The workspace of a split call (tk/src/ops/attention.rs:285-293).
+int64_t svodk_attention_workspace(const svodk_tensor *q, const svodk_tensor *k, const svodk_attn *opts) {
+  if (!well_formed(q) || !well_formed(k) || opts == nullptr || q->rank != 4 || k->rank != 4) return 0;
+  const int splits = split_count(opts->splits, k->shape[1]);
+  if (splits <= 1) return 0;
+  const int64_t batch = opts->batch_live > 0 ? opts->batch_live : q->shape[0];
+  return (int64_t)splits * batch * q->shape[1] * q->shape[2] * (q->shape[3] + 2) * 4;
 }
 
 // heads (tk/src/ops/heads.rs:37-102).

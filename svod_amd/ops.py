@@ -40,7 +40,7 @@ class _Attn(ctypes.Structure):
         ("chunk_left", ctypes.c_int64), ("chunk_right", ctypes.c_int64),
         ("seg_start", ctypes.POINTER(_Tensor)), ("has_cache", ctypes.c_int32), ("bias", ctypes.POINTER(_Tensor)),
         ("splits", ctypes.c_int32), ("has_scale", ctypes.c_int32), ("scale", ctypes.c_float),
-        ("batch_live", ctypes.c_int32),
+        ("batch_live", ctypes.c_int32), ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_int64),
     ]
 
 
@@ -70,6 +70,8 @@ def load_library() -> ctypes.CDLL:
     tp = ctypes.POINTER(_Tensor)
     lib.svodk_attention.restype = ctypes.c_int
     lib.svodk_attention.argtypes = [tp, tp, tp, ctypes.POINTER(_Attn), tp, ctypes.c_void_p]
+    lib.svodk_attention_workspace.restype = ctypes.c_int64
+    lib.svodk_attention_workspace.argtypes = [tp, tp, ctypes.POINTER(_Attn)]
     lib.svodk_heads.restype = ctypes.c_int
     lib.svodk_heads.argtypes = [tp, ctypes.POINTER(_Qkv), tp, tp, tp, ctypes.c_void_p]
     i32p, i64p = ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int64)
@@ -208,7 +210,7 @@ class Qkv:
 
 
 def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, opts: Optional[Attn] = None,
-              out: Optional[torch.Tensor] = None) -> torch.Tensor:
+              out: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``softmax(q·kᵀ·scale)·v`` over ``q [B,T,H,D]`` and ``k``/``v [B,Tk,H_kv,D]``;
     returns ``[B,T,H,D]`` (tk/src/ops/attention.rs:98-103).  Enqueued on the
     current stream of ``q``'s device; returns without synchronising."""
@@ -236,6 +238,15 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, opts: Optional[
         a.has_scale, a.scale = 1, float(opts.scale)
     a.batch_live = opts.batch_live or 0
     qd, kd, vd, od = _desc(q), _desc(k), _desc(v), _desc(out)
+    if opts.splits is not None and opts.splits > 1:
+        # The partial tensors of a split call, which the reference op allocates itself
+        # (tk/src/ops/attention.rs:285-293): here the harness does, like the output.
+        need = int(lib.svodk_attention_workspace(ctypes.byref(qd), ctypes.byref(kd), ctypes.byref(a)))
+        if workspace is None and need > 0:
+            workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
+        if workspace is not None:
+            keep.append(workspace)
+            a.workspace, a.workspace_bytes = workspace.data_ptr(), workspace.numel() * workspace.element_size()
     status = lib.svodk_attention(ctypes.byref(qd), ctypes.byref(kd), ctypes.byref(vd), ctypes.byref(a),
                                  ctypes.byref(od), ctypes.c_void_p(_stream(q)))
     _finish("attention", status)

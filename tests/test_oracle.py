@@ -303,3 +303,43 @@ def test_rope_table_follows_the_reference_formula():
     assert np.abs(sin - np.sin(ang.astype(np.float64))).max() < 1e-5
     assert cos[0].min() == 1.0 and sin[0].max() == 0.0
     assert abs(inv[-1] - 1e6 ** (-126.0 / 128)) < 1e-9
+
+
+# ---- key splits: the merge of partial states (tk/src/kernels/attention.rs:948-1014)
+@pytest.mark.parametrize("splits", [2, 3, 4, 7, 16])
+def test_split_states_merge_to_the_direct_softmax(splits):
+    """The merge is an identity of the softmax: sum_s 2^(m_s - m) (l_s, o_s) over any partition of
+    the keys is the whole sum.  In f32 without bf16 rounding the merged tile program must sit on the
+    f64 direct softmax like the unsplit one (1e-5), for any split count, more splits than blocks,
+    a lane with no keys and a causal mask (whose late splits see no key for early rows)."""
+    rng = np.random.default_rng(splits)
+    b, t, tk, h, hkv, d = 2, 70, 200, 4, 2, 64
+    q, k, v = (rng.standard_normal(s).astype(np.float32) for s in ((b, t, h, d), (b, tk, hkv, d), (b, tk, hkv, d)))
+    for causal, lens in ((False, [200, 70]), (True, [200, 0]), (False, None)):
+        p = oracle.AttnProblem(q, k, v, causal=causal, key_lens=None if lens is None else np.asarray(lens), bf16=False)
+        want = oracle.attention_direct(p)
+        got = oracle.attention_flash(p, bq=64, bkv=64, splits=splits)
+        assert np.abs(got - want).max() <= 1e-5 * max(1.0, np.abs(want).max())
+        if lens is not None and 0 in lens:
+            assert not got[lens.index(0)].any()
+
+
+def test_a_hand_merged_pair_of_halves_is_what_the_split_program_returns():
+    """Brute force on a tiny case: run the unsplit program on each half of the keys, rebuild (m, l, o)
+    of each half from first principles in f64, merge by the rule, compare."""
+    rng = np.random.default_rng(3)
+    t, tk, d = 4, 128, 16
+    q, k, v = (rng.standard_normal(s).astype(np.float32) for s in ((1, t, 1, d), (1, tk, 1, d), (1, tk, 1, d)))
+    scale = 0.25
+    p = oracle.AttnProblem(q, k, v, scale=scale, bf16=False)
+    got = oracle.attention_flash(p, bq=64, bkv=64, splits=2)[0, :, 0, :]
+    s = (q[0, :, 0, :].astype(np.float64) @ k[0, :, 0, :].astype(np.float64).T) * scale * np.log2(np.e)
+    parts = []
+    for lo, hi in ((0, 64), (64, 128)):
+        m = s[:, lo:hi].max(axis=1)
+        e = np.exp2(s[:, lo:hi] - m[:, None])
+        parts.append((m, e.sum(axis=1), e @ v[0, lo:hi, 0, :].astype(np.float64)))
+    m = np.maximum(parts[0][0], parts[1][0])
+    l = sum(pl * np.exp2(pm - m) for pm, pl, _ in parts)
+    o = sum(po * np.exp2(pm - m)[:, None] for pm, _, po in parts)
+    assert np.abs(got - o / l[:, None]).max() <= 2e-6

@@ -131,6 +131,15 @@ int svodk_attention(const svodk_tensor *q, const svodk_tensor *k, const svodk_te
                     const svodk_tensor *out, void *hip_stream);
 
 /*
+ * ops::attention_packed (tk/src/ops/attention.rs:104-122): attention over a fused
+ * projection qkv [B, T, (heads + 2*kv_heads)*D] of queries, keys and values side
+ * by side, read in place; out [B, T, heads, D].  No cache.  Bit-identical to
+ * svodk_attention on the three split tensors (tk/src/test/unit/ops.rs:519-521).
+ */
+int svodk_attention_packed(const svodk_tensor *qkv, int32_t heads, int32_t kv_heads, const svodk_attn *opts,
+                           const svodk_tensor *out, void *hip_stream);
+
+/*
  * Bytes of `workspace` svodk_attention needs for these operands and options:
  * the f32 partial tensors o_part [splits, B, T, H, D], m_part and l_part
  * [splits, B, T, H] of tk/src/ops/attention.rs:285-293, for the split count the

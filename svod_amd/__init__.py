@@ -15,6 +15,7 @@ from .ops import (  # noqa: F401
     OpError,
     Qkv,
     attention,
+    attention_packed,
     chosen,
     heads,
     library_path,

@@ -514,7 +514,8 @@ __global__ __launch_bounds__(NW * 64, D == 64 ? 3 : 2) void flash_fwd_kernel(
     uint32_t unit_size, uint32_t unit_rcp, uint32_t nqt_u, uint32_t nqt_rcp, uint32_t kvh_u, uint32_t kvh_rcp,
     uint32_t units, uint32_t heads_group, const void *__restrict__ key_lens, const uint16_t *__restrict__ q, int32_t t,
     uint32_t tk_lens64, const uint16_t *__restrict__ k, const uint16_t *__restrict__ v,
-    uint16_t *__restrict__ o, const void *__restrict__ key_mask, int32_t mask_bytes, float scale, Splits sp) {
+    uint16_t *__restrict__ o, const void *__restrict__ key_mask, int32_t mask_bytes, float scale, Splits sp,
+    int32_t q_row_elems, int32_t kv_row_elems) {
   // The body is device code only: the host pass needs the kernel's handle, not its
   // instructions (and drops the whole instantiation over the LDS-fill instructions).
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -569,7 +570,10 @@ __global__ __launch_bounds__(NW * 64, D == 64 ? 3 : 2) void flash_fwd_kernel(
   w.g = w.lane >> 5;           // half-wave: the k-chunk of MFMA operands
   const int ln = w.lane & 31;  // the query column this lane owns
 
-  const int64_t q_row_stride = (int64_t)heads * D;
+  // Elements from a token's row to the next: heads * D and kv_heads * D for separate q, k, v;
+  // the fused projection's row for operands read in place (tk/src/ops/attention.rs:104-122).
+  const int64_t q_row_stride = q_row_elems;
+  const int64_t o_row_stride = (int64_t)heads * D;
   // ---- Q fragments: B operand of the score product, resident for the block.
   const int row = q_off + w.wave * kWaveRows + ln;  // this lane's query
   {
@@ -613,9 +617,9 @@ __global__ __launch_bounds__(NW * 64, D == 64 ? 3 : 2) void flash_fwd_kernel(
   w.wave_first_row = q_off + w.wave * kWaveRows - first_key;
   w.my_row = w.wave_first_row + ln;
 
-  w.kv_row_bytes = kv_heads * D * 2;
-  w.k_base = (const uint8_t *)(k + (((int64_t)b * tk + first_key) * kv_heads + kvh) * D);
-  w.v_base = (const uint8_t *)(v + (((int64_t)b * tk + first_key) * kv_heads + kvh) * D);
+  w.kv_row_bytes = kv_row_elems * 2;
+  w.k_base = (const uint8_t *)(k + ((int64_t)b * tk + first_key) * kv_row_elems + (int64_t)kvh * D);
+  w.v_base = (const uint8_t *)(v + ((int64_t)b * tk + first_key) * kv_row_elems + (int64_t)kvh * D);
   w.kv_bytes = len > 0 ? (int64_t)(len - 1) * w.kv_row_bytes + D * 2 : 0;
   w.lds0 = (int)(uintptr_t)(LDS_PTR(uint8_t))(smem);
 
@@ -738,7 +742,7 @@ __global__ __launch_bounds__(NW * 64, D == 64 ? 3 : 2) void flash_fwd_kernel(
   // ---- out = o / (l == 0 ? 1 : l), bounded store (L892-898, L974-980).
   const float inv = 1.0f / (l_tot == 0.0f ? 1.0f : l_tot);
   if (row < t) {
-    uint16_t *o_ptr = o + ((int64_t)b * t + row) * q_row_stride + (int64_t)h * D + 4 * w.g;
+    uint16_t *o_ptr = o + ((int64_t)b * t + row) * o_row_stride + (int64_t)h * D + 4 * w.g;
 #pragma unroll
     for (int db = 0; db < DB; db++) {
 #pragma unroll
@@ -763,8 +767,10 @@ hipError_t launch(const AttnArgs &a, hipStream_t stream) {
   if (blocks == 0) return hipSuccess;
   if (blocks > 0x7ffffff0LL) return hipErrorInvalidConfiguration;
   constexpr int smem = TL::kLds;
+  const int64_t q_row = a.q_row_elems > 0 ? a.q_row_elems : (int64_t)a.heads * a.d;
+  const int64_t kv_row = a.kv_row_elems > 0 ? a.kv_row_elems : (int64_t)a.kv_heads * a.d;
   // The fills address a (batch, kv head)'s rows with 32-bit byte offsets.
-  if ((int64_t)a.tk * a.kv_heads * a.d * 2 > 0x7fffffffLL) return hipErrorInvalidValue;
+  if ((int64_t)a.tk * kv_row * 2 > 0x7fffffffLL || q_row > 0x7fffffffLL) return hipErrorInvalidValue;
   auto kernel = flash_fwd_kernel<D, NW, CAUSAL, SPLIT>;
   static bool configured = false;  // one attribute call per instantiation
   if (!configured) {
@@ -803,7 +809,8 @@ hipError_t launch(const AttnArgs &a, hipStream_t stream) {
   hipLaunchKernelGGL(kernel, dim3((uint32_t)grid), dim3(NW * 64), smem, stream, geo.unit_size, geo.unit_rcp, geo.nqt,
                      geo.nqt_rcp, geo.kv_heads, geo.kvh_rcp, geo.units, heads_group, a.key_lens,
                      (const uint16_t *)a.q, a.t, tk_lens64, (const uint16_t *)a.k,
-                     (const uint16_t *)a.v, (uint16_t *)a.o, a.key_mask, a.mask_bytes, a.scale, sp);
+                     (const uint16_t *)a.v, (uint16_t *)a.o, a.key_mask, a.mask_bytes, a.scale, sp, (int32_t)q_row,
+                     (int32_t)kv_row);
   return hipGetLastError();
 }
 

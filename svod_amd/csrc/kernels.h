@@ -43,6 +43,9 @@ struct AttnArgs {
   // m_part and l_part [splits, batch, t, heads], all f32; launch_combine merges them.
   int32_t splits;
   float *o_part, *m_part, *l_part;
+  // Elements from a token's row to the next in q and in k/v; 0 = dense (heads * d, kv_heads * d).
+  // A fused projection read in place (tk/src/ops/attention.rs:104-122) has its own row for both.
+  int64_t q_row_elems, kv_row_elems;
 };
 hipError_t launch_attention(const AttnArgs &a, hipStream_t stream);
 

@@ -249,9 +249,10 @@ static int split_count(int32_t asked, int64_t tk) {
   return (int)(asked < most ? asked : most);
 }
 
-// attend (tk/src/ops/attention.rs:126-303).
-int svodk_attention(const svodk_tensor *q, const svodk_tensor *k, const svodk_tensor *v, const svodk_attn *opts,
-                    const svodk_tensor *out, void *hip_stream) {
+// attend (tk/src/ops/attention.rs:126-303): attention of q, k and v, or of the `packed` operand
+// they are views of.
+static int attend(const svodk_tensor *q, const svodk_tensor *k, const svodk_tensor *v, const svodk_tensor *packed,
+                  const svodk_attn *opts, const svodk_tensor *out, void *hip_stream) {
   const char *op = OP_ATTN;
   if (!well_formed(q) || !well_formed(k) || !well_formed(v) || !well_formed(out) || opts == nullptr)
     return fail(SVODK_ERR_ARGUMENT, "%s: a null or malformed tensor descriptor", op);
@@ -340,9 +341,12 @@ int svodk_attention(const svodk_tensor *q, const svodk_tensor *k, const svodk_te
   if (t > 0x7fffffff || tk > 0x7fffffff || heads > 0x7fffffff || cap > 0x7fffffff)
     return ran_graph(op, SVODK_GRAPH_SHAPE);
 
-  Span spans[6] = {{"q", q->data, (size_t)numel(q) * 2, false},
-                   {"k", k->data, (size_t)numel(k) * 2, false},
-                   {"v", v->data, (size_t)numel(v) * 2, false},
+  // A packed operand is one parameter (L268): its views overlap one another by construction.
+  const size_t packed_bytes = packed ? (size_t)numel(packed) * 2 : 0;
+  Span spans[6] = {{packed ? "qkv" : "q", packed ? packed->data : q->data, packed ? packed_bytes : (size_t)numel(q) * 2,
+                    false},
+                   {"k", packed ? nullptr : k->data, packed ? 0 : (size_t)numel(k) * 2, false},
+                   {"v", packed ? nullptr : v->data, packed ? 0 : (size_t)numel(v) * 2, false},
                    {"o", out->data, (size_t)numel(out) * 2, true},
                    {"key_lens", lens ? lens->data : nullptr, lens ? (size_t)numel(lens) * dtype_bytes(lens->dtype) : 0,
                     false},
@@ -371,6 +375,7 @@ int svodk_attention(const svodk_tensor *q, const svodk_tensor *k, const svodk_te
   a.causal = opts->causal != 0;
   // L230: the default scale is 1/sqrt(D) in f32.
   a.scale = opts->has_scale ? opts->scale : 1.0f / std::sqrt((float)d);
+  if (packed != nullptr) a.q_row_elems = a.kv_row_elems = (heads + 2 * kv_heads) * d;
   // L280-302: key splits.  The partial tensors live in the caller's workspace.
   a.splits = split_count(opts->splits, tk);
   if (a.splits > 1) {
@@ -404,6 +409,38 @@ int svodk_attention(const svodk_tensor *q, const svodk_tensor *k, const svodk_te
     if (e != hipSuccess) return fail(SVODK_ERR_LAUNCH, "%s: %s", op, hipGetErrorString(e));
   }
   return SVODK_KERNEL;
+}
+
+int svodk_attention(const svodk_tensor *q, const svodk_tensor *k, const svodk_tensor *v, const svodk_attn *opts,
+                    const svodk_tensor *out, void *hip_stream) {
+  return attend(q, k, v, nullptr, opts, out, hip_stream);
+}
+
+// attention_packed (tk/src/ops/attention.rs:104-122).
+int svodk_attention_packed(const svodk_tensor *qkv, int32_t heads, int32_t kv_heads, const svodk_attn *opts,
+                           const svodk_tensor *out, void *hip_stream) {
+  const char *op = OP_ATTN;
+  if (!well_formed(qkv) || !well_formed(out) || opts == nullptr)
+    return fail(SVODK_ERR_ARGUMENT, "%s: a null or malformed tensor descriptor", op);
+  // L109: whole groups of query heads per KV head.
+  if (!(kv_heads > 0 && heads >= 0 && heads % kv_heads == 0))
+    return fail(SVODK_ERR_HEADS, "%s: %lld query heads are not a multiple of %lld key/value heads", op,
+                (long long)heads, (long long)kv_heads);
+  // L110-114: qkv is [B, T, slots * D] and a packed call has no cache.
+  const int64_t slots = (int64_t)heads + 2 * kv_heads;
+  if (!(qkv->rank == 3 && qkv->shape[2] > 0 && qkv->shape[2] % slots == 0))
+    return fail(SVODK_ERR_SHAPE, "%s: qkv has shape %s, expected [B, T, slots·D]", op, fmt_shape(qkv).c_str());
+  if (opts->has_cache)
+    return fail(SVODK_ERR_SHAPE, "%s: qkv has shape %s, expected [B, T, slots·D] with no cache", op,
+                fmt_shape(qkv).c_str());
+  // L115-121: the three views of the fused row.
+  const int64_t d = qkv->shape[2] / slots;
+  uint16_t *base = (uint16_t *)qkv->data;
+  svodk_tensor q = {base, qkv->dtype, 4, {qkv->shape[0], qkv->shape[1], heads, d}};
+  svodk_tensor k = {base ? base + (int64_t)heads * d : nullptr, qkv->dtype, 4, {qkv->shape[0], qkv->shape[1], kv_heads, d}};
+  svodk_tensor v = {base ? base + ((int64_t)heads + kv_heads) * d : nullptr, qkv->dtype, 4,
+                    {qkv->shape[0], qkv->shape[1], kv_heads, d}};
+  return attend(&q, &k, &v, qkv, opts, out, hip_stream);
 }
 
 // The workspace of a split call (tk/src/ops/attention.rs:285-293).

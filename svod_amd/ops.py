@@ -70,6 +70,8 @@ def load_library() -> ctypes.CDLL:
     tp = ctypes.POINTER(_Tensor)
     lib.svodk_attention.restype = ctypes.c_int
     lib.svodk_attention.argtypes = [tp, tp, tp, ctypes.POINTER(_Attn), tp, ctypes.c_void_p]
+    lib.svodk_attention_packed.restype = ctypes.c_int
+    lib.svodk_attention_packed.argtypes = [tp, ctypes.c_int32, ctypes.c_int32, ctypes.POINTER(_Attn), tp, ctypes.c_void_p]
     lib.svodk_attention_workspace.restype = ctypes.c_int64
     lib.svodk_attention_workspace.argtypes = [tp, tp, ctypes.POINTER(_Attn)]
     lib.svodk_heads.restype = ctypes.c_int
@@ -209,17 +211,7 @@ class Qkv:
     batch_live: Optional[int] = None
 
 
-def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, opts: Optional[Attn] = None,
-              out: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """``softmax(q·kᵀ·scale)·v`` over ``q [B,T,H,D]`` and ``k``/``v [B,Tk,H_kv,D]``;
-    returns ``[B,T,H,D]`` (tk/src/ops/attention.rs:98-103).  Enqueued on the
-    current stream of ``q``'s device; returns without synchronising."""
-    opts = opts or Attn()
-    lib = load_library()
-    if out is None:
-        # The op allocates its output at capacity (tk/src/ops/mod.rs:423-429).
-        out = torch.empty_like(q)
-    keep: list = []
+def _attn_options(opts: Attn, keep: list) -> _Attn:
     a = _Attn()
     a.causal = int(opts.causal)
     a.key_kind = opts.keys.kind
@@ -237,18 +229,63 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, opts: Optional[
     if opts.scale is not None:
         a.has_scale, a.scale = 1, float(opts.scale)
     a.batch_live = opts.batch_live or 0
+    return a
+
+
+def _lend_workspace(lib, a: _Attn, qd: _Tensor, kd: _Tensor, device, workspace, keep: list) -> None:
+    """The partial tensors of a split call, which the reference op allocates itself
+    (tk/src/ops/attention.rs:285-293): here the harness does, like the output."""
+    if a.splits <= 1:
+        return
+    need = int(lib.svodk_attention_workspace(ctypes.byref(qd), ctypes.byref(kd), ctypes.byref(a)))
+    if workspace is None and need > 0:
+        workspace = torch.empty(need, dtype=torch.uint8, device=device)
+    if workspace is not None:
+        keep.append(workspace)
+        a.workspace, a.workspace_bytes = workspace.data_ptr(), workspace.numel() * workspace.element_size()
+
+
+def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, opts: Optional[Attn] = None,
+              out: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``softmax(q·kᵀ·scale)·v`` over ``q [B,T,H,D]`` and ``k``/``v [B,Tk,H_kv,D]``;
+    returns ``[B,T,H,D]`` (tk/src/ops/attention.rs:98-103).  Enqueued on the
+    current stream of ``q``'s device; returns without synchronising."""
+    opts = opts or Attn()
+    lib = load_library()
+    if out is None:
+        # The op allocates its output at capacity (tk/src/ops/mod.rs:423-429).
+        out = torch.empty_like(q)
+    keep: list = []
+    a = _attn_options(opts, keep)
     qd, kd, vd, od = _desc(q), _desc(k), _desc(v), _desc(out)
-    if opts.splits is not None and opts.splits > 1:
-        # The partial tensors of a split call, which the reference op allocates itself
-        # (tk/src/ops/attention.rs:285-293): here the harness does, like the output.
-        need = int(lib.svodk_attention_workspace(ctypes.byref(qd), ctypes.byref(kd), ctypes.byref(a)))
-        if workspace is None and need > 0:
-            workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
-        if workspace is not None:
-            keep.append(workspace)
-            a.workspace, a.workspace_bytes = workspace.data_ptr(), workspace.numel() * workspace.element_size()
+    _lend_workspace(lib, a, qd, kd, q.device, workspace, keep)
     status = lib.svodk_attention(ctypes.byref(qd), ctypes.byref(kd), ctypes.byref(vd), ctypes.byref(a),
                                  ctypes.byref(od), ctypes.c_void_p(_stream(q)))
+    _finish("attention", status)
+    return out
+
+
+def attention_packed(qkv: torch.Tensor, heads: int, kv_heads: int, opts: Optional[Attn] = None,
+                     out: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``attention`` over a fused projection ``qkv [B,T,(heads+2·kv_heads)·D]`` read in place;
+    returns ``[B,T,heads,D]`` (tk/src/ops/attention.rs:104-122)."""
+    opts = opts or Attn()
+    lib = load_library()
+    slots = heads + 2 * kv_heads
+    if out is None and qkv.dim() == 3 and slots > 0 and qkv.shape[2] % slots == 0:
+        out = torch.empty((qkv.shape[0], qkv.shape[1], heads, qkv.shape[2] // slots), dtype=qkv.dtype, device=qkv.device)
+    if out is None:
+        out = torch.empty((1, 1, 1, 1), dtype=qkv.dtype, device=qkv.device)  # the op rejects the shape itself
+    keep: list = []
+    a = _attn_options(opts, keep)
+    xd, od = _desc(qkv), _desc(out)
+    if a.splits > 1 and qkv.dim() == 3:
+        kd = _Tensor()  # the keys' view of the fused rows: [B, T, kv_heads, D]
+        kd.data, kd.dtype, kd.rank = xd.data, xd.dtype, 4
+        kd.shape[0], kd.shape[1], kd.shape[2], kd.shape[3] = qkv.shape[0], qkv.shape[1], kv_heads, out.shape[3]
+        _lend_workspace(lib, a, od, kd, qkv.device, workspace, keep)
+    status = lib.svodk_attention_packed(ctypes.byref(xd), heads, kv_heads, ctypes.byref(a), ctypes.byref(od),
+                                        ctypes.c_void_p(_stream(qkv)))
     _finish("attention", status)
     return out
 

@@ -163,3 +163,30 @@ def test_a_missing_library_is_a_hard_error(monkeypatch, tmp_path):
     monkeypatch.setattr(ops, "_HERE", str(tmp_path))
     with pytest.raises(ImportError, match="no fallback"):
         ops.load_library()
+
+
+# ---- attention_packed: tk/src/ops/attention.rs:107-114
+def test_packed_attention_validates_its_operand():
+    with pytest.raises(OpError) as e:
+        svod_amd.attention_packed(t([2, 16, 100]), 4, 4)  # 100 is not a multiple of 12 slots
+    assert e.value.kind == "Shape"
+    with pytest.raises(OpError) as e:
+        svod_amd.attention_packed(t([2, 16, 12 * 64]), 5, 2)
+    assert e.value.kind == "Heads"
+    with pytest.raises(OpError) as e:
+        svod_amd.attention_packed(t([2, 16, 12 * 64]), 4, 4, Attn(cache=True))
+    assert e.value.kind == "Shape"
+
+
+def test_the_split_workspace_is_the_partial_tensors():
+    """tk/src/ops/attention.rs:285-293: o_part [S,B,T,H,D] + m_part + l_part [S,B,T,H], f32; the count
+    capped at the 64-key blocks of Tk (:405-410)."""
+    lib = svod_amd.load_library()
+    from svod_amd.ops import _attn_options, _desc
+    q, k = t([2, 100, 8, 64]), t([2, 300, 2, 64])
+    for asked, want in ((None, 0), (1, 0), (2, 2), (4, 4), (9, 5)):
+        a = _attn_options(Attn(splits=asked), [])
+        qd, kd = _desc(q), _desc(k)
+        import ctypes
+        got = lib.svodk_attention_workspace(ctypes.byref(qd), ctypes.byref(kd), ctypes.byref(a))
+        assert got == want * 2 * 100 * 8 * (64 + 2) * 4

@@ -116,3 +116,31 @@ def test_full_size_split_equals_unsplit(device):
     torch.cuda.synchronize()
     diff = (whole.float() - part.float()).abs().max().item()
     assert diff <= 2 ** -8, diff
+
+
+# ---- attention_packed (tk/src/ops/attention.rs:104-122)
+def packed_case(b, t, h, hkv, d, seed=31):
+    return Lcg(seed).bf16((b, t, (h + 2 * hkv) * d))
+
+
+@pytest.mark.parametrize("b,t,h,hkv,d,causal,lens,splits", [
+    (2, 100, 4, 4, 64, False, [100, 61], None),
+    (2, 200, 8, 2, 64, True, None, None),
+    (1, 130, 4, 2, 128, True, [99], None),
+    (2, 256, 4, 4, 64, False, [256, 70], 2),
+], ids=["lens", "causal gqa", "d 128 causal gqa ragged", "two splits"])
+def test_packed_attention_is_the_split_call_bit_for_bit(device, b, t, h, hkv, d, causal, lens, splits):
+    """ops.rs:519-521: the packed kernel and the kernel over the three split tensors agree bit for bit;
+    and the packed call sits on the direct softmax like any other."""
+    x = packed_case(b, t, h, hkv, d)
+    xt = bf16_tensor(x, device)
+    q, k, v = (p.contiguous() for p in xt.split([h * d, hkv * d, hkv * d], dim=-1))
+    q, k, v = q.view(b, t, h, d), k.view(b, t, hkv, d), v.view(b, t, hkv, d)
+    keys = KeyMask.none() if lens is None else KeyMask.lens(torch.tensor(lens, dtype=torch.int32, device=device))
+    opts = Attn(causal=causal, keys=keys, splits=splits)
+    packed = svod_amd.attention_packed(xt, h, hkv, opts)
+    split = svod_amd.attention(q, k, v, opts)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(packed), bits(split))
+    p = oracle.AttnProblem(to_np(q), to_np(k), to_np(v), causal=causal, key_lens=None if lens is None else np.asarray(lens))
+    assert max_abs(to_np(packed), oracle.attention_direct(p)) < 2e-2

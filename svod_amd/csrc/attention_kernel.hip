@@ -31,10 +31,21 @@
 // "one MFMA, a share of the VALU work, the LDS reads two MFMAs ahead".
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+
 #include "kernels.h"
 
 namespace svodk {
 namespace {
+
+// The kernel's body is compiled for the device only (see flash_fwd_kernel): to the host pass
+// the helpers below have no caller.
+#if !defined(__HIP_DEVICE_COMPILE__)
+#pragma clang diagnostic ignored "-Wunused-function"
+#pragma clang diagnostic ignored "-Wunused-const-variable"
+#pragma clang diagnostic ignored "-Wunneeded-internal-declaration"
+#pragma clang diagnostic ignored "-Wunused-template"
+#endif
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
@@ -551,7 +562,6 @@ __global__ __launch_bounds__(NW * 64, D == 64 ? 3 : 2) void flash_fwd_kernel(
   const int b = (int)div_by(unit, geo.kv_heads, geo.kvh_rcp);
   const int kvh = (int)(unit - (uint32_t)b * geo.kv_heads);  // L548: query head h reads KV head h / (heads / kv_heads)
   const int h = kvh * (int)geo.group + (int)head_in_group;
-  const int kv_heads = (int)geo.kv_heads;
   // Grid x of the reference is order * splits + split (L523); geo.nqt counts those.
   int split = 0, tile = order, nqt = (int)geo.nqt;
   if (SPLIT) {
@@ -772,12 +782,17 @@ hipError_t launch(const AttnArgs &a, hipStream_t stream) {
   // The fills address a (batch, kv head)'s rows with 32-bit byte offsets.
   if ((int64_t)a.tk * kv_row * 2 > 0x7fffffffLL || q_row > 0x7fffffffLL) return hipErrorInvalidValue;
   auto kernel = flash_fwd_kernel<D, NW, CAUSAL, SPLIT>;
-  static bool configured = false;  // one attribute call per instantiation
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+  // The LDS ring is above the default limit of a launch: one attribute call per instantiation
+  // and device, from whichever thread gets there first (a second call is harmless).
+  static std::atomic<uint64_t> configured{0};  // a bit per device ordinal, devices past 63 always ask
+  int device = 0;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) return e;
+  const uint64_t bit = device < 64 ? 1ull << device : 0;
+  if ((configured.load(std::memory_order_acquire) & bit) == 0) {
+    e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return e;
-    configured = true;
+    configured.fetch_or(bit, std::memory_order_release);
   }
   // Units of work (batch, KV head) are dealt over the XCDs in whole rounds; the workgroups of
   // a round's missing units exit at once.

@@ -52,6 +52,10 @@ _i32 = ctypes.c_int32
 def _declare(l: ctypes.CDLL) -> None:
     l.svod_oracle_round_bf16.restype = ctypes.c_double
     l.svod_oracle_round_bf16.argtypes = [ctypes.c_double]
+    l.svod_oracle_round_f16.restype = ctypes.c_double
+    l.svod_oracle_round_f16.argtypes = [ctypes.c_double]
+    l.svod_oracle_set_stream_dtype.restype = None
+    l.svod_oracle_set_stream_dtype.argtypes = [ctypes.c_int32]
     l.svod_oracle_trunc_bf16.restype = ctypes.c_double
     l.svod_oracle_trunc_bf16.argtypes = [ctypes.c_double]
     l.svod_oracle_bf16_bits.restype = ctypes.c_uint16
@@ -102,6 +106,29 @@ def round_bf16(x):
     nan = np.isnan(a)
     rounded = np.where(nan, (a.view(np.uint32) | 0x00400000) & 0xFFFF0000, rounded).astype(np.uint32)
     return rounded.view(np.float32).reshape(a.shape)
+
+
+def round_f16(x):
+    """The Float16 arm of tk/src/interp.rs:37-50 applied elementwise; float32 values that are f16-exact."""
+    a = np.asarray(x, dtype=np.float32)
+    f = np.vectorize(lambda v: lib().svod_oracle_round_f16(float(v)), otypes=[np.float64])
+    return f(a).astype(np.float32)
+
+
+class stream_dtype:
+    """``with oracle.stream_dtype("f16"):`` — the restatements round their 16-bit values to f16
+    instead of bf16 (the reference kernels run both, tk/src/ops/shape.rs:92-99)."""
+
+    def __init__(self, name: str):
+        self.which = {"bf16": 1, "f16": 2}[name]
+
+    def __enter__(self):
+        lib().svod_oracle_set_stream_dtype(self.which)
+        return self
+
+    def __exit__(self, *exc):
+        lib().svod_oracle_set_stream_dtype(1)
+        return False
 
 
 def bf16_bits(x) -> np.ndarray:

@@ -74,6 +74,43 @@ static inline float round_bf16_f32(float x) {
 
 double svod_oracle_round_bf16(double x) { return (double)round_bf16_f32((float)x); }
 
+/* tk/src/interp.rs:37-50, the Float16 arm: IEEE binary16, round to nearest even, overflow to
+ * infinity, gradual underflow.  Written out on the bits so that it does not lean on the
+ * compiler's own half type. */
+static inline float round_f16_f32(float x) {
+  const uint32_t bits = f32_bits(x), sign = bits & 0x80000000u;
+  const uint32_t exp = (bits >> 23) & 0xffu, man = bits & 0x7fffffu;
+  if (exp == 0xffu) return man ? bits_f32(bits | 0x00400000u) : x; /* NaN quieted, inf kept */
+  const int32_t e = (int32_t)exp - 127 + 15;                        /* biased half exponent */
+  if (e >= 31) return bits_f32(sign | 0x7f800000u);
+  uint32_t half;
+  if (e <= 0) {
+    if (e < -10) return bits_f32(sign); /* below half the smallest subnormal */
+    const uint32_t full = man | 0x800000u;
+    const int shift = 14 - e; /* 14 .. 24 */
+    half = full >> shift;
+    const uint32_t rem = full & ((1u << shift) - 1u), mid = 1u << (shift - 1);
+    if (rem > mid || (rem == mid && (half & 1u))) half++;
+  } else {
+    half = ((uint32_t)e << 10) | (man >> 13);
+    const uint32_t rem = man & 0x1fffu;
+    if (rem > 0x1000u || (rem == 0x1000u && (half & 1u))) half++; /* may carry into the exponent */
+  }
+  /* back to f32 */
+  const uint32_t he = (half >> 10) & 0x1fu, hm = half & 0x3ffu;
+  if (he == 31u) return bits_f32(sign | 0x7f800000u);
+  if (he == 0u) return (sign ? -1.0f : 1.0f) * (float)hm * 5.9604644775390625e-8f; /* hm * 2^-24 */
+  return bits_f32(sign | ((he + 112u) << 23) | (hm << 13));
+}
+
+double svod_oracle_round_f16(double x) { return (double)round_f16_f32((float)x); }
+
+/* The 16-bit type of the operand stream the restatements below round to: 1 bf16 (the default),
+ * 2 f16.  Set once before a run; the restatements only read it. */
+static int stream_dtype = 1;
+void svod_oracle_set_stream_dtype(int32_t which) { stream_dtype = which == 2 ? 2 : 1; }
+static inline float round_stream(float x) { return stream_dtype == 2 ? round_f16_f32(x) : round_bf16_f32(x); }
+
 uint16_t svod_oracle_bf16_bits(float x) { return (uint16_t)(f32_bits(round_bf16_f32(x)) >> 16); }
 
 /* tk/src/interp.rs TileOp::Cast with Round::Zero: the low 16 bits dropped. */
@@ -330,7 +367,7 @@ static void graph_slice(const void *ctxp, int32_t b, int32_t h) {
       const float *kj = kh + (int64_t)j * d;
       float s = 0.0f;
       if (bf)
-        for (int32_t dd = 0; dd < d; dd++) s += round_bf16_f32(qi[dd] * kj[dd]);
+        for (int32_t dd = 0; dd < d; dd++) s += round_stream(qi[dd] * kj[dd]);
       else
         for (int32_t dd = 0; dd < d; dd++) s += qi[dd] * kj[dd];
       s *= p->scale;
@@ -346,7 +383,7 @@ static void graph_slice(const void *ctxp, int32_t b, int32_t h) {
     }
     for (int32_t j = 0; j < tk; j++) {
       float w = keep[j] ? row[j] / sum : 0.0f;
-      row[j] = bf ? round_bf16_f32(w) : w;
+      row[j] = bf ? round_stream(w) : w;
     }
     for (int32_t dd = 0; dd < d; dd++) acc[dd] = 0.0f;
     for (int32_t j = 0; j < tk; j++) {
@@ -354,11 +391,11 @@ static void graph_slice(const void *ctxp, int32_t b, int32_t h) {
       if (w == 0.0f) continue; /* +0 products leave an f32 sum unchanged */
       const float *vj = vh + (int64_t)j * d;
       if (bf)
-        for (int32_t dd = 0; dd < d; dd++) acc[dd] += round_bf16_f32(w * vj[dd]);
+        for (int32_t dd = 0; dd < d; dd++) acc[dd] += round_stream(w * vj[dd]);
       else
         for (int32_t dd = 0; dd < d; dd++) acc[dd] += w * vj[dd];
     }
-    for (int32_t dd = 0; dd < d; dd++) oi[dd] = bf ? round_bf16_f32(acc[dd]) : acc[dd];
+    for (int32_t dd = 0; dd < d; dd++) oi[dd] = bf ? round_stream(acc[dd]) : acc[dd];
   }
   free(row);
   free(keep);
@@ -494,7 +531,7 @@ static void flash_slice(const void *ctxp, int32_t b, int32_t h) {
         for (int32_t cc = 0; cc < bkv; cc++) {
           const double e = r32(exp2(r32(s[(int64_t)r * bkv + cc] - m_new)));
           block_sum += e;
-          p16[(int64_t)r * bkv + cc] = bf ? (double)round_bf16_f32((float)e) : e;
+          p16[(int64_t)r * bkv + cc] = bf ? (double)round_stream((float)e) : e;
         }
         block_sum = r32(block_sum);
         l[r] = r32(r32(l[r] * corr) + block_sum);
@@ -547,7 +584,7 @@ static void flash_slice(const void *ctxp, int32_t b, int32_t h) {
       float *oi = c->out + ((int64_t)b * t + i) * stride + (int64_t)h * d;
       for (int32_t dd = 0; dd < d; dd++) {
         const float val = (float)r32(o[(int64_t)r * d + dd] / ll);
-        oi[dd] = bf ? round_bf16_f32(val) : val;
+        oi[dd] = bf ? round_stream(val) : val;
       }
     }
   }
@@ -641,7 +678,7 @@ int svod_oracle_heads_direct(int32_t batch, int32_t t, int32_t heads, int32_t kv
         }
         const int32_t width = which == 0 ? heads : kv_heads;
         float *dst = (which == 0 ? q : which == 1 ? k : v) + (((int64_t)b * t + i) * width + head) * d;
-        for (int32_t c = 0; c < d; c++) dst[c] = round_bf16_f32((float)x[c]);
+        for (int32_t c = 0; c < d; c++) dst[c] = round_stream((float)x[c]);
       }
   free(x);
   free(y);
@@ -696,8 +733,8 @@ int svod_oracle_heads_kernel(int32_t batch, int32_t t, int32_t heads, int32_t kv
             y1 = r32(c1 - s2);
             y2 = r32(s1 + c2);
           }
-          dst[c] = round_bf16_f32((float)y1);
-          dst[c + half] = round_bf16_f32((float)y2);
+          dst[c] = round_stream((float)y1);
+          dst[c + half] = round_stream((float)y2);
         }
       }
   return 0;
@@ -734,7 +771,7 @@ int svod_oracle_heads_graph(int32_t batch, int32_t t, int32_t heads, int32_t kv_
           for (int32_t c = 0; c < d; c++) ss += x[c] * x[c];
           const float mean = ss / (float)d;
           const float inv = 1.0f / sqrtf(mean + (float)eps);
-          for (int32_t c = 0; c < d; c++) x[c] = round_bf16_f32((x[c] * inv) * w[c]);
+          for (int32_t c = 0; c < d; c++) x[c] = round_stream((x[c] * inv) * w[c]);
         }
         const int32_t width = which == 0 ? heads : kv_heads;
         float *dst = (which == 0 ? q : which == 1 ? k : v) + (((int64_t)b * t + i) * width + head) * d;
@@ -743,8 +780,8 @@ int svod_oracle_heads_graph(int32_t batch, int32_t t, int32_t heads, int32_t kv_
           for (int32_t c = 0; c < half; c++) {
             const float cs = cos_t[row * half + c], sn = sin_t[row * half + c];
             const float x1 = x[c], x2 = x[c + half];
-            dst[c] = round_bf16_f32(round_bf16_f32(x1 * cs) - round_bf16_f32(x2 * sn));
-            dst[c + half] = round_bf16_f32(round_bf16_f32(x1 * sn) + round_bf16_f32(x2 * cs));
+            dst[c] = round_stream(round_stream(x1 * cs) - round_stream(x2 * sn));
+            dst[c + half] = round_stream(round_stream(x1 * sn) + round_stream(x2 * cs));
           }
         } else {
           memcpy(dst, x, sizeof(float) * (size_t)d);

@@ -48,6 +48,8 @@ namespace {
 #endif
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 typedef __attribute__((ext_vector_type(4))) short s16x4;
 typedef __attribute__((ext_vector_type(8))) short s16x8;
@@ -97,10 +99,28 @@ __device__ __forceinline__ float max3(float a, float b, float c) {
   return __builtin_fmaxf(__builtin_fmaxf(a, b), c);
 }
 
+// Two f32 values as a pair of the operands' 16-bit type, rounded to nearest even
+// (tk/src/interp.rs:37-50).
+template <bool F16>
 __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
   f32x2 f = {lo, hi};
-  bf16x2 b = __builtin_convertvector(f, bf16x2);
-  return __builtin_bit_cast(uint32_t, b);
+  if constexpr (F16) {
+    f16x2 h = __builtin_convertvector(f, f16x2);
+    return __builtin_bit_cast(uint32_t, h);
+  } else {
+    bf16x2 b = __builtin_convertvector(f, bf16x2);
+    return __builtin_bit_cast(uint32_t, b);
+  }
+}
+
+// D = A . B + C on the 32x32x16 atom of the operands' type: A 32 rows x 16, B 16 x 32 columns,
+// eight 16-bit values a lane each.
+template <bool F16>
+__device__ __forceinline__ f32x16 mma(const u32x4 &a, const u32x4 &b, const f32x16 &c) {
+  if constexpr (F16)
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
 }
 
 // `x` of this lane and of its partner in the other half-wave (lane l <-> l^32),
@@ -131,7 +151,7 @@ __device__ __forceinline__ i32x4 make_rsrc(const void *base, int64_t bytes) {
 }
 
 // Everything a wave carries through the key loop.
-template <int D, int NW>
+template <int D, int NW, bool F16>
 struct Wave {
   static constexpr int KS = D / 16;  // k-steps of the score product
   static constexpr int DB = D / 32;  // 32-row blocks of O^T
@@ -154,7 +174,7 @@ struct Wave {
   int k_src[CH], v_src[CH];  // global byte offsets of this lane's chunk in each fill
   int k_read[KS], v_read[DB];
   // state
-  bf16x8 qf[KS];
+  u32x4 qf[KS];
   f32x16 acc[DB];
   float m_run, l_run;
   int mask_next;
@@ -164,13 +184,13 @@ struct Wave {
 // it knows about as aliasing every later LDS read and would park the wave on the NEXT tile's
 // fills in the middle of the current tile.  The kernel waits for them itself (vmcnt(0) before
 // the barrier that ends a step).  m0 carries the LDS address of a wave instruction's 1 KiB.
-template <int D, int NW>
-__device__ __forceinline__ void fill_tile(const Wave<D, NW> &w, const uint8_t *base, int blk, int lds_at,
-                                          const int (&src)[Wave<D, NW>::CH]) {
+template <int D, int NW, bool F16>
+__device__ __forceinline__ void fill_tile(const Wave<D, NW, F16> &w, const uint8_t *base, int blk, int lds_at,
+                                          const int (&src)[Wave<D, NW, F16>::CH]) {
   const int64_t off = (int64_t)blk * kBkv * w.kv_row_bytes;
   const i32x4 r = make_rsrc(base + off, w.kv_bytes - off);
 #pragma unroll
-  for (int i = 0; i < Wave<D, NW>::CH; i++) {
+  for (int i = 0; i < Wave<D, NW, F16>::CH; i++) {
     const int j = w.wave + NW * i;
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
                  :
@@ -178,19 +198,19 @@ __device__ __forceinline__ void fill_tile(const Wave<D, NW> &w, const uint8_t *b
                  : "memory");
   }
 }
-template <int D, int NW>
-__device__ __forceinline__ void fill_k(const Wave<D, NW> &w, int blk, int slot) {
+template <int D, int NW, bool F16>
+__device__ __forceinline__ void fill_k(const Wave<D, NW, F16> &w, int blk, int slot) {
   fill_tile<D, NW>(w, w.k_base, blk, w.lds0 + slot * Tile<D>::kBytes, w.k_src);
 }
-template <int D, int NW>
-__device__ __forceinline__ void fill_v(const Wave<D, NW> &w, int blk, int slot) {
+template <int D, int NW, bool F16>
+__device__ __forceinline__ void fill_v(const Wave<D, NW, F16> &w, int blk, int slot) {
   fill_tile<D, NW>(w, w.v_base, blk, w.lds0 + (2 + slot) * Tile<D>::kBytes, w.v_src);
 }
 
 // A key mask row is read 64 keys (one per lane) a block, one block ahead: the load is issued
 // before that block's fills and is long back when the block's step needs it.
-template <int D, int NW>
-__device__ __forceinline__ int mask_lane(const Wave<D, NW> &w, int blk) {
+template <int D, int NW, bool F16>
+__device__ __forceinline__ int mask_lane(const Wave<D, NW, F16> &w, int blk) {
   const int key = blk * kBkv + w.lane;
   if (w.key_mask == nullptr || key >= w.tk) return 0;
   const int64_t at = w.mask_row + key;
@@ -199,18 +219,18 @@ __device__ __forceinline__ int mask_lane(const Wave<D, NW> &w, int blk) {
 
 // S^T = K . Q^T of the key block in K slot `slot`, as 32 scalars: sv[16kb + i] is the score of
 // key 32kb + 8(i/4) + 4g + i%4 (sub-registers of the two accumulators: no moves).
-template <int D, int NW>
-__device__ __forceinline__ void scores(const Wave<D, NW> &w, const uint8_t *smem, int slot, float (&sv)[32]) {
+template <int D, int NW, bool F16>
+__device__ __forceinline__ void scores(const Wave<D, NW, F16> &w, const uint8_t *smem, int slot, float (&sv)[32]) {
   using TL = Tile<D>;
   const uint8_t *ks_ = smem + slot * TL::kBytes;
   const f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
   f32x16 s0 = zero, s1 = zero;
 #pragma unroll
-  for (int ks = 0; ks < Wave<D, NW>::KS; ks++) {
+  for (int ks = 0; ks < Wave<D, NW, F16>::KS; ks++) {
     const u32x4 a0 = *reinterpret_cast<const u32x4 *>(ks_ + w.k_read[ks]);
     const u32x4 a1 = *reinterpret_cast<const u32x4 *>(ks_ + w.k_read[ks] + 32 * TL::kRowBytes);
-    s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a0), w.qf[ks], s0, 0, 0, 0);
-    s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a1), w.qf[ks], s1, 0, 0, 0);
+    s0 = mma<F16>(a0, w.qf[ks], s0);
+    s1 = mma<F16>(a1, w.qf[ks], s1);
   }
 #pragma unroll
   for (int i = 0; i < 16; i++) {
@@ -221,8 +241,8 @@ __device__ __forceinline__ void scores(const Wave<D, NW> &w, const uint8_t *smem
 
 // The wave-uniform part of block `blk`'s mask: bit j = key 64 blk + j is below the length and
 // kept by the key mask (`word` is this lane's key-mask element of the block).
-template <int D, int NW>
-__device__ __forceinline__ uint64_t uniform_bits(const Wave<D, NW> &w, int blk, int word) {
+template <int D, int NW, bool F16>
+__device__ __forceinline__ uint64_t uniform_bits(const Wave<D, NW, F16> &w, int blk, int word) {
   const int k0 = blk * kBkv;
   uint64_t kbits = ~0ull;
   if (w.key_mask != nullptr) kbits = __builtin_amdgcn_ballot_w64(word != 0);
@@ -231,15 +251,15 @@ __device__ __forceinline__ uint64_t uniform_bits(const Wave<D, NW> &w, int blk, 
 }
 
 // Whether a mask edge crosses block `blk` for this wave (L698-733).
-template <int D, int NW, bool CAUSAL>
-__device__ __forceinline__ bool on_edge(const Wave<D, NW> &w, int blk, uint64_t kbits) {
+template <int D, int NW, bool CAUSAL, bool F16>
+__device__ __forceinline__ bool on_edge(const Wave<D, NW, F16> &w, int blk, uint64_t kbits) {
   return kbits != ~0ull || (CAUSAL && (blk * kBkv + kBkv - 1 > w.wave_first_row));
 }
 
 // Scales (a non-positive scale only) and masks (L641-697) the scores of block `blk`: hidden
 // scores become -inf.  `kbits` is the uniform word; causality adds a per-lane one.
-template <int D, int NW, bool CAUSAL>
-__device__ __forceinline__ void mask_scores(const Wave<D, NW> &w, int blk, uint64_t kbits, float (&sv)[32]) {
+template <int D, int NW, bool CAUSAL, bool F16>
+__device__ __forceinline__ void mask_scores(const Wave<D, NW, F16> &w, int blk, uint64_t kbits, float (&sv)[32]) {
   const int k0 = blk * kBkv;
   uint64_t mine = kbits;
   if (CAUSAL && (k0 + kBkv - 1 > w.wave_first_row)) {
@@ -271,6 +291,7 @@ __device__ __forceinline__ float row_max(const float (&sv)[32]) {
 
 // Half a block's probabilities: p = 2^(s*unit - m*unit) for 16 scores, summed unrounded in
 // four chains, then held as bf16 (L432-444).
+template <bool F16>
 __device__ __forceinline__ void probabilities(const float *sv, float unit, float m_exp, float (&bs)[4],
                                               uint32_t *pk) {
 #pragma unroll
@@ -283,26 +304,26 @@ __device__ __forceinline__ void probabilities(const float *sv, float unit, float
     bs[1] += p1;
     bs[2] += p2;
     bs[3] += p3;
-    pk[i / 2] = pack2(p0, p1);
-    pk[i / 2 + 1] = pack2(p2, p3);
+    pk[i / 2] = pack2<F16>(p0, p1);
+    pk[i / 2 + 1] = pack2<F16>(p2, p3);
   }
 }
 
 // O^T += V^T . P^T over 32 keys (half a block): chunks c of 16 keys, fragment registers 4c..4c+3.
-template <int D, int NW>
-__device__ __forceinline__ void accumulate(Wave<D, NW> &w, const uint8_t *vs_, int half, const uint32_t *pk) {
+template <int D, int NW, bool F16>
+__device__ __forceinline__ void accumulate(Wave<D, NW, F16> &w, const uint8_t *vs_, int half, const uint32_t *pk) {
   using TL = Tile<D>;
 #pragma unroll
   for (int c = 0; c < 2; c++) {
     const u32x4 pw = {pk[4 * c], pk[4 * c + 1], pk[4 * c + 2], pk[4 * c + 3]};
-    const bf16x8 pf = __builtin_bit_cast(bf16x8, pw);
+
 #pragma unroll
-    for (int db = 0; db < Wave<D, NW>::DB; db++) {
+    for (int db = 0; db < Wave<D, NW, F16>::DB; db++) {
       const uint8_t *at = vs_ + w.v_read[db] + (32 * half + 16 * c) * TL::kRowBytes;
       const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_PTR(s16x4))(at));
       const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_PTR(s16x4))(at + 8 * TL::kRowBytes));
       const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-      w.acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, both), pf, w.acc[db], 0, 0, 0);
+      w.acc[db] = mma<F16>(__builtin_bit_cast(u32x4, both), pw, w.acc[db]);
     }
   }
 }
@@ -310,8 +331,8 @@ __device__ __forceinline__ void accumulate(Wave<D, NW> &w, const uint8_t *vs_, i
 // The running maximum's update for a block whose row maximum is `bm`: the lazy rescale of
 // L418-431, and the O^T rescale that a wave skips when all its rows kept their maximum
 // (L56-59).  Returns the exponent's offset m*unit; `corr` is the correction of l.
-template <int D, int NW>
-__device__ __forceinline__ float adopt_maximum(Wave<D, NW> &w, float bm, float &corr) {
+template <int D, int NW, bool F16>
+__device__ __forceinline__ float adopt_maximum(Wave<D, NW, F16> &w, float bm, float &corr) {
   const float m_max = __builtin_fmaxf(w.m_run, bm);
   const bool grows = w.limit < (m_max - w.m_run);
   const float m_new = grows ? m_max : w.m_run;
@@ -319,7 +340,7 @@ __device__ __forceinline__ float adopt_maximum(Wave<D, NW> &w, float bm, float &
   w.m_run = m_new;
   if (__builtin_amdgcn_ballot_w64(corr != 1.0f) != 0) {
 #pragma unroll
-    for (int db = 0; db < Wave<D, NW>::DB; db++) w.acc[db] *= corr;
+    for (int db = 0; db < Wave<D, NW, F16>::DB; db++) w.acc[db] *= corr;
   }
   return m_new * w.unit;
 }
@@ -330,12 +351,13 @@ __device__ __forceinline__ void pin(float &x) { asm volatile("" : "+v"(x)); }
 
 // One unit of the exponentials: two scores to two probabilities (p = 2^(s*unit - m*unit)),
 // each added unrounded to a row-sum chain, the pair held as bf16 (L432-444).
+template <bool F16>
 __device__ __forceinline__ uint32_t p_unit(float s_a, float s_b, float unit, float m_exp, float &sum_a, float &sum_b) {
   const float pa = fast_exp2(__builtin_fmaf(s_a, unit, -m_exp));
   const float pb = fast_exp2(__builtin_fmaf(s_b, unit, -m_exp));
   sum_a += pa;
   sum_b += pb;
-  return pack2(pa, pb);
+  return pack2<F16>(pa, pb);
 }
 
 // The hot step: block `blk` (parity PAR = blk & 1: V(blk) in V slot PAR, K(blk+1) in K slot
@@ -349,11 +371,11 @@ __device__ __forceinline__ uint32_t p_unit(float s_a, float s_b, float unit, flo
 // never waits for the VALU's whole job.  2 KS slots compute S(blk+1) beside the exponentials
 // of keys 0..31; 2 DB slots add P V of keys 0..31 beside the exponentials of keys 32..63;
 // 2 DB slots add P V of keys 32..63 beside the row maximum of S(blk+1).
-template <int D, int NW, int PAR>
-__device__ __forceinline__ void hot_step(Wave<D, NW> &w, const uint8_t *smem, int blk, const float (&sv)[32],
+template <int D, int NW, int PAR, bool F16>
+__device__ __forceinline__ void hot_step(Wave<D, NW, F16> &w, const uint8_t *smem, int blk, const float (&sv)[32],
                                          float (&nv)[32], float &bm) {
   using TL = Tile<D>;
-  constexpr int KS = Wave<D, NW>::KS, DB = Wave<D, NW>::DB;
+  constexpr int KS = Wave<D, NW, F16>::KS, DB = Wave<D, NW, F16>::DB;
   constexpr int NQK = 2 * KS;  // score slots
   constexpr int NPV = 4 * DB;  // P V slots, half of them per 32 keys
   const uint8_t *ks_ = smem + (PAR ^ 1) * TL::kBytes;
@@ -388,18 +410,17 @@ __device__ __forceinline__ void hot_step(Wave<D, NW> &w, const uint8_t *smem, in
   // ---- S(blk+1) beside the probabilities of keys 0..31 (8 units over NQK slots).
 #pragma unroll
   for (int i = 0; i < NQK; i++) {
-    const bf16x8 a = __builtin_bit_cast(bf16x8, kf[i & 3]);
     if (i & 1)
-      s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, w.qf[i >> 1], s1, 0, 0, 0);
+      s1 = mma<F16>(kf[i & 3], w.qf[i >> 1], s1);
     else
-      s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, w.qf[i >> 1], s0, 0, 0, 0);
+      s0 = mma<F16>(kf[i & 3], w.qf[i >> 1], s0);
     if (i + 4 < NQK)
       kf[i & 3] = k_frag(i + 4);
     else
       vf[(i + 4 - NQK) & 3] = v_frag(i + 4 - NQK);
 #pragma unroll
     for (int u = 8 * i / NQK; u < 8 * (i + 1) / NQK; u++)
-      pk[u] = p_unit(sv[2 * u], sv[2 * u + 1], w.unit, m_exp, bs[(2 * u) & 3], bs[(2 * u + 1) & 3]);
+      pk[u] = p_unit<F16>(sv[2 * u], sv[2 * u + 1], w.unit, m_exp, bs[(2 * u) & 3], bs[(2 * u + 1) & 3]);
     if (8 * i / NQK < 8 * (i + 1) / NQK) {
 #pragma unroll
       for (int x = 0; x < 4; x++) pin(bs[x]);
@@ -418,13 +439,12 @@ __device__ __forceinline__ void hot_step(Wave<D, NW> &w, const uint8_t *smem, in
   for (int j = 0; j < NPV; j++) {
     const int c = j / DB;
     const u32x4 pw = {pk[4 * c], pk[4 * c + 1], pk[4 * c + 2], pk[4 * c + 3]};
-    w.acc[j % DB] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vf[j & 3]),
-                                                           __builtin_bit_cast(bf16x8, pw), w.acc[j % DB], 0, 0, 0);
+    w.acc[j % DB] = mma<F16>(__builtin_bit_cast(u32x4, vf[j & 3]), pw, w.acc[j % DB]);
     if (j + 4 < NPV) vf[j & 3] = v_frag(j + 4);
     if (j < NPV / 2) {
 #pragma unroll
       for (int u = 8 + 16 * j / NPV; u < 8 + 16 * (j + 1) / NPV; u++)
-        pk[u] = p_unit(sv[2 * u], sv[2 * u + 1], w.unit, m_exp, bs[(2 * u) & 3], bs[(2 * u + 1) & 3]);
+        pk[u] = p_unit<F16>(sv[2 * u], sv[2 * u + 1], w.unit, m_exp, bs[(2 * u) & 3], bs[(2 * u + 1) & 3]);
 #pragma unroll
       for (int x = 0; x < 4; x++) pin(bs[x]);
     } else {
@@ -452,8 +472,8 @@ __device__ __forceinline__ void hot_step(Wave<D, NW> &w, const uint8_t *smem, in
 // The general step, for the blocks at the edges: any block, a next block or none, masks, any
 // scale.  Slots are picked at run time.  `sv` holds the masked S(blk) and `bm` its row maximum;
 // on exit they hold block blk+1's (when this wave has one).
-template <int D, int NW, bool CAUSAL>
-__device__ __forceinline__ void edge_step(Wave<D, NW> &w, const uint8_t *smem, int blk, int my_end, float (&sv)[32],
+template <int D, int NW, bool CAUSAL, bool F16>
+__device__ __forceinline__ void edge_step(Wave<D, NW, F16> &w, const uint8_t *smem, int blk, int my_end, float (&sv)[32],
                                           float &bm) {
   using TL = Tile<D>;
   const int par = blk & 1;
@@ -470,8 +490,8 @@ __device__ __forceinline__ void edge_step(Wave<D, NW> &w, const uint8_t *smem, i
   const uint8_t *vs_ = smem + (2 + par) * TL::kBytes;
   float bs[4] = {0.0f, 0.0f, 0.0f, 0.0f};
   uint32_t pk[16];
-  probabilities(sv, w.unit, m_exp, bs, pk);
-  probabilities(sv + 16, w.unit, m_exp, bs, pk + 8);
+  probabilities<F16>(sv, w.unit, m_exp, bs, pk);
+  probabilities<F16>(sv + 16, w.unit, m_exp, bs, pk + 8);
   accumulate<D, NW>(w, vs_, 0, pk);
   accumulate<D, NW>(w, vs_, 1, pk + 8);
   w.l_run = w.l_run * corr + ((bs[0] + bs[1]) + (bs[2] + bs[3]));
@@ -489,8 +509,8 @@ __device__ __forceinline__ void edge_step(Wave<D, NW> &w, const uint8_t *smem, i
 }
 
 // A step of a wave with nothing to compute: fills and the barrier only.
-template <int D, int NW>
-__device__ __forceinline__ void idle_step(Wave<D, NW> &w, int blk) {
+template <int D, int NW, bool F16>
+__device__ __forceinline__ void idle_step(Wave<D, NW, F16> &w, int blk) {
   const int par = blk & 1;
   if (blk + 1 < w.end) fill_v<D, NW>(w, blk + 1, par ^ 1);
   if (blk + 2 < w.end) fill_k<D, NW>(w, blk + 2, par);
@@ -520,7 +540,7 @@ struct Splits {
   uint32_t nbatch;
 };
 
-template <int D, int NW, bool CAUSAL, bool SPLIT>
+template <int D, int NW, bool CAUSAL, bool SPLIT, bool F16>
 __global__ __launch_bounds__(NW * 64, D == 64 ? 3 : 2) void flash_fwd_kernel(
     uint32_t unit_size, uint32_t unit_rcp, uint32_t nqt_u, uint32_t nqt_rcp, uint32_t kvh_u, uint32_t kvh_rcp,
     uint32_t units, uint32_t heads_group, const void *__restrict__ key_lens, const uint16_t *__restrict__ q, int32_t t,
@@ -539,7 +559,7 @@ __global__ __launch_bounds__(NW * 64, D == 64 ? 3 : 2) void flash_fwd_kernel(
   const int tk = (int)(tk_lens64 & 0x7fffffffu);
   const bool lens_i64 = (tk_lens64 >> 31) != 0;
   using TL = Tile<D>;
-  using W = Wave<D, NW>;
+  using W = Wave<D, NW, F16>;
   constexpr int BQ = NW * kWaveRows;
   constexpr int KS = W::KS, DB = W::DB, CH = W::CH;
   static_assert(TL::kInstrs % NW == 0, "the tile fills in whole wave instructions per wave");
@@ -592,7 +612,7 @@ __global__ __launch_bounds__(NW * 64, D == 64 ? 3 : 2) void flash_fwd_kernel(
     for (int ks = 0; ks < KS; ks++) {
       u32x4 x = {0, 0, 0, 0};
       if (row < t) x = *reinterpret_cast<const u32x4 *>(q_ptr + ks * 16);
-      w.qf[ks] = __builtin_bit_cast(bf16x8, x);
+      w.qf[ks] = x;
     }
   }
 
@@ -758,8 +778,8 @@ __global__ __launch_bounds__(NW * 64, D == 64 ? 3 : 2) void flash_fwd_kernel(
 #pragma unroll
       for (int c = 0; c < 4; c++) {
         u32x2 x;
-        x[0] = pack2(w.acc[db][4 * c] * inv, w.acc[db][4 * c + 1] * inv);
-        x[1] = pack2(w.acc[db][4 * c + 2] * inv, w.acc[db][4 * c + 3] * inv);
+        x[0] = pack2<F16>(w.acc[db][4 * c] * inv, w.acc[db][4 * c + 1] * inv);
+        x[1] = pack2<F16>(w.acc[db][4 * c + 2] * inv, w.acc[db][4 * c + 3] * inv);
         *reinterpret_cast<u32x2 *>(o_ptr + 32 * db + 8 * c) = x;
       }
     }
@@ -767,7 +787,7 @@ __global__ __launch_bounds__(NW * 64, D == 64 ? 3 : 2) void flash_fwd_kernel(
 #endif  // __HIP_DEVICE_COMPILE__
 }
 
-template <int D, int NW, bool CAUSAL, bool SPLIT>
+template <int D, int NW, bool CAUSAL, bool SPLIT, bool F16>
 hipError_t launch(const AttnArgs &a, hipStream_t stream) {
   using TL = Tile<D>;
   constexpr int BQ = NW * kWaveRows;
@@ -781,7 +801,7 @@ hipError_t launch(const AttnArgs &a, hipStream_t stream) {
   const int64_t kv_row = a.kv_row_elems > 0 ? a.kv_row_elems : (int64_t)a.kv_heads * a.d;
   // The fills address a (batch, kv head)'s rows with 32-bit byte offsets.
   if ((int64_t)a.tk * kv_row * 2 > 0x7fffffffLL || q_row > 0x7fffffffLL) return hipErrorInvalidValue;
-  auto kernel = flash_fwd_kernel<D, NW, CAUSAL, SPLIT>;
+  auto kernel = flash_fwd_kernel<D, NW, CAUSAL, SPLIT, F16>;
   // The LDS ring is above the default limit of a launch: one attribute call per instantiation
   // and device, from whichever thread gets there first (a second call is harmless).
   static std::atomic<uint64_t> configured{0};  // a bit per device ordinal, devices past 63 always ask
@@ -829,10 +849,16 @@ hipError_t launch(const AttnArgs &a, hipStream_t stream) {
   return hipGetLastError();
 }
 
+template <int D, bool F16>
+hipError_t launch_t(const AttnArgs &a, hipStream_t stream) {
+  if (a.splits > 1)
+    return a.causal ? launch<D, 4, true, true, F16>(a, stream) : launch<D, 4, false, true, F16>(a, stream);
+  return a.causal ? launch<D, 4, true, false, F16>(a, stream) : launch<D, 4, false, false, F16>(a, stream);
+}
+
 template <int D>
 hipError_t launch_d(const AttnArgs &a, hipStream_t stream) {
-  if (a.splits > 1) return a.causal ? launch<D, 4, true, true>(a, stream) : launch<D, 4, false, true>(a, stream);
-  return a.causal ? launch<D, 4, true, false>(a, stream) : launch<D, 4, false, false>(a, stream);
+  return a.f16 ? launch_t<D, true>(a, stream) : launch_t<D, false>(a, stream);
 }
 
 }  // namespace
@@ -840,9 +866,16 @@ hipError_t launch_d(const AttnArgs &a, hipStream_t stream) {
 bool attention_supports(int32_t d) { return d == 64 || d == 128; }
 
 const char *attention_config(const AttnArgs &a) {
-  (void)a;
-  return "FaCfg { bq: 128, bkv: 64, stages: 2, splits: 1, forms: { raw_max, skip_rescale }, warp_rows: 32, core: "
-         "mfma_f32_32x32x16_bf16 }";
+  static const char *const kCfg[2][2] = {
+      {"FaCfg { bq: 128, bkv: 64, stages: 2, splits: 1, forms: { raw_max, skip_rescale }, warp_rows: 32, core: "
+       "mfma_f32_32x32x16_bf16 }",
+       "FaCfg { bq: 128, bkv: 64, stages: 2, splits: n, forms: { raw_max, skip_rescale }, warp_rows: 32, core: "
+       "mfma_f32_32x32x16_bf16 }"},
+      {"FaCfg { bq: 128, bkv: 64, stages: 2, splits: 1, forms: { raw_max, skip_rescale }, warp_rows: 32, core: "
+       "mfma_f32_32x32x16_f16 }",
+       "FaCfg { bq: 128, bkv: 64, stages: 2, splits: n, forms: { raw_max, skip_rescale }, warp_rows: 32, core: "
+       "mfma_f32_32x32x16_f16 }"}};
+  return kCfg[a.f16 ? 1 : 0][a.splits > 1 ? 1 : 0];
 }
 
 hipError_t launch_attention(const AttnArgs &a, hipStream_t stream) {

@@ -20,13 +20,19 @@ typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 
 constexpr int kThreads = 256;
 
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
+
+// Round to nearest even into the output's type.
+template <bool F16>
 __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
   f32x2 f = {lo, hi};
-  bf16x2 b = __builtin_convertvector(f, bf16x2);  // round to nearest even
-  return __builtin_bit_cast(uint32_t, b);
+  if constexpr (F16)
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, f16x2));
+  else
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
 }
 
-template <int D>
+template <int D, bool F16>
 __global__ __launch_bounds__(kThreads) void combine_kernel(const float *__restrict__ o_part,
                                                            const float *__restrict__ m_part,
                                                            const float *__restrict__ l_part, uint16_t *__restrict__ o,
@@ -52,18 +58,18 @@ __global__ __launch_bounds__(kThreads) void combine_kernel(const float *__restri
   }
   const float ll = l == 0.0f ? 1.0f : l;
   u32x2 out;
-  out[0] = pack2(acc[0] / ll, acc[1] / ll);
-  out[1] = pack2(acc[2] / ll, acc[3] / ll);
+  out[0] = pack2<F16>(acc[0] / ll, acc[1] / ll);
+  out[1] = pack2<F16>(acc[2] / ll, acc[3] / ll);
   *(reinterpret_cast<u32x2 *>(o + row * D) + part) = out;
 }
 
-template <int D>
+template <int D, bool F16>
 hipError_t launch(const CombineArgs &a, hipStream_t stream) {
   const int64_t threads = a.rows * (D / 4);
   if (threads == 0) return hipSuccess;
   const int64_t blocks = (threads + kThreads - 1) / kThreads;
   if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;
-  hipLaunchKernelGGL(combine_kernel<D>, dim3((uint32_t)blocks), dim3(kThreads), 0, stream, a.o_part, a.m_part,
+  hipLaunchKernelGGL((combine_kernel<D, F16>), dim3((uint32_t)blocks), dim3(kThreads), 0, stream, a.o_part, a.m_part,
                      a.l_part, (uint16_t *)a.o, a.rows, a.splits);
   return hipGetLastError();
 }
@@ -73,8 +79,8 @@ hipError_t launch(const CombineArgs &a, hipStream_t stream) {
 hipError_t launch_combine(const CombineArgs &a, hipStream_t stream) {
   if (a.splits < 1) return hipErrorInvalidValue;
   switch (a.d) {
-    case 64: return launch<64>(a, stream);
-    case 128: return launch<128>(a, stream);
+    case 64: return a.f16 ? launch<64, true>(a, stream) : launch<64, false>(a, stream);
+    case 128: return a.f16 ? launch<128, true>(a, stream) : launch<128, false>(a, stream);
     default: return hipErrorInvalidValue;
   }
 }

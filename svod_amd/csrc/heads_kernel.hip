@@ -38,11 +38,34 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
   return to_bf16_bits(lo) | (to_bf16_bits(hi) << 16);
 }
 
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+
+// Eight 16-bit values of the operands' type, widened exactly.
+template <bool F16>
 __device__ __forceinline__ void widen(const u32x4 &w, float (&x)[8]) {
 #pragma unroll
   for (int i = 0; i < 4; i++) {
-    x[2 * i] = bf16_lo(w[i]);
-    x[2 * i + 1] = bf16_hi(w[i]);
+    if constexpr (F16) {
+      const uint32_t pair = w[i];  // a copy: the cast below wants an object of its own, not a vector's element
+      const f32x2 f = __builtin_convertvector(__builtin_bit_cast(f16x2, pair), f32x2);
+      x[2 * i] = f[0];
+      x[2 * i + 1] = f[1];
+    } else {
+      x[2 * i] = bf16_lo(w[i]);
+      x[2 * i + 1] = bf16_hi(w[i]);
+    }
+  }
+}
+
+// Two f32 values rounded to the operands' type, nearest even (tk/src/interp.rs:37-50).
+template <bool F16>
+__device__ __forceinline__ uint32_t narrow(float lo, float hi) {
+  if constexpr (F16) {
+    const f32x2 f = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, f16x2));
+  } else {
+    return pack_bf16(lo, hi);
   }
 }
 
@@ -71,7 +94,7 @@ struct Div64 {
 // and every byte is touched once, so loads and stores are marked non-temporal.
 constexpr int kItems = 1;
 
-template <int D, typename Div>
+template <int D, typename Div, bool F16>
 __global__ __launch_bounds__(kThreads) void heads_kernel(const uint16_t *__restrict__ qkv,
                                                          const uint16_t *__restrict__ q_w,
                                                          const uint16_t *__restrict__ k_w,
@@ -127,8 +150,8 @@ __global__ __launch_bounds__(kThreads) void heads_kernel(const uint16_t *__restr
     // Slots are uniform across the lanes of a slot, not across the wave: the
     // exchanges below run for every lane, the arithmetic is selected per lane.
     float y1[8], y2[8];
-    widen(w1[u], y1);
-    widen(w2[u], y2);
+    widen<F16>(w1[u], y1);
+    widen<F16>(w2[u], y2);
     float sum = 0.0f;
 #pragma unroll
     for (int i = 0; i < 8; i++) sum += y1[i] * y1[i] + y2[i] * y2[i];
@@ -140,8 +163,8 @@ __global__ __launch_bounds__(kThreads) void heads_kernel(const uint16_t *__restr
       const u32x4 g1 = *reinterpret_cast<const u32x4 *>(weight + part * 8);
       const u32x4 g2 = *reinterpret_cast<const u32x4 *>(weight + kHalf + part * 8);
       float a1[8], a2[8];
-      widen(g1, a1);
-      widen(g2, a2);
+      widen<F16>(g1, a1);
+      widen<F16>(g2, a2);
 #pragma unroll
       for (int i = 0; i < 8; i++) {
         y1[i] = (y1[i] * inv) * a1[i];
@@ -153,8 +176,8 @@ __global__ __launch_bounds__(kThreads) void heads_kernel(const uint16_t *__restr
       const u32x4 cw = *reinterpret_cast<const u32x4 *>(cos_t + (int64_t)trow * kHalf + part * 8);
       const u32x4 sw = *reinterpret_cast<const u32x4 *>(sin_t + (int64_t)trow * kHalf + part * 8);
       float c[8], s[8];
-      widen(cw, c);
-      widen(sw, s);
+      widen<F16>(cw, c);
+      widen<F16>(sw, s);
 #pragma unroll
       for (int i = 0; i < 8; i++) {
         const float r1 = y1[i] * c[i] - y2[i] * s[i];
@@ -168,8 +191,8 @@ __global__ __launch_bounds__(kThreads) void heads_kernel(const uint16_t *__restr
     if (weight != nullptr || rotate) {
 #pragma unroll
       for (int i = 0; i < 4; i++) {
-        o1[i] = pack_bf16(y1[2 * i], y1[2 * i + 1]);
-        o2[i] = pack_bf16(y2[2 * i], y2[2 * i + 1]);
+        o1[i] = narrow<F16>(y1[2 * i], y1[2 * i + 1]);
+        o2[i] = narrow<F16>(y2[2 * i], y2[2 * i + 1]);
       }
     } else {
       o1 = w1[u];  // untouched slots (v, or q/k with neither norm nor rope) keep their bits
@@ -180,7 +203,7 @@ __global__ __launch_bounds__(kThreads) void heads_kernel(const uint16_t *__restr
   }
 }
 
-template <int D>
+template <int D, bool F16>
 hipError_t launch(const HeadsArgs &a, hipStream_t stream) {
   constexpr int kLanes = D / 16;
   const int64_t slots = a.heads + 2 * a.kv_heads;
@@ -194,13 +217,13 @@ hipError_t launch(const HeadsArgs &a, hipStream_t stream) {
   if (blocks * per_block < 0xffffffffLL) {
     auto rcp = [](uint32_t d) { return d == 1 ? 0xffffffffu : (uint32_t)((1ull << 32) / d); };
     const Div32 by_slots = {(uint32_t)slots, rcp((uint32_t)slots)}, by_t = {(uint32_t)t, rcp((uint32_t)t)};
-    hipLaunchKernelGGL((heads_kernel<D, Div32>), dim3((uint32_t)blocks), dim3(kThreads), 0, stream,
+    hipLaunchKernelGGL((heads_kernel<D, Div32, F16>), dim3((uint32_t)blocks), dim3(kThreads), 0, stream,
                        (const uint16_t *)a.qkv, (const uint16_t *)a.q_w, (const uint16_t *)a.k_w,
                        (const uint16_t *)a.cos, (const uint16_t *)a.sin, (uint16_t *)a.q, (uint16_t *)a.k,
                        (uint16_t *)a.v, items, by_slots, by_t, a.heads, a.kv_heads, a.eps, a.rope);
   } else {
     const Div64 by_slots = {slots, 0}, by_t = {t, 0};
-    hipLaunchKernelGGL((heads_kernel<D, Div64>), dim3((uint32_t)blocks), dim3(kThreads), 0, stream,
+    hipLaunchKernelGGL((heads_kernel<D, Div64, F16>), dim3((uint32_t)blocks), dim3(kThreads), 0, stream,
                        (const uint16_t *)a.qkv, (const uint16_t *)a.q_w, (const uint16_t *)a.k_w,
                        (const uint16_t *)a.cos, (const uint16_t *)a.sin, (uint16_t *)a.q, (uint16_t *)a.k,
                        (uint16_t *)a.v, items, by_slots, by_t, a.heads, a.kv_heads, a.eps, a.rope);
@@ -212,15 +235,20 @@ hipError_t launch(const HeadsArgs &a, hipStream_t stream) {
 
 bool heads_supports(int32_t d) { return d == 16 || d == 32 || d == 64 || d == 128 || d == 256; }
 
-hipError_t launch_heads(const HeadsArgs &a, hipStream_t stream) {
+template <bool F16>
+static hipError_t launch_any(const HeadsArgs &a, hipStream_t stream) {
   switch (a.d) {
-    case 16: return launch<16>(a, stream);
-    case 32: return launch<32>(a, stream);
-    case 64: return launch<64>(a, stream);
-    case 128: return launch<128>(a, stream);
-    case 256: return launch<256>(a, stream);
+    case 16: return launch<16, F16>(a, stream);
+    case 32: return launch<32, F16>(a, stream);
+    case 64: return launch<64, F16>(a, stream);
+    case 128: return launch<128, F16>(a, stream);
+    case 256: return launch<256, F16>(a, stream);
     default: return hipErrorInvalidValue;
   }
+}
+
+hipError_t launch_heads(const HeadsArgs &a, hipStream_t stream) {
+  return a.f16 ? launch_any<true>(a, stream) : launch_any<false>(a, stream);
 }
 
 }  // namespace svodk

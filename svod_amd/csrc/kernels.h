@@ -19,6 +19,7 @@ struct HeadsArgs {
   int32_t t, heads, kv_heads, d;
   float eps;
   int32_t rope;  // 0 none, 1 tables by position [t, d/2], 2 by token [rows, d/2]
+  int32_t f16;   // every 16-bit operand is f16, not bf16
 };
 hipError_t launch_heads(const HeadsArgs &a, hipStream_t stream);
 // Head sizes the prologue kernel is built for.
@@ -38,6 +39,7 @@ struct AttnArgs {
   int32_t t, tk, heads, kv_heads, d;
   int32_t causal;
   float scale;
+  int32_t f16;  // the operands are f16, not bf16
   // Key splits (FaCfg::splits, tk/src/kernels/attention.rs:19-21, 487-492): with splits > 1 each
   // split writes its partial state instead of `o`: o_part [splits, batch, t, heads, d],
   // m_part and l_part [splits, batch, t, heads], all f32; launch_combine merges them.
@@ -52,9 +54,10 @@ hipError_t launch_attention(const AttnArgs &a, hipStream_t stream);
 // combine_splits: tk/src/kernels/attention.rs:948-1014.
 struct CombineArgs {
   const float *o_part, *m_part, *l_part;
-  void *o;       // [rows, d] bf16
+  void *o;       // [rows, d] bf16 or f16
   int64_t rows;  // batch * t * heads
   int32_t d, splits;
+  int32_t f16;
 };
 hipError_t launch_combine(const CombineArgs &a, hipStream_t stream);
 bool attention_supports(int32_t d);

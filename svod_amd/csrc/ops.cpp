@@ -157,7 +157,7 @@ bool current_device_has_kernels() {
 
 // ---- shape gates (tk/src/ops/shape.rs).
 // gate (L92-99): a target with kernels, every operand the same 16-bit type the
-// target has a matrix core for.  This library's kernels are bf16.
+// target has a matrix core for: gfx950 has one for bf16 and for f16, and both have kernels here.
 int gate(bool has_target, const int32_t *dtypes, int n) {
   if (!has_target) return SVODK_GRAPH_TARGET;
   if (n <= 0) return SVODK_GRAPH_DTYPE;
@@ -165,9 +165,6 @@ int gate(bool has_target, const int32_t *dtypes, int n) {
   if (!(first == SVODK_BF16 || first == SVODK_F16)) return SVODK_GRAPH_DTYPE;
   for (int i = 0; i < n; i++)
     if (dtypes[i] != first) return SVODK_GRAPH_DTYPE;
-  // f16 has a matrix core on gfx950 but no kernel in this library: "another
-  // type without a kernel on the target" (shape.rs:30-31).
-  if (first != SVODK_BF16) return SVODK_GRAPH_DTYPE;
   return 0;
 }
 
@@ -375,6 +372,7 @@ static int attend(const svodk_tensor *q, const svodk_tensor *k, const svodk_tens
   a.causal = opts->causal != 0;
   // L230: the default scale is 1/sqrt(D) in f32.
   a.scale = opts->has_scale ? opts->scale : 1.0f / std::sqrt((float)d);
+  a.f16 = q->dtype == SVODK_F16;
   if (packed != nullptr) a.q_row_elems = a.kv_row_elems = (heads + 2 * kv_heads) * d;
   // L280-302: key splits.  The partial tensors live in the caller's workspace.
   a.splits = split_count(opts->splits, tk);
@@ -404,6 +402,7 @@ static int attend(const svodk_tensor *q, const svodk_tensor *k, const svodk_tens
     c.rows = (int64_t)a.batch * t * heads;
     c.d = a.d;
     c.splits = a.splits;
+    c.f16 = a.f16;
     ran(op, "combine_splits", "NormCfg { br: 4 }");
     e = svodk::launch_combine(c, (hipStream_t)hip_stream);
     if (e != hipSuccess) return fail(SVODK_ERR_LAUNCH, "%s: %s", op, hipGetErrorString(e));
@@ -564,6 +563,7 @@ int svodk_heads(const svodk_tensor *qkv, const svodk_qkv *opts, const svodk_tens
   a.d = (int32_t)d;
   a.eps = (float)opts->eps;
   a.rope = opts->cos ? (per_batch ? 2 : 1) : 0;
+  a.f16 = qkv->dtype == SVODK_F16;
   ran(op, "heads", "NormCfg { lanes_per_head: d/16, block: 256 }");
   const hipError_t e = svodk::launch_heads(a, (hipStream_t)hip_stream);
   if (e != hipSuccess) return fail(SVODK_ERR_LAUNCH, "%s: %s", op, hipGetErrorString(e));

@@ -64,9 +64,11 @@ def test_an_empty_dim_keeps_the_graph():
     assert svod_amd.plan_heads(True, [BF16], [2, 0, 768], 64) == Fallback.Shape
 
 
-def test_f16_has_no_kernel_here():
-    """The reference runs f16 on its kernels; this library is bf16 only and says Dtype."""
-    assert svod_amd.plan_attention(True, [F16] * 3, [2, 100, 8, 64], [2, 37, 2, 64]) == Fallback.Dtype
+def test_f16_plans_like_bf16():
+    """tk/src/ops/shape.rs:92-99: either 16-bit float type takes the kernel, one type per call."""
+    assert svod_amd.plan_attention(True, [F16] * 3, [2, 100, 8, 64], [2, 37, 2, 64]) is None
+    assert svod_amd.plan_attention(True, [F16, BF16, F16], [2, 100, 8, 64], [2, 37, 2, 64]) == Fallback.Dtype
+    assert svod_amd.plan_heads(True, [F16], [2, 100, 12 * 64], 64) is None
 
 
 # ---- ops_plan.rs:1465-1487 (heads_plan and friends)

@@ -343,3 +343,33 @@ def test_a_hand_merged_pair_of_halves_is_what_the_split_program_returns():
     l = sum(pl * np.exp2(pm - m) for pm, pl, _ in parts)
     o = sum(po * np.exp2(pm - m)[:, None] for pm, _, po in parts)
     assert np.abs(got - o / l[:, None]).max() <= 2e-6
+
+
+# ---- the Float16 arm of the interpreter's rounding (tk/src/interp.rs:37-50)
+def test_f16_rounding_is_ieee_binary16_nearest_even():
+    """Against numpy's float16 (an independent IEEE implementation): random values over 15 decades,
+    ties, the subnormal range, overflow and the largest finite value."""
+    rng = np.random.default_rng(0)
+    x = (rng.standard_normal(4000) * 10.0 ** rng.integers(-9, 6, 4000)).astype(np.float32)
+    edge = np.array([0.0, -0.0, 65504.0, 65519.99, 65520.0, 1e-8, 2.98e-8, 2.9802322e-8, 6e-8, 6.1035156e-5,
+                     1 + 2 ** -11, 1 + 2 ** -11 + 2 ** -20, 1 + 3 * 2 ** -11, np.inf, -np.inf], dtype=np.float32)
+    x = np.concatenate([x, edge, -edge])
+    with np.errstate(over="ignore"):
+        want = x.astype(np.float16).astype(np.float32)
+    got = oracle.round_f16(x)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_the_stream_dtype_switch_only_changes_the_rounding():
+    rng = np.random.default_rng(5)
+    q, k, v = (oracle.round_f16(oracle.round_bf16(rng.uniform(-1, 1, s).astype(np.float32)))
+               for s in ((1, 40, 2, 64), (1, 70, 2, 64), (1, 70, 2, 64)))
+    p = oracle.AttnProblem(q, k, v)
+    bf = oracle.attention_flash(p, 64, 64)
+    with oracle.stream_dtype("f16"):
+        f16 = oracle.attention_flash(p, 64, 64)
+    again = oracle.attention_flash(p, 64, 64)
+    assert np.array_equal(bf, again)  # the switch is back to bf16 after the block
+    assert np.array_equal(oracle.round_f16(f16), f16) and np.array_equal(oracle.round_bf16(bf), bf)
+    d = oracle.attention_direct(p)
+    assert np.abs(f16 - d).max() < np.abs(bf - d).max()  # f16 keeps three more bits

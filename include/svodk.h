@@ -73,8 +73,8 @@ typedef enum svodk_key_mask {
 
 /*
  * Attn of tk/src/ops/attention.rs:60-86.  Zero-initialise, then set fields.
- * Options this library has no kernel for (window, chunk, seg_start, cache,
- * bias) are still validated as the reference validates them and then answered
+ * Options this library has no kernel for (chunk, seg_start, cache, bias) are
+ * still validated as the reference validates them and then answered
  * with SVODK_GRAPH_CONFIG.
  *
  * `splits` > 1 asks for key splits (tk/src/ops/attention.rs:79, 280-302): the

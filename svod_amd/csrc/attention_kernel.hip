@@ -170,6 +170,10 @@ struct Wave {
   int wave_first_row, my_row;
   bool positive;
   float c_exp, unit, limit;
+  // A window (tk/src/ops/attention.rs:64-65): query i sees keys [i - reach_left, i + reach_right].
+  // reach_right is 0 under a causal mask; both are unused unless `windowed`.
+  bool windowed;
+  int reach_left, reach_right;
   // per-lane addressing
   int k_src[CH], v_src[CH];  // global byte offsets of this lane's chunk in each fill
   int k_read[KS], v_read[DB];
@@ -253,7 +257,11 @@ __device__ __forceinline__ uint64_t uniform_bits(const Wave<D, NW, F16> &w, int 
 // Whether a mask edge crosses block `blk` for this wave (L698-733).
 template <int D, int NW, bool CAUSAL, bool F16>
 __device__ __forceinline__ bool on_edge(const Wave<D, NW, F16> &w, int blk, uint64_t kbits) {
-  return kbits != ~0ull || (CAUSAL && (blk * kBkv + kBkv - 1 > w.wave_first_row));
+  const int k0 = blk * kBkv;
+  if (kbits != ~0ull || (CAUSAL && (k0 + kBkv - 1 > w.wave_first_row))) return true;
+  // L715-719: the window's right edge for the wave's first row, its left edge for the last.
+  return w.windowed && (k0 + kBkv - 1 > w.wave_first_row + w.reach_right ||
+                        k0 < w.wave_first_row + kWaveRows - 1 - w.reach_left);
 }
 
 // Scales (a non-positive scale only) and masks (L641-697) the scores of block `blk`: hidden
@@ -262,9 +270,15 @@ template <int D, int NW, bool CAUSAL, bool F16>
 __device__ __forceinline__ void mask_scores(const Wave<D, NW, F16> &w, int blk, uint64_t kbits, float (&sv)[32]) {
   const int k0 = blk * kBkv;
   uint64_t mine = kbits;
-  if (CAUSAL && (k0 + kBkv - 1 > w.wave_first_row)) {
-    const int seen = w.my_row - k0 + 1;  // keys k0 .. my_row
+  if ((CAUSAL && (k0 + kBkv - 1 > w.wave_first_row)) || w.windowed) {
+    // Keys k0 .. my_row (+ the window's reach to the right) are seen from above ...
+    const int seen = w.my_row + (CAUSAL ? 0 : w.reach_right) - k0 + 1;
     mine &= seen >= 64 ? ~0ull : (seen <= 0 ? 0ull : (~0ull >> (64 - seen)));
+    if (w.windowed) {
+      // ... and those from my_row - reach_left on from below (L659-668).
+      const int below = w.my_row - w.reach_left - k0;
+      mine &= below <= 0 ? ~0ull : (below >= 64 ? 0ull : (~0ull << below));
+    }
   }
   mine >>= 4 * w.g;
   const uint32_t lo = (uint32_t)mine, hi = (uint32_t)(mine >> 32);
@@ -546,7 +560,7 @@ __global__ __launch_bounds__(NW * 64, D == 64 ? 3 : 2) void flash_fwd_kernel(
     uint32_t units, uint32_t heads_group, const void *__restrict__ key_lens, const uint16_t *__restrict__ q, int32_t t,
     uint32_t tk_lens64, const uint16_t *__restrict__ k, const uint16_t *__restrict__ v,
     uint16_t *__restrict__ o, const void *__restrict__ key_mask, int32_t mask_bytes, float scale, Splits sp,
-    int32_t q_row_elems, int32_t kv_row_elems) {
+    int32_t q_row_elems, int32_t kv_row_elems, int32_t win_left, int32_t win_right) {
   // The body is device code only: the host pass needs the kernel's handle, not its
   // instructions (and drops the whole instantiation over the LDS-fill instructions).
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -624,20 +638,28 @@ __global__ __launch_bounds__(NW * 64, D == 64 ? 3 : 2) void flash_fwd_kernel(
     len = n < (long long)tk ? (int)n : tk;
   }
 
-  // L596-608: key blocks some query of the tile sees.
-  int end = (tk + kBkv - 1) / kBkv;
+  // L584-608: key blocks [first, end) hold every key some query of the tile sees.  A negative
+  // win_left means no window; the host caps both reaches at the sequence lengths.
+  w.windowed = win_left >= 0;
+  w.reach_left = win_left;
+  w.reach_right = CAUSAL ? 0 : win_right;
+  int first = 0, end = (tk + kBkv - 1) / kBkv;
+  if (w.windowed) first = max(q_off - win_left, 0) / kBkv;
   if (CAUSAL) end = min(end, (q_off + BQ + kBkv - 1) / kBkv);
+  if (w.windowed) end = min(end, (q_off + BQ + win_right + kBkv - 1) / kBkv);
   if (key_lens != nullptr) end = min(end, (len + kBkv - 1) / kBkv);
+  end = max(end, first);
   // L609-612: a split takes an even share of those blocks.  From here on the kernel works in
   // the split's own frame: keys, lengths and query rows count from the split's first key.
-  int first_key = 0;
   if (SPLIT) {
-    const int s_first = (int)div_by((uint32_t)end * (uint32_t)split, sp.count, sp.rcp);
-    const int s_end = (int)div_by((uint32_t)end * (uint32_t)(split + 1), sp.count, sp.rcp);
-    first_key = s_first * kBkv;
-    end = s_end - s_first;
-    len = max(len - first_key, 0);
+    const uint32_t n = (uint32_t)(end - first);
+    const int s_first = first + (int)div_by(n * (uint32_t)split, sp.count, sp.rcp);
+    end = first + (int)div_by(n * (uint32_t)(split + 1), sp.count, sp.rcp);
+    first = s_first;
   }
+  const int first_key = first * kBkv;
+  end -= first;
+  len = max(len - first_key, 0);
   w.end = end;
   w.len = len;
   w.tk = tk - first_key;
@@ -708,9 +730,10 @@ __global__ __launch_bounds__(NW * 64, D == 64 ? 3 : 2) void flash_fwd_kernel(
   // A causal wave past its last visible key has nothing to add from a block: it only keeps
   // filling and meeting the barriers.  Blocks [0, my_end) are this wave's.
   int my_end = end;
-  if (CAUSAL) {
-    const int last_row = w.wave_first_row + kWaveRows - 1;  // negative: the split lies past every row's diagonal
-    my_end = min(end, last_row < 0 ? 0 : last_row / kBkv + 1);
+  if (CAUSAL || w.windowed) {
+    // The last key the wave's last row sees; negative: the blocks lie past every row's reach.
+    const int last_seen = w.wave_first_row + kWaveRows - 1 + w.reach_right;
+    my_end = min(end, last_seen < 0 ? 0 : last_seen / kBkv + 1);
   }
 
   float sv[32], nv[32];  // S of the current and of the next block, swapping roles each hot step
@@ -736,9 +759,16 @@ __global__ __launch_bounds__(NW * 64, D == 64 ? 3 : 2) void flash_fwd_kernel(
   int full = 0;
   if (w.positive && key_mask == nullptr) {
     full = min(my_end, len / kBkv);
-    if (CAUSAL) full = min(full, (w.wave_first_row + 1) / kBkv);
+    if (CAUSAL || w.windowed) full = min(full, (w.wave_first_row + w.reach_right + 1) / kBkv);
   }
   int blk = 0;
+  if (w.windowed) {
+    // The window's left edge crosses the blocks below the last row's reach: general steps, an
+    // even number of them so that the hot pairs start on an even block.
+    const int below = w.wave_first_row + kWaveRows - 1 - w.reach_left;
+    const int lead = min(my_end, below <= 0 ? 0 : ((below + kBkv - 1) / kBkv + 1) & ~1);
+    for (; blk < lead; blk++) edge_step<D, NW, CAUSAL>(w, smem, blk, my_end, sv, bm);
+  }
   for (; blk + 2 < full; blk += 2) {
     hot_step<D, NW, 0>(w, smem, blk, sv, nv, bm);
     hot_step<D, NW, 1>(w, smem, blk + 1, nv, sv, bm);
@@ -845,7 +875,7 @@ hipError_t launch(const AttnArgs &a, hipStream_t stream) {
                      geo.nqt_rcp, geo.kv_heads, geo.kvh_rcp, geo.units, heads_group, a.key_lens,
                      (const uint16_t *)a.q, a.t, tk_lens64, (const uint16_t *)a.k,
                      (const uint16_t *)a.v, (uint16_t *)a.o, a.key_mask, a.mask_bytes, a.scale, sp, (int32_t)q_row,
-                     (int32_t)kv_row);
+                     (int32_t)kv_row, a.win_left, a.win_right);
   return hipGetLastError();
 }
 

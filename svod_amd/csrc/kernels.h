@@ -48,6 +48,9 @@ struct AttnArgs {
   // Elements from a token's row to the next in q and in k/v; 0 = dense (heads * d, kv_heads * d).
   // A fused projection read in place (tk/src/ops/attention.rs:104-122) has its own row for both.
   int64_t q_row_elems, kv_row_elems;
+  // Attn::window (tk/src/ops/attention.rs:64-65): query i sees keys [i - win_left, i + win_right];
+  // win_left < 0 = no window.
+  int32_t win_left, win_right;
 };
 hipError_t launch_attention(const AttnArgs &a, hipStream_t stream);
 

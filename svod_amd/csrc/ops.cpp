@@ -8,6 +8,7 @@
 // it behaves the same on a machine without a GPU.
 #include <hip/hip_runtime_api.h>
 
+#include <algorithm>
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
@@ -332,8 +333,10 @@ static int attend(const svodk_tensor *q, const svodk_tensor *k, const svodk_tens
   if (why != 0) return ran_graph(op, why);
   // Options the reference's kernel holds and this library's does not: no
   // config here holds them (the reference's own use of Fallback::Config, L210-214).
-  if (opts->has_window || opts->has_chunk || opts->seg_start != nullptr || opts->has_cache || opts->bias != nullptr)
+  if (opts->has_chunk || opts->seg_start != nullptr || opts->has_cache || opts->bias != nullptr)
     return ran_graph(op, SVODK_GRAPH_CONFIG);
+  if (opts->has_window && (opts->window_left < 0 || opts->window_right < 0))
+    return fail(SVODK_ERR_ARGUMENT, "%s: a negative window reach", op);
   const int64_t t = q->shape[1], tk = k->shape[1], d = q->shape[3];
   if (t > 0x7fffffff || tk > 0x7fffffff || heads > 0x7fffffff || cap > 0x7fffffff)
     return ran_graph(op, SVODK_GRAPH_SHAPE);
@@ -373,6 +376,12 @@ static int attend(const svodk_tensor *q, const svodk_tensor *k, const svodk_tens
   // L230: the default scale is 1/sqrt(D) in f32.
   a.scale = opts->has_scale ? opts->scale : 1.0f / std::sqrt((float)d);
   a.f16 = q->dtype == SVODK_F16;
+  // The window's reaches, capped where they no longer hide anything (and stay 32-bit).
+  a.win_left = -1;
+  if (opts->has_window) {
+    a.win_left = (int32_t)std::min<int64_t>(opts->window_left, t + tk);
+    a.win_right = (int32_t)std::min<int64_t>(opts->window_right, t + tk);
+  }
   if (packed != nullptr) a.q_row_elems = a.kv_row_elems = (heads + 2 * kv_heads) * d;
   // L280-302: key splits.  The partial tensors live in the caller's workspace.
   a.splits = split_count(opts->splits, tk);

@@ -169,6 +169,15 @@ int svodk_plan_heads(int32_t has_target, const int32_t *dtypes, int32_t n_dtypes
                      int32_t head_dim);
 
 /*
+ * A tuning knob in place of the reference's per-shape tuner (tk/src/tune.rs): attention calls
+ * with head size 64, no key mask tensor, no window and no splits can run as "streaming"
+ * workgroups that each walk a run of query tiles, the next tile's keys loading under the
+ * current tile's last steps.  n > 0 = stream, n workgroups per XCD (96 fills an MI355X);
+ * n <= 0 (the default) = a workgroup per tile.  Process-wide.  Results are bit-equal either way.
+ */
+void svodk_tune_streaming(int32_t workgroups_per_xcd);
+
+/*
  * ops::supported (tk/src/ops/mod.rs:164-166): 1 when the current HIP device is
  * a gfx950 this library has kernels for.
  */

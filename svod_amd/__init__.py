@@ -16,6 +16,7 @@ from .ops import (  # noqa: F401
     Qkv,
     attention,
     attention_packed,
+    tune_streaming,
     chosen,
     heads,
     library_path,

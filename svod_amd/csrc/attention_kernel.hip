@@ -68,6 +68,10 @@ constexpr int kXcds = 8;       // accelerator dies of an MI355X, each with its o
 constexpr float kLog2e = 1.44269504088896340736f;
 constexpr float kRescaleAbove = 8.0f;  // tk/src/kernels/attention.rs:379
 
+// Workgroups an XCD's item list is split over in the streaming form: 0 = as many as the XCD
+// holds, when the list is long enough to be worth it; > 0 = always that many; < 0 = never stream.
+std::atomic<int> g_stream_slots{0};
+
 // A ring slot holds a [64 keys, D] tile, rows unpadded (D*2 bytes), filled by
 // buffer_load_dwordx4 ... lds: a wave instruction lands 64 consecutive 16-byte
 // chunks, so the only freedom is WHICH global chunk a lane fetches.  Each row's
@@ -175,13 +179,19 @@ struct Wave {
   bool windowed;
   int reach_left, reach_right;
   // per-lane addressing
-  int k_src[CH], v_src[CH];  // global byte offsets of this lane's chunk in each fill
+  int k_src, v_src;  // global byte offsets of this lane's chunk in this wave's first fill of a tile
   int k_read[KS], v_read[DB];
   // state
   u32x4 qf[KS];
   f32x16 acc[DB];
   float m_run, l_run;
   int mask_next;
+  // A streaming workgroup's next item (nxt_end = 0: none, as in the one-item kernel): this item's
+  // last steps request its first blocks.  The next item's blocks follow this item's at an even
+  // position of the ring (end_even = end rounded up), so every item starts in slot 0.
+  const uint8_t *nxt_k, *nxt_v;
+  int64_t nxt_bytes;
+  int nxt_end, end_even;
 };
 
 // The fills are issued as raw instructions: the compiler's wait-count pass treats an LDS fill
@@ -189,26 +199,40 @@ struct Wave {
 // fills in the middle of the current tile.  The kernel waits for them itself (vmcnt(0) before
 // the barrier that ends a step).  m0 carries the LDS address of a wave instruction's 1 KiB.
 template <int D, int NW, bool F16>
-__device__ __forceinline__ void fill_tile(const Wave<D, NW, F16> &w, const uint8_t *base, int blk, int lds_at,
-                                          const int (&src)[Wave<D, NW, F16>::CH]) {
+__device__ __forceinline__ void fill_tile(const Wave<D, NW, F16> &w, const uint8_t *base, int64_t bytes, int blk,
+                                          int lds_at, int src) {
+  // This wave's fills of a tile are NW instructions apart; the swizzle repeats with that period,
+  // so they share the lanes' offsets and differ in the descriptor's base.
+  constexpr int kRowsPer = 64 / Tile<D>::kCpr;  // rows a wave instruction covers
+  static_assert((NW * kRowsPer) % 16 == 0, "the swizzle repeats from one of a wave's fills to its next");
   const int64_t off = (int64_t)blk * kBkv * w.kv_row_bytes;
-  const i32x4 r = make_rsrc(base + off, w.kv_bytes - off);
 #pragma unroll
   for (int i = 0; i < Wave<D, NW, F16>::CH; i++) {
-    const int j = w.wave + NW * i;
+    const int64_t at = off + (int64_t)(NW * i * kRowsPer) * w.kv_row_bytes;
+    const i32x4 r = make_rsrc(base + at, bytes - at);
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
                  :
-                 : "s"(lds_at + j * 1024), "v"(src[i]), "s"(r)
+                 : "s"(lds_at + (w.wave + NW * i) * 1024), "v"(src), "s"(r)
                  : "memory");
   }
 }
+// Block `n` of the stream of blocks that starts with this item's: the item's own while n < end,
+// then (past the padding to an even count) the next item's.  Nothing past either.
 template <int D, int NW, bool F16>
-__device__ __forceinline__ void fill_k(const Wave<D, NW, F16> &w, int blk, int slot) {
-  fill_tile<D, NW>(w, w.k_base, blk, w.lds0 + slot * Tile<D>::kBytes, w.k_src);
+__device__ __forceinline__ void fill_k(const Wave<D, NW, F16> &w, int n, int slot) {
+  const int at = w.lds0 + slot * Tile<D>::kBytes;
+  if (n < w.end)
+    fill_tile<D, NW>(w, w.k_base, w.kv_bytes, n, at, w.k_src);
+  else if (n >= w.end_even && n - w.end_even < w.nxt_end)
+    fill_tile<D, NW>(w, w.nxt_k, w.nxt_bytes, n - w.end_even, at, w.k_src);
 }
 template <int D, int NW, bool F16>
-__device__ __forceinline__ void fill_v(const Wave<D, NW, F16> &w, int blk, int slot) {
-  fill_tile<D, NW>(w, w.v_base, blk, w.lds0 + (2 + slot) * Tile<D>::kBytes, w.v_src);
+__device__ __forceinline__ void fill_v(const Wave<D, NW, F16> &w, int n, int slot) {
+  const int at = w.lds0 + (2 + slot) * Tile<D>::kBytes;
+  if (n < w.end)
+    fill_tile<D, NW>(w, w.v_base, w.kv_bytes, n, at, w.v_src);
+  else if (n >= w.end_even && n - w.end_even < w.nxt_end)
+    fill_tile<D, NW>(w, w.nxt_v, w.nxt_bytes, n - w.end_even, at, w.v_src);
 }
 
 // A key mask row is read 64 keys (one per lane) a block, one block ahead: the load is issued
@@ -410,7 +434,7 @@ __device__ __forceinline__ void hot_step(Wave<D, NW, F16> &w, const uint8_t *sme
 #pragma unroll
   for (int f = 0; f < 4; f++) kf[f] = k_frag(f);
   fill_v<D, NW>(w, blk + 1, PAR ^ 1);
-  if (blk + 2 < w.end) fill_k<D, NW>(w, blk + 2, PAR);
+  fill_k<D, NW>(w, blk + 2, PAR);
   w.mask_next = 0;  // hot steps run without a key mask only
   float corr;
   const float m_exp = adopt_maximum<D, NW>(w, bm, corr);
@@ -493,11 +517,9 @@ __device__ __forceinline__ void edge_step(Wave<D, NW, F16> &w, const uint8_t *sm
   const int par = blk & 1;
   const bool more = blk + 1 < my_end;
   const uint64_t kbits_next = uniform_bits<D, NW>(w, blk + 1, w.mask_next);
-  if (blk + 1 < w.end) fill_v<D, NW>(w, blk + 1, par ^ 1);
-  if (blk + 2 < w.end) {
-    w.mask_next = mask_lane<D, NW>(w, blk + 2);
-    fill_k<D, NW>(w, blk + 2, par);
-  }
+  fill_v<D, NW>(w, blk + 1, par ^ 1);
+  if (blk + 2 < w.end) w.mask_next = mask_lane<D, NW>(w, blk + 2);
+  fill_k<D, NW>(w, blk + 2, par);
   float corr;
   const float m_exp = adopt_maximum<D, NW>(w, bm, corr);
 
@@ -526,8 +548,8 @@ __device__ __forceinline__ void edge_step(Wave<D, NW, F16> &w, const uint8_t *sm
 template <int D, int NW, bool F16>
 __device__ __forceinline__ void idle_step(Wave<D, NW, F16> &w, int blk) {
   const int par = blk & 1;
-  if (blk + 1 < w.end) fill_v<D, NW>(w, blk + 1, par ^ 1);
-  if (blk + 2 < w.end) fill_k<D, NW>(w, blk + 2, par);
+  fill_v<D, NW>(w, blk + 1, par ^ 1);
+  fill_k<D, NW>(w, blk + 2, par);
   __builtin_amdgcn_s_waitcnt(0x0f70);
   __syncthreads();
 }
@@ -675,23 +697,23 @@ __global__ __launch_bounds__(NW * 64, D == 64 ? 3 : 2) void flash_fwd_kernel(
   w.kv_bytes = len > 0 ? (int64_t)(len - 1) * w.kv_row_bytes + D * 2 : 0;
   w.lds0 = (int)(uintptr_t)(LDS_PTR(uint8_t))(smem);
 
-  // ---- this wave's share of a tile fill: CH wave-wide 1 KiB instructions.  Fill j lands on
-  // rows [j*rows_per, ...): lane i at physical chunk i % kCpr of row i / kCpr.
+  // ---- this wave's share of a tile fill: CH wave-wide 1 KiB instructions, NW apart.  Fill j
+  // lands on rows [j*rows_per, ...): lane i at physical chunk i % kCpr of row i / kCpr.
   constexpr int kRowsPer = 64 / TL::kCpr;
-#pragma unroll
-  for (int i = 0; i < CH; i++) {
-    const int j = w.wave + NW * i;
-    const int row = j * kRowsPer + w.lane / TL::kCpr;
+  {
+    const int row = w.wave * kRowsPer + w.lane / TL::kCpr;
     const int pc = w.lane % TL::kCpr;
-    w.k_src[i] = row * w.kv_row_bytes + ((pc ^ TL::swz_k(row)) << 4);
-    w.v_src[i] = row * w.kv_row_bytes + ((pc ^ (TL::swz_v(row) << 2)) << 4);
+    w.k_src = row * w.kv_row_bytes + ((pc ^ TL::swz_k(row)) << 4);
+    w.v_src = row * w.kv_row_bytes + ((pc ^ (TL::swz_v(row) << 2)) << 4);
   }
   // ---- K(0), V(0), K(1) go first: everything below runs in the shadow of their flight.
-  if (end > 0) {
-    fill_k<D, NW>(w, 0, 0);
-    fill_v<D, NW>(w, 0, 0);
-  }
-  if (end > 1) fill_k<D, NW>(w, 1, 1);
+  w.nxt_end = 0;  // one item a workgroup
+  w.end_even = end;
+  w.nxt_k = w.nxt_v = nullptr;
+  w.nxt_bytes = 0;
+  fill_k<D, NW>(w, 0, 0);
+  fill_v<D, NW>(w, 0, 0);
+  fill_k<D, NW>(w, 1, 1);
   // Key-mask words are read two blocks ahead of their use.
   const int word0 = mask_lane<D, NW>(w, 0);
   w.mask_next = mask_lane<D, NW>(w, 1);
@@ -817,6 +839,400 @@ __global__ __launch_bounds__(NW * 64, D == 64 ? 3 : 2) void flash_fwd_kernel(
 #endif  // __HIP_DEVICE_COMPILE__
 }
 
+// ---------------------------------------------------------------------------------------------
+// The streaming form: a workgroup takes a run of consecutive query tiles (items) and walks them
+// as one stream of key blocks.  The last steps of an item fill the ring with the next item's
+// first blocks, and the next item's Q rows are already staged in LDS, so an item starts without
+// the launch, the argument loads, the first fills' flight and the output drain that a
+// workgroup of its own pays; with 1 to 8 key blocks an item (BGE-M3) those are a third of its
+// time.  Runs are fixed from the key lengths alone (no shared counters): every workgroup works
+// out the same split of the XCD's item list into runs of equal estimated cost.
+// ---------------------------------------------------------------------------------------------
+
+// Key blocks of query tile `qt` of a batch row with `len` keys (L596-608), at least 1 (a tile
+// with no visible block still takes one step, of a block whose keys are all hidden).
+template <int NW, bool CAUSAL>
+__device__ __forceinline__ int item_blocks(int qt, int len, int tk, bool has_lens) {
+  constexpr int BQ = NW * kWaveRows;
+  int end = (tk + kBkv - 1) / kBkv;
+  if (CAUSAL) end = min(end, (qt * BQ + BQ + kBkv - 1) / kBkv);
+  if (has_lens) end = min(end, (len + kBkv - 1) / kBkv);
+  return max(end, 1);
+}
+
+// The estimated cost of an item in steps: its key blocks plus one for the switch.
+__device__ __forceinline__ int item_cost(int blocks) { return blocks + 1; }
+
+__device__ __forceinline__ int wave_sum(int x) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) x += __shfl_xor(x, m, 64);
+  return x;
+}
+// Exclusive prefix sum over the wave's lanes.
+__device__ __forceinline__ int wave_scan(int x, int lane) {
+  int inc = x;
+#pragma unroll
+  for (int m = 1; m < 64; m <<= 1) {
+    const int up = __shfl_up(inc, m, 64);
+    if (lane >= m) inc += up;
+  }
+  return inc - x;
+}
+
+// One XCD's list of items and the cost model over it.  Unit r of the list is (batch, kv head)
+// number r * 8 + xcd; a unit's items run head-in-group major, then query tile in launch order.
+template <int NW, bool CAUSAL>
+struct ItemList {
+  const Geometry &geo;
+  uint32_t xcd, units_here;
+  const void *key_lens;
+  bool lens_i64;
+  int tk, nqt;
+
+  __device__ __forceinline__ int len_of(int b) const {
+    if (key_lens == nullptr) return tk;
+    long long n = lens_i64 ? ((const long long *)key_lens)[b] : (long long)((const int *)key_lens)[b];
+    n = n < 0 ? 0 : n;
+    return n < (long long)tk ? (int)n : tk;
+  }
+  // The same for a wave-uniform b, as a scalar load: inside the item loop a vector load would
+  // bring a vmcnt wait that also sits out the fills and stores in flight.
+  __device__ __forceinline__ int len_of_uniform(int b) const {
+    if (key_lens == nullptr) return tk;
+    auto word = [&](int byte) {
+      int x;
+      asm volatile("s_load_dword %0, %1, %2\n\ts_waitcnt lgkmcnt(0)" : "=s"(x) : "s"(key_lens), "s"(byte) : "memory");
+      return x;
+    };
+    long long n;
+    if (lens_i64)
+      n = (long long)(((uint64_t)(uint32_t)word(b * 8 + 4) << 32) | (uint32_t)word(b * 8));
+    else
+      n = (long long)word(b * 4);
+    n = n < 0 ? 0 : n;
+    return n < (long long)tk ? (int)n : tk;
+  }
+  // Query tile of place `order` within a head (L524-528: longest first under a causal mask).
+  __device__ __forceinline__ int tile_of(int order) const { return CAUSAL ? nqt - 1 - order : order; }
+  // Cost of one head's tiles of batch row b, and the number of them whose start lies below x.
+  __device__ __forceinline__ int head_cost(int len) const {
+    int c = 0;
+    for (int order = 0; order < nqt; order++)
+      c += item_cost(item_blocks<NW, CAUSAL>(tile_of(order), len, tk, key_lens != nullptr));
+    return c;
+  }
+  __device__ __forceinline__ int tiles_below(int len, int x) const {
+    int c = 0, n = 0;
+    for (int order = 0; order < nqt; order++) {
+      if (c < x) n++;
+      c += item_cost(item_blocks<NW, CAUSAL>(tile_of(order), len, tk, key_lens != nullptr));
+    }
+    return n;
+  }
+  // Items of the list whose start cost lies below `bound`, and the list's whole cost.  Every
+  // lane returns the same numbers.
+  __device__ __forceinline__ void count(int64_t bound_a, int64_t bound_b, int lane, int64_t &total, uint32_t &below_a,
+                                        uint32_t &below_b) const {
+    const int group = (int)geo.group;
+    int64_t before = 0;
+    uint32_t na = 0, nb = 0;
+    for (uint32_t r0 = 0; r0 < units_here; r0 += 64) {
+      const uint32_t r = r0 + lane;
+      int per_head = 0, len = 0;
+      if (r < units_here) {
+        const uint32_t unit = r * kXcds + xcd;
+        len = len_of((int)div_by(unit, geo.kv_heads, geo.kvh_rcp));
+        per_head = head_cost(len);
+      }
+      const int mine = per_head * group;
+      const int64_t start = before + wave_scan(mine, lane);
+      auto inside = [&](int64_t bound) -> uint32_t {
+        if (r >= units_here || bound <= start) return 0u;
+        const int64_t x = bound - start;
+        if (x >= mine) return geo.unit_size;
+        const int heads_done = (int)(x / per_head);
+        return (uint32_t)(heads_done * nqt + tiles_below(len, (int)(x - (int64_t)heads_done * per_head)));
+      };
+      na += (uint32_t)wave_sum((int)inside(bound_a));
+      nb += (uint32_t)wave_sum((int)inside(bound_b));
+      before += wave_sum(mine);
+    }
+    total = before;
+    below_a = na;
+    below_b = nb;
+  }
+};
+
+template <int D, int NW, bool CAUSAL, bool F16>
+__global__ __launch_bounds__(NW * 64, 3) void flash_stream_kernel(
+    uint32_t unit_size, uint32_t unit_rcp, uint32_t nqt_u, uint32_t nqt_rcp, uint32_t kvh_u, uint32_t kvh_rcp,
+    uint32_t units, uint32_t heads_group, const void *__restrict__ key_lens, const uint16_t *__restrict__ q, int32_t t,
+    uint32_t tk_lens64, const uint16_t *__restrict__ k, const uint16_t *__restrict__ v,
+    uint16_t *__restrict__ o, float scale, int32_t q_row_elems, int32_t kv_row_elems, uint32_t slots) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  const Geometry geo = {unit_size, unit_rcp, nqt_u, nqt_rcp, kvh_u, kvh_rcp, heads_group >> 16, units};
+  const int heads = (int)(heads_group & 0xffffu);
+  const int tk = (int)(tk_lens64 & 0x7fffffffu);
+  const bool lens_i64 = (tk_lens64 >> 31) != 0;
+  using TL = Tile<D>;
+  using W = Wave<D, NW, F16>;
+  constexpr int BQ = NW * kWaveRows;
+  constexpr int KS = W::KS, DB = W::DB, CH = W::CH;
+  constexpr int kStageRows = 1024 / TL::kRowBytes;                  // rows a wave instruction stages
+  constexpr int kStageInstrs = kWaveRows * TL::kRowBytes / 1024;    // per wave and item
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+  uint8_t *stage = smem + TL::kLds;  // [BQ rows][D] of the next item's Q
+
+  W w;
+  const int tid = __builtin_amdgcn_workitem_id_x();
+  w.lane = tid & 63;
+  w.wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  w.g = w.lane >> 5;
+  const int ln = w.lane & 31;
+
+  // ---- this workgroup's run of the XCD's list: items [run_first, run_end).
+  const uint32_t wg = __builtin_amdgcn_workgroup_id_x();
+  const uint32_t xcd = wg % kXcds, slot = wg / kXcds;
+  const uint32_t units_here = geo.units > xcd ? (geo.units - xcd + kXcds - 1) / kXcds : 0;
+  const ItemList<NW, CAUSAL> list = {geo, xcd, units_here, key_lens, lens_i64, tk, (int)geo.nqt};
+  uint32_t run_first, run_end;
+  {
+    // Two passes: the list's whole cost, then the items below this slot's two bounds.
+    int64_t total;
+    uint32_t a, b;
+    list.count(0, 0, w.lane, total, a, b);
+    const int64_t lo = total * slot / slots, hi = total * (slot + 1) / slots;
+    list.count(lo, hi, w.lane, total, a, b);
+    run_first = __builtin_amdgcn_readfirstlane(a);
+    run_end = __builtin_amdgcn_readfirstlane(b);
+  }
+  if (run_first >= run_end) return;
+
+  // ---- call constants
+  const int64_t o_row_stride = (int64_t)heads * D;
+  w.tk = tk;
+  w.key_mask = nullptr;
+  w.mask_row = 0;
+  w.mask_bytes = 0;
+  w.mask_next = 0;
+  w.windowed = false;
+  w.reach_left = 0;
+  w.reach_right = 0;
+  w.kv_row_bytes = kv_row_elems * 2;
+  w.lds0 = (int)(uintptr_t)(LDS_PTR(uint8_t))(smem);
+  constexpr int kRowsPer = 64 / TL::kCpr;
+  {
+    const int row = w.wave * kRowsPer + w.lane / TL::kCpr;
+    const int pc = w.lane % TL::kCpr;
+    w.k_src = row * w.kv_row_bytes + ((pc ^ TL::swz_k(row)) << 4);
+    w.v_src = row * w.kv_row_bytes + ((pc ^ (TL::swz_v(row) << 2)) << 4);
+  }
+#pragma unroll
+  for (int ks = 0; ks < KS; ks++) w.k_read[ks] = ln * TL::kRowBytes + (((2 * ks + w.g) ^ TL::swz_k(ln)) << 4);
+  const int vq = (w.lane & 15) >> 2;
+  const int vc = 2 * ((w.lane >> 4) & 1) + ((w.lane & 3) >> 1);
+#pragma unroll
+  for (int db = 0; db < DB; db++)
+    w.v_read[db] = (4 * w.g + vq) * TL::kRowBytes + ((db ^ TL::swz_v(vq)) << 6) + (vc << 4) + ((w.lane & 1) << 3);
+  w.positive = scale > 0.0f;
+  w.c_exp = scale * kLog2e;
+  w.unit = w.positive ? w.c_exp : 1.0f;
+  w.limit = kRescaleAbove / w.unit;
+
+  // An item of the list: where its rows and keys are.
+  struct Item {
+    int b, h, q_off, len, end;
+    const uint8_t *k_base, *v_base;
+    int64_t kv_bytes;
+  };
+  auto item = [&](uint32_t s) -> Item {
+    Item it;
+    const uint32_t round = div_by(s, geo.unit_size, geo.unit_rcp);
+    const uint32_t unit = round * kXcds + xcd;
+    const uint32_t within = s - round * geo.unit_size;
+    const uint32_t head_in_group = div_by(within, geo.nqt, geo.nqt_rcp);
+    const int order = (int)(within - head_in_group * geo.nqt);
+    it.b = (int)div_by(unit, geo.kv_heads, geo.kvh_rcp);
+    const int kvh = (int)(unit - (uint32_t)it.b * geo.kv_heads);
+    it.h = kvh * (int)geo.group + (int)head_in_group;
+    const int qt = list.tile_of(order);
+    it.q_off = qt * BQ;
+    it.len = list.len_of_uniform(it.b);
+    it.end = item_blocks<NW, CAUSAL>(qt, it.len, tk, key_lens != nullptr);
+    it.k_base = (const uint8_t *)(k + (int64_t)it.b * tk * kv_row_elems + (int64_t)kvh * D);
+    it.v_base = (const uint8_t *)(v + (int64_t)it.b * tk * kv_row_elems + (int64_t)kvh * D);
+    it.kv_bytes = it.len > 0 ? (int64_t)(it.len - 1) * w.kv_row_bytes + D * 2 : 0;
+    return it;
+  };
+  // This wave's rows of an item's Q, global -> LDS: rows past t read as zeros.
+  const int stage_lds = w.lds0 + TL::kLds + w.wave * kWaveRows * TL::kRowBytes;
+  const int q_row_bytes = q_row_elems * 2;
+  auto stage_q = [&](const Item &it) {
+    // The lane's offset is worked out afresh each time (the empty asm keeps the compiler from
+    // carrying it, and spilling it, across the item loop).
+    int lane = w.lane;
+    asm volatile("" : "+v"(lane));
+    const int stage_src = (lane / TL::kCpr) * q_row_bytes + (lane % TL::kCpr) * 16;
+    const int row0 = it.q_off + w.wave * kWaveRows;
+    const uint8_t *base = (const uint8_t *)q + ((int64_t)it.b * t + row0) * q_row_bytes + (int64_t)it.h * (D * 2);
+    const int64_t rows = (int64_t)t - row0;
+    const int64_t bytes = rows > 0 ? (rows - 1) * q_row_bytes + D * 2 : 0;
+#pragma unroll
+    for (int i = 0; i < kStageInstrs; i++) {
+      const int64_t skip = (int64_t)(i * kStageRows) * q_row_bytes;
+      const i32x4 r = make_rsrc(base + skip, bytes - skip);
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                   :
+                   : "s"(stage_lds + i * 1024), "v"(stage_src), "s"(r)
+                   : "memory");
+    }
+  };
+
+  // ---- the first item: K(0), V(0), K(1) and its Q rows in flight, then everything lands.
+  Item cur = item(run_first);
+  auto adopt = [&](const Item &it) {
+    int lane = w.lane;
+    asm volatile("" : "+v"(lane));
+    const int ln = lane & 31;
+    w.k_base = it.k_base;
+    w.v_base = it.v_base;
+    w.kv_bytes = it.kv_bytes;
+    w.end = it.end;
+    w.end_even = (it.end + 1) & ~1;
+    w.len = it.len;
+    w.wave_first_row = it.q_off + w.wave * kWaveRows;
+    w.my_row = w.wave_first_row + ln;
+  };
+  adopt(cur);
+  w.nxt_end = 0;
+  w.nxt_k = w.nxt_v = nullptr;
+  w.nxt_bytes = 0;
+  fill_k<D, NW>(w, 0, 0);
+  fill_v<D, NW>(w, 0, 0);
+  fill_k<D, NW>(w, 1, 1);
+  stage_q(cur);
+  w.m_run = -1e30f;
+  w.l_run = 0.0f;
+  const f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+  for (int db = 0; db < DB; db++) w.acc[db] = zero;
+  __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+  __syncthreads();
+
+  for (uint32_t s = run_first; s < run_end; s++) {
+    // ---- the item after this one: its first blocks ride this item's last steps.
+    const bool more_items = s + 1 < run_end;
+    Item nxt = cur;
+    if (more_items) nxt = item(s + 1);
+    w.nxt_end = more_items ? nxt.end : 0;
+    w.nxt_k = nxt.k_base;
+    w.nxt_v = nxt.v_base;
+    w.nxt_bytes = nxt.kv_bytes;
+    // ---- this item's Q rows from the stage to registers; the stage is then free for the next
+    // item's rows, which have the whole item to arrive.
+    {
+      int lane = w.lane;
+      asm volatile("" : "+v"(lane));
+      const uint8_t *mine = stage + (w.wave * kWaveRows + (lane & 31)) * TL::kRowBytes + (lane >> 5) * 16;
+#pragma unroll
+      for (int ks = 0; ks < KS; ks++) w.qf[ks] = *reinterpret_cast<const u32x4 *>(mine + ks * 32);
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the reads are done before the refill is issued
+      if (more_items) stage_q(nxt);
+    }
+    const int end = w.end;
+    int my_end = end;
+    if (CAUSAL) {
+      const int last_seen = w.wave_first_row + kWaveRows - 1;
+      my_end = min(end, last_seen / kBkv + 1);
+    }
+    float sv[32], nv[32];
+    float bm = -INFINITY;
+    {
+      scores<D, NW>(w, smem, 0, sv);
+      if (!w.positive) {
+#pragma unroll
+        for (int i = 0; i < 32; i++) sv[i] *= w.c_exp;
+      }
+      const uint64_t kbits0 = uniform_bits<D, NW>(w, 0, 0);
+      if (on_edge<D, NW, CAUSAL>(w, 0, kbits0)) mask_scores<D, NW, CAUSAL>(w, 0, kbits0, sv);
+      bm = row_max(sv);
+    }
+    // Step 0 refills the K slot those scores were read from: every wave has read it first.
+    __syncthreads();
+
+    int full = 0;
+    if (w.positive) {
+      full = min(my_end, w.len / kBkv);
+      if (CAUSAL) full = min(full, (w.wave_first_row + 1) / kBkv);
+    }
+    int blk = 0;
+    for (; blk + 2 < full; blk += 2) {
+      hot_step<D, NW, 0>(w, smem, blk, sv, nv, bm);
+      hot_step<D, NW, 1>(w, smem, blk + 1, nv, sv, bm);
+    }
+    for (; blk < my_end; blk++) edge_step<D, NW, CAUSAL>(w, smem, blk, my_end, sv, bm);
+    // Steps with nothing to compute: a causal wave past its diagonal, and the padding of an odd
+    // item, which keeps the next item's blocks in the slots a first item's would be in.
+    const int steps = more_items ? w.end_even : end;
+    for (; blk < steps; blk++) idle_step<D, NW>(w, blk);
+
+    // ---- out = o / (l == 0 ? 1 : l), bounded store (L892-898, L974-980).  The stores fly under
+    // the next item's first step.
+    {
+      const Pair lp = both_halves(w.l_run);
+      const float l_tot = lp.a + lp.b;
+      const float inv = 1.0f / (l_tot == 0.0f ? 1.0f : l_tot);
+      if (w.my_row < t) {
+        uint16_t *o_ptr = o + ((int64_t)cur.b * t + w.my_row) * o_row_stride + (int64_t)cur.h * D + 4 * w.g;
+#pragma unroll
+        for (int db = 0; db < DB; db++) {
+#pragma unroll
+          for (int c = 0; c < 4; c++) {
+            u32x2 x;
+            x[0] = pack2<F16>(w.acc[db][4 * c] * inv, w.acc[db][4 * c + 1] * inv);
+            x[1] = pack2<F16>(w.acc[db][4 * c + 2] * inv, w.acc[db][4 * c + 3] * inv);
+            *reinterpret_cast<u32x2 *>(o_ptr + 32 * db + 8 * c) = x;
+          }
+        }
+      }
+      w.m_run = -1e30f;
+      w.l_run = 0.0f;
+#pragma unroll
+      for (int db = 0; db < DB; db++) w.acc[db] = zero;
+    }
+    if (more_items) {
+      cur = nxt;
+      adopt(cur);
+    }
+  }
+#endif  // __HIP_DEVICE_COMPILE__
+}
+
+template <int D, int NW, bool CAUSAL, bool F16>
+hipError_t launch_stream(const AttnArgs &a, hipStream_t stream, int64_t slots, const Geometry &geo, int64_t q_row,
+                         int64_t kv_row) {
+  using TL = Tile<D>;
+  constexpr int smem = TL::kLds + NW * kWaveRows * TL::kRowBytes;
+  auto kernel = flash_stream_kernel<D, NW, CAUSAL, F16>;
+  static std::atomic<uint64_t> configured{0};
+  int device = 0;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) return e;
+  const uint64_t bit = device < 64 ? 1ull << device : 0;
+  if ((configured.load(std::memory_order_acquire) & bit) == 0) {
+    e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return e;
+    configured.fetch_or(bit, std::memory_order_release);
+  }
+  const uint32_t heads_group = (uint32_t)a.heads | geo.group << 16;
+  const uint32_t tk_lens64 = (uint32_t)a.tk | (a.lens_i64 ? 0x80000000u : 0u);
+  hipLaunchKernelGGL(kernel, dim3((uint32_t)(slots * kXcds)), dim3(NW * 64), smem, stream, geo.unit_size, geo.unit_rcp,
+                     geo.nqt, geo.nqt_rcp, geo.kv_heads, geo.kvh_rcp, geo.units, heads_group, a.key_lens,
+                     (const uint16_t *)a.q, a.t, tk_lens64, (const uint16_t *)a.k, (const uint16_t *)a.v,
+                     (uint16_t *)a.o, a.scale, (int32_t)q_row, (int32_t)kv_row, (uint32_t)slots);
+  return hipGetLastError();
+}
+
 template <int D, int NW, bool CAUSAL, bool SPLIT, bool F16>
 hipError_t launch(const AttnArgs &a, hipStream_t stream) {
   using TL = Tile<D>;
@@ -861,6 +1277,14 @@ hipError_t launch(const AttnArgs &a, hipStream_t stream) {
   geo.group = (uint32_t)(a.heads / a.kv_heads);
   geo.units = (uint32_t)units;
   if (a.heads > 0xffff) return hipErrorInvalidConfiguration;  // heads and group share an argument
+  // The streaming form, where asked for and where it has a kernel (head size 64, lengths or no
+  // key mask, no window, no splits): `knob` workgroups per XCD, each walking its run of tiles.
+  // It is never chosen unasked: measured, it has not beaten a workgroup per tile.
+  if constexpr (D == 64 && !SPLIT) {
+    const int knob = g_stream_slots.load(std::memory_order_relaxed);
+    if (knob > 0 && a.key_mask == nullptr && a.win_left < 0)
+      return launch_stream<D, NW, CAUSAL, F16>(a, stream, knob, geo, q_row, kv_row);
+  }
   const uint32_t heads_group = (uint32_t)a.heads | geo.group << 16;
   const uint32_t tk_lens64 = (uint32_t)a.tk | (a.lens_i64 ? 0x80000000u : 0u);
   Splits sp;
@@ -894,6 +1318,8 @@ hipError_t launch_d(const AttnArgs &a, hipStream_t stream) {
 }  // namespace
 
 bool attention_supports(int32_t d) { return d == 64 || d == 128; }
+
+void attention_stream_slots(int32_t slots) { g_stream_slots.store(slots, std::memory_order_relaxed); }
 
 const char *attention_config(const AttnArgs &a) {
   static const char *const kCfg[2][2] = {

@@ -64,6 +64,8 @@ struct CombineArgs {
 };
 hipError_t launch_combine(const CombineArgs &a, hipStream_t stream);
 bool attention_supports(int32_t d);
+// Tuning of the streaming form (workgroups that walk runs of query tiles): see svodk_tune_streaming.
+void attention_stream_slots(int32_t slots);
 // Text of the tile configuration launch_attention picks for `a` (for chosen()).
 const char *attention_config(const AttnArgs &a);
 

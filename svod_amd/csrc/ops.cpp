@@ -451,6 +451,8 @@ int svodk_attention_packed(const svodk_tensor *qkv, int32_t heads, int32_t kv_he
   return attend(&q, &k, &v, qkv, opts, out, hip_stream);
 }
 
+void svodk_tune_streaming(int32_t workgroups_per_xcd) { svodk::attention_stream_slots(workgroups_per_xcd); }
+
 // The workspace of a split call (tk/src/ops/attention.rs:285-293).
 int64_t svodk_attention_workspace(const svodk_tensor *q, const svodk_tensor *k, const svodk_attn *opts) {
   if (!well_formed(q) || !well_formed(k) || opts == nullptr || q->rank != 4 || k->rank != 4) return 0;

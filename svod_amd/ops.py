@@ -81,6 +81,8 @@ def load_library() -> ctypes.CDLL:
     lib.svodk_plan_attention.argtypes = [ctypes.c_int32, i32p, ctypes.c_int32, i64p, i64p, ctypes.c_int32, ctypes.c_int32]
     lib.svodk_plan_heads.restype = ctypes.c_int
     lib.svodk_plan_heads.argtypes = [ctypes.c_int32, i32p, ctypes.c_int32, i64p, ctypes.c_int32, ctypes.c_int32]
+    lib.svodk_tune_streaming.restype = None
+    lib.svodk_tune_streaming.argtypes = [ctypes.c_int32]
     lib.svodk_supported.restype = ctypes.c_int
     lib.svodk_last_chosen.restype = ctypes.c_char_p
     lib.svodk_last_error.restype = ctypes.c_char_p
@@ -263,6 +265,13 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, opts: Optional[
                                  ctypes.byref(od), ctypes.c_void_p(_stream(q)))
     _finish("attention", status)
     return out
+
+
+def tune_streaming(workgroups_per_xcd: int) -> None:
+    """n > 0 = attention calls that can (head size 64, lengths or no key mask, no window, no splits)
+    run as n streaming workgroups per XCD, each walking a run of query tiles; n <= 0 (the default)
+    = a workgroup per tile.  Process-wide; results are bit-equal either way."""
+    load_library().svodk_tune_streaming(int(workgroups_per_xcd))
 
 
 def attention_packed(qkv: torch.Tensor, heads: int, kv_heads: int, opts: Optional[Attn] = None,

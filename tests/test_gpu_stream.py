@@ -1,0 +1,77 @@
+"""The streaming form of the attention kernel (workgroups that walk runs of query tiles, the next
+tile's first key blocks and Q rows fetched under the current tile's steps) against the one-tile
+form: a tile's arithmetic is the same steps in the same order, so the two agree bit for bit
+whatever the runs are.  The knob forces streaming with few workgroups, so that runs are long and
+cross heads, batch rows, one-block tiles, odd and even block counts and idle causal waves."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import svod_amd
+from svod_amd import Attn, KeyMask
+from util import Lcg, bf16_tensor, bits, max_abs, to_np
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(autouse=True)
+def automatic_again():
+    yield
+    svod_amd.tune_streaming(0)
+
+
+def case(b, t, tk, h, hkv, d=64, seed=13):
+    g = Lcg(seed)
+    return g.bf16((b, t, h, d)), g.bf16((b, tk, hkv, d)), g.bf16((b, tk, hkv, d))
+
+
+# (name, b, t, tk, h, hkv, causal, lens)
+CASES = [
+    ("ragged lengths, one to eight blocks", 12, 512, 512, 4, 4, False, [64, 65, 512, 1, 128, 300, 0, 449, 191, 192, 193, 7]),
+    ("no mask, odd block count", 3, 300, 320, 2, 2, False, None),
+    ("causal gqa", 4, 384, 384, 8, 2, True, None),
+    ("causal with lengths", 5, 256, 256, 4, 4, True, [256, 50, 0, 129, 64]),
+    ("one query row, many keys", 9, 1, 700, 2, 2, False, [700, 1, 64, 128, 129, 500, 0, 699, 65]),
+    ("cross attention, more heads than units per XCD", 2, 130, 90, 16, 8, False, [90, 33]),
+]
+
+
+@pytest.mark.parametrize("slots", [1, 2, 5], ids=["1 workgroup an XCD", "2", "5"])
+@pytest.mark.parametrize("name,b,t,tk,h,hkv,causal,lens", CASES, ids=[c[0] for c in CASES])
+def test_streaming_is_the_one_tile_kernel_bit_for_bit(device, name, b, t, tk, h, hkv, causal, lens, slots):
+    q, k, v = (bf16_tensor(x, device) for x in case(b, t, tk, h, hkv))
+    keys = KeyMask.none() if lens is None else KeyMask.lens(torch.tensor(lens, dtype=torch.int32, device=device))
+    opts = Attn(causal=causal, keys=keys)
+    svod_amd.tune_streaming(-1)
+    plain = svod_amd.attention(q, k, v, opts)
+    svod_amd.tune_streaming(slots)
+    streamed = svod_amd.attention(q, k, v, opts)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(streamed), bits(plain))
+
+
+def test_streaming_matches_a_direct_softmax(device):
+    b, t, tk, h, hkv = 6, 200, 260, 4, 2
+    q, k, v = case(b, t, tk, h, hkv)
+    lens = [260, 1, 64, 200, 0, 131]
+    svod_amd.tune_streaming(3)
+    got = svod_amd.attention(bf16_tensor(q, device), bf16_tensor(k, device), bf16_tensor(v, device),
+                             Attn(keys=KeyMask.lens(torch.tensor(lens, dtype=torch.int64, device=device))))
+    torch.cuda.synchronize()
+    p = oracle.AttnProblem(q, k, v, key_lens=np.asarray(lens))
+    assert max_abs(to_np(got), oracle.attention_direct(p)) < 2e-2
+    assert not bits(got[4]).any()  # the batch row with no keys
+
+
+def test_streaming_f16_and_packed(device):
+    b, t, h, hkv, d = 5, 190, 4, 2, 64
+    x = torch.from_numpy(oracle.round_f16(Lcg(3).bf16((b, t, (h + 2 * hkv) * d)))).to(torch.float16).to(device)
+    opts = Attn(causal=True, keys=KeyMask.lens(torch.tensor([190, 64, 1, 0, 100], dtype=torch.int32, device=device)))
+    svod_amd.tune_streaming(-1)
+    plain = svod_amd.attention_packed(x, h, hkv, opts)
+    svod_amd.tune_streaming(2)
+    streamed = svod_amd.attention_packed(x, h, hkv, opts)
+    torch.cuda.synchronize()
+    a, c = (y.detach().cpu().view(torch.int16).numpy() for y in (plain, streamed))
+    assert np.array_equal(a, c)

@@ -25,7 +25,10 @@ DEVICE_FLAGS = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang"
 # The attention kernel folds MFMA results with max(): without this every operand is first
 # quieted by a max(x, x) of its own (32 extra VALU ops a step).  Nothing in that kernel tests
 # for NaN, and infinities (the masks) stay honoured.
-EXTRA_FLAGS = {"attention_kernel.hip": ["-fno-honor-nans", "-mllvm", "-amdgpu-kernarg-preload-count=16"]}
+# The last one keeps an atomic add what the source says (one lane, no wait on the spot): the
+# rewrite for wave-uniform operands waits for the answer where the add is issued.
+EXTRA_FLAGS = {"attention_kernel.hip": ["-fno-honor-nans", "-mllvm", "-amdgpu-kernarg-preload-count=16",
+                                        "-mllvm", "-amdgpu-atomic-optimizer-strategy=None"]}
 COMMON_FLAGS = ["-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-command-line-argument"]
 
 

@@ -68,9 +68,10 @@ constexpr int kXcds = 8;       // accelerator dies of an MI355X, each with its o
 constexpr float kLog2e = 1.44269504088896340736f;
 constexpr float kRescaleAbove = 8.0f;  // tk/src/kernels/attention.rs:379
 
-// Workgroups an XCD's item list is split over in the streaming form: 0 = as many as the XCD
-// holds, when the list is long enough to be worth it; > 0 = always that many; < 0 = never stream.
+// Workgroups per XCD of the streaming form; <= 0 = a workgroup per query tile instead.
 std::atomic<int> g_stream_slots{0};
+// Streaming launches so far: each takes the next set of shared counters.
+std::atomic<uint32_t> g_queue_turn{0};
 
 // A ring slot holds a [64 keys, D] tile, rows unpadded (D*2 bytes), filled by
 // buffer_load_dwordx4 ... lds: a wave instruction lands 64 consecutive 16-byte
@@ -597,7 +598,7 @@ __global__ __launch_bounds__(NW * 64, D == 64 ? 3 : 2) void flash_fwd_kernel(
   using TL = Tile<D>;
   using W = Wave<D, NW, F16>;
   constexpr int BQ = NW * kWaveRows;
-  constexpr int KS = W::KS, DB = W::DB, CH = W::CH;
+  constexpr int KS = W::KS, DB = W::DB;
   static_assert(TL::kInstrs % NW == 0, "the tile fills in whole wave instructions per wave");
 
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
@@ -636,6 +637,14 @@ __global__ __launch_bounds__(NW * 64, D == 64 ? 3 : 2) void flash_fwd_kernel(
   w.g = w.lane >> 5;           // half-wave: the k-chunk of MFMA operands
   const int ln = w.lane & 31;  // the query column this lane owns
 
+  // L533-536: len = min(key_lens[b], tk).
+  int len = tk;
+  if (key_lens != nullptr) {
+    long long n = lens_i64 ? ((const long long *)key_lens)[b] : (long long)((const int *)key_lens)[b];
+    n = n < 0 ? 0 : n;
+    len = n < (long long)tk ? (int)n : tk;
+  }
+
   // Elements from a token's row to the next: heads * D and kv_heads * D for separate q, k, v;
   // the fused projection's row for operands read in place (tk/src/ops/attention.rs:104-122).
   const int64_t q_row_stride = q_row_elems;
@@ -650,14 +659,6 @@ __global__ __launch_bounds__(NW * 64, D == 64 ? 3 : 2) void flash_fwd_kernel(
       if (row < t) x = *reinterpret_cast<const u32x4 *>(q_ptr + ks * 16);
       w.qf[ks] = x;
     }
-  }
-
-  // L533-536: len = min(key_lens[b], tk).
-  int len = tk;
-  if (key_lens != nullptr) {
-    long long n = lens_i64 ? ((const long long *)key_lens)[b] : (long long)((const int *)key_lens)[b];
-    n = n < 0 ? 0 : n;
-    len = n < (long long)tk ? (int)n : tk;
   }
 
   // L584-608: key blocks [first, end) hold every key some query of the tile sees.  A negative
@@ -840,13 +841,14 @@ __global__ __launch_bounds__(NW * 64, D == 64 ? 3 : 2) void flash_fwd_kernel(
 }
 
 // ---------------------------------------------------------------------------------------------
-// The streaming form: a workgroup takes a run of consecutive query tiles (items) and walks them
-// as one stream of key blocks.  The last steps of an item fill the ring with the next item's
-// first blocks, and the next item's Q rows are already staged in LDS, so an item starts without
-// the launch, the argument loads, the first fills' flight and the output drain that a
-// workgroup of its own pays; with 1 to 8 key blocks an item (BGE-M3) those are a third of its
-// time.  Runs are fixed from the key lengths alone (no shared counters): every workgroup works
-// out the same split of the XCD's item list into runs of equal estimated cost.
+// The streaming form: a workgroup walks query tiles (items) one after another as a single stream
+// of key blocks.  The last steps of an item fill the ring with the next item's first blocks, and
+// the next item's Q rows are already staged in LDS, so an item starts without the launch, the
+// argument loads, the first fills' flight and the output drain that a workgroup of its own pays;
+// with 1 to 8 key blocks an item (BGE-M3) those are a third of its time.  Each XCD has a list of
+// items; a workgroup starts with two of them by its index and takes the rest from the list's
+// shared counter, one item ahead of need (the oldest workgroup of a CU wins the arbitration for
+// its SIMDs and runs half again as fast as the youngest, so fixed runs would end far apart).
 // ---------------------------------------------------------------------------------------------
 
 // Key blocks of query tile `qt` of a batch row with `len` keys (L596-608), at least 1 (a tile
@@ -860,115 +862,41 @@ __device__ __forceinline__ int item_blocks(int qt, int len, int tk, bool has_len
   return max(end, 1);
 }
 
-// The estimated cost of an item in steps: its key blocks plus one for the switch.
-__device__ __forceinline__ int item_cost(int blocks) { return blocks + 1; }
-
-__device__ __forceinline__ int wave_sum(int x) {
-#pragma unroll
-  for (int m = 32; m >= 1; m >>= 1) x += __shfl_xor(x, m, 64);
-  return x;
+// The key length of batch row b, b wave-uniform, as a scalar load: inside the item loop a vector
+// load would bring a vmcnt wait that also sits out the fills and stores in flight.
+__device__ __forceinline__ int len_of_uniform(const void *key_lens, bool lens_i64, int tk, int b) {
+  if (key_lens == nullptr) return tk;
+  auto word = [&](int byte) {
+    int x;
+    asm volatile("s_load_dword %0, %1, %2\n\ts_waitcnt lgkmcnt(0)" : "=s"(x) : "s"(key_lens), "s"(byte) : "memory");
+    return x;
+  };
+  long long n;
+  if (lens_i64)
+    n = (long long)(((uint64_t)(uint32_t)word(b * 8 + 4) << 32) | (uint32_t)word(b * 8));
+  else
+    n = (long long)word(b * 4);
+  n = n < 0 ? 0 : n;
+  return n < (long long)tk ? (int)n : tk;
 }
-// Exclusive prefix sum over the wave's lanes.
-__device__ __forceinline__ int wave_scan(int x, int lane) {
-  int inc = x;
-#pragma unroll
-  for (int m = 1; m < 64; m <<= 1) {
-    const int up = __shfl_up(inc, m, 64);
-    if (lane >= m) inc += up;
-  }
-  return inc - x;
-}
 
-// One XCD's list of items and the cost model over it.  Unit r of the list is (batch, kv head)
-// number r * 8 + xcd; a unit's items run head-in-group major, then query tile in launch order.
-template <int NW, bool CAUSAL>
-struct ItemList {
-  const Geometry &geo;
-  uint32_t xcd, units_here;
-  const void *key_lens;
-  bool lens_i64;
-  int tk, nqt;
-
-  __device__ __forceinline__ int len_of(int b) const {
-    if (key_lens == nullptr) return tk;
-    long long n = lens_i64 ? ((const long long *)key_lens)[b] : (long long)((const int *)key_lens)[b];
-    n = n < 0 ? 0 : n;
-    return n < (long long)tk ? (int)n : tk;
-  }
-  // The same for a wave-uniform b, as a scalar load: inside the item loop a vector load would
-  // bring a vmcnt wait that also sits out the fills and stores in flight.
-  __device__ __forceinline__ int len_of_uniform(int b) const {
-    if (key_lens == nullptr) return tk;
-    auto word = [&](int byte) {
-      int x;
-      asm volatile("s_load_dword %0, %1, %2\n\ts_waitcnt lgkmcnt(0)" : "=s"(x) : "s"(key_lens), "s"(byte) : "memory");
-      return x;
-    };
-    long long n;
-    if (lens_i64)
-      n = (long long)(((uint64_t)(uint32_t)word(b * 8 + 4) << 32) | (uint32_t)word(b * 8));
-    else
-      n = (long long)word(b * 4);
-    n = n < 0 ? 0 : n;
-    return n < (long long)tk ? (int)n : tk;
-  }
-  // Query tile of place `order` within a head (L524-528: longest first under a causal mask).
-  __device__ __forceinline__ int tile_of(int order) const { return CAUSAL ? nqt - 1 - order : order; }
-  // Cost of one head's tiles of batch row b, and the number of them whose start lies below x.
-  __device__ __forceinline__ int head_cost(int len) const {
-    int c = 0;
-    for (int order = 0; order < nqt; order++)
-      c += item_cost(item_blocks<NW, CAUSAL>(tile_of(order), len, tk, key_lens != nullptr));
-    return c;
-  }
-  __device__ __forceinline__ int tiles_below(int len, int x) const {
-    int c = 0, n = 0;
-    for (int order = 0; order < nqt; order++) {
-      if (c < x) n++;
-      c += item_cost(item_blocks<NW, CAUSAL>(tile_of(order), len, tk, key_lens != nullptr));
-    }
-    return n;
-  }
-  // Items of the list whose start cost lies below `bound`, and the list's whole cost.  Every
-  // lane returns the same numbers.
-  __device__ __forceinline__ void count(int64_t bound_a, int64_t bound_b, int lane, int64_t &total, uint32_t &below_a,
-                                        uint32_t &below_b) const {
-    const int group = (int)geo.group;
-    int64_t before = 0;
-    uint32_t na = 0, nb = 0;
-    for (uint32_t r0 = 0; r0 < units_here; r0 += 64) {
-      const uint32_t r = r0 + lane;
-      int per_head = 0, len = 0;
-      if (r < units_here) {
-        const uint32_t unit = r * kXcds + xcd;
-        len = len_of((int)div_by(unit, geo.kv_heads, geo.kvh_rcp));
-        per_head = head_cost(len);
-      }
-      const int mine = per_head * group;
-      const int64_t start = before + wave_scan(mine, lane);
-      auto inside = [&](int64_t bound) -> uint32_t {
-        if (r >= units_here || bound <= start) return 0u;
-        const int64_t x = bound - start;
-        if (x >= mine) return geo.unit_size;
-        const int heads_done = (int)(x / per_head);
-        return (uint32_t)(heads_done * nqt + tiles_below(len, (int)(x - (int64_t)heads_done * per_head)));
-      };
-      na += (uint32_t)wave_sum((int)inside(bound_a));
-      nb += (uint32_t)wave_sum((int)inside(bound_b));
-      before += wave_sum(mine);
-    }
-    total = before;
-    below_a = na;
-    below_b = nb;
-  }
+// The shared counters of one XCD's item list in one launch.  `next` counts the items handed out
+// beyond every workgroup's first two, `done` the workgroups that have left; the last to leave
+// puts both back to zero for the launch that gets this set next.  Launches take the sets in
+// turn, so a set is met again only kQueueSets launches later.
+struct alignas(64) TileQueue {
+  uint32_t next, done;
 };
+constexpr int kQueueSets = 256;
+__device__ __attribute__((unused)) TileQueue g_tile_queues[kQueueSets][kXcds];
 
 template <int D, int NW, bool CAUSAL, bool F16>
 __global__ __launch_bounds__(NW * 64, 3) void flash_stream_kernel(
     uint32_t unit_size, uint32_t unit_rcp, uint32_t nqt_u, uint32_t nqt_rcp, uint32_t kvh_u, uint32_t kvh_rcp,
     uint32_t units, uint32_t heads_group, const void *__restrict__ key_lens, const uint16_t *__restrict__ q, int32_t t,
     uint32_t tk_lens64, const uint16_t *__restrict__ k, const uint16_t *__restrict__ v,
-    uint16_t *__restrict__ o, float scale, int32_t q_row_elems, int32_t kv_row_elems, uint32_t slots) {
+    uint16_t *__restrict__ o, float scale, int32_t q_row_elems, int32_t kv_row_elems, uint32_t slots,
+    uint32_t queue_set) {
 #if defined(__HIP_DEVICE_COMPILE__)
   const Geometry geo = {unit_size, unit_rcp, nqt_u, nqt_rcp, kvh_u, kvh_rcp, heads_group >> 16, units};
   const int heads = (int)(heads_group & 0xffffu);
@@ -977,11 +905,14 @@ __global__ __launch_bounds__(NW * 64, 3) void flash_stream_kernel(
   using TL = Tile<D>;
   using W = Wave<D, NW, F16>;
   constexpr int BQ = NW * kWaveRows;
-  constexpr int KS = W::KS, DB = W::DB, CH = W::CH;
+  constexpr int KS = W::KS, DB = W::DB;
   constexpr int kStageRows = 1024 / TL::kRowBytes;                  // rows a wave instruction stages
   constexpr int kStageInstrs = kWaveRows * TL::kRowBytes / 1024;    // per wave and item
+  constexpr int kStageBytes = BQ * TL::kRowBytes;
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
   uint8_t *stage = smem + TL::kLds;  // [BQ rows][D] of the next item's Q
+  // Two words after the stage: the counter's answers, written by wave 0, read by every wave.
+  LDS_PTR(uint32_t) answers = (LDS_PTR(uint32_t))(smem + TL::kLds + kStageBytes);
 
   W w;
   const int tid = __builtin_amdgcn_workitem_id_x();
@@ -990,23 +921,30 @@ __global__ __launch_bounds__(NW * 64, 3) void flash_stream_kernel(
   w.g = w.lane >> 5;
   const int ln = w.lane & 31;
 
-  // ---- this workgroup's run of the XCD's list: items [run_first, run_end).
+  // ---- this workgroup's place: XCD `xcd` (workgroups are dealt over the XCDs in turn), number
+  // `slot` of `slots` on it.  Items of the XCD's list: unit r of the list is (batch, kv head)
+  // number r * 8 + xcd; a unit's items run head-in-group major, then query tile in launch order.
   const uint32_t wg = __builtin_amdgcn_workgroup_id_x();
   const uint32_t xcd = wg % kXcds, slot = wg / kXcds;
   const uint32_t units_here = geo.units > xcd ? (geo.units - xcd + kXcds - 1) / kXcds : 0;
-  const ItemList<NW, CAUSAL> list = {geo, xcd, units_here, key_lens, lens_i64, tk, (int)geo.nqt};
-  uint32_t run_first, run_end;
-  {
-    // Two passes: the list's whole cost, then the items below this slot's two bounds.
-    int64_t total;
-    uint32_t a, b;
-    list.count(0, 0, w.lane, total, a, b);
-    const int64_t lo = total * slot / slots, hi = total * (slot + 1) / slots;
-    list.count(lo, hi, w.lane, total, a, b);
-    run_first = __builtin_amdgcn_readfirstlane(a);
-    run_end = __builtin_amdgcn_readfirstlane(b);
+  const uint32_t total = units_here * geo.unit_size;
+  TileQueue *queue = &g_tile_queues[queue_set][xcd];
+  // Every workgroup of the launch comes by here exactly once, after its last look at `next`.
+  auto leave = [&]() {
+    // The lane number afresh, not a register kept from the kernel's start.
+    const uint32_t lane_now = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+    if (w.wave == 0 && lane_now == 0) {
+      const uint32_t before = __hip_atomic_fetch_add(&queue->done, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (before == slots - 1) {
+        __hip_atomic_store(&queue->next, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&queue->done, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+  };
+  if (slot >= total) {
+    leave();
+    return;
   }
-  if (run_first >= run_end) return;
 
   // ---- call constants
   const int64_t o_row_stride = (int64_t)heads * D;
@@ -1055,9 +993,9 @@ __global__ __launch_bounds__(NW * 64, 3) void flash_stream_kernel(
     it.b = (int)div_by(unit, geo.kv_heads, geo.kvh_rcp);
     const int kvh = (int)(unit - (uint32_t)it.b * geo.kv_heads);
     it.h = kvh * (int)geo.group + (int)head_in_group;
-    const int qt = list.tile_of(order);
+    const int qt = CAUSAL ? (int)geo.nqt - 1 - order : order;  // L524-528: longest first under a causal mask
     it.q_off = qt * BQ;
-    it.len = list.len_of_uniform(it.b);
+    it.len = len_of_uniform(key_lens, lens_i64, tk, it.b);
     it.end = item_blocks<NW, CAUSAL>(qt, it.len, tk, key_lens != nullptr);
     it.k_base = (const uint8_t *)(k + (int64_t)it.b * tk * kv_row_elems + (int64_t)kvh * D);
     it.v_base = (const uint8_t *)(v + (int64_t)it.b * tk * kv_row_elems + (int64_t)kvh * D);
@@ -1089,7 +1027,7 @@ __global__ __launch_bounds__(NW * 64, 3) void flash_stream_kernel(
   };
 
   // ---- the first item: K(0), V(0), K(1) and its Q rows in flight, then everything lands.
-  Item cur = item(run_first);
+  Item cur = item(slot);
   auto adopt = [&](const Item &it) {
     int lane = w.lane;
     asm volatile("" : "+v"(lane));
@@ -1116,18 +1054,25 @@ __global__ __launch_bounds__(NW * 64, 3) void flash_stream_kernel(
   const f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
   for (int db = 0; db < DB; db++) w.acc[db] = zero;
+  // The second item is fixed as well; the counter hands out the items from 2 * slots on.
+  bool more_items = slot + slots < total;
+  Item nxt = cur;
+  if (more_items) nxt = item(slot + slots);
   __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
   __syncthreads();
 
-  for (uint32_t s = run_first; s < run_end; s++) {
+  for (uint32_t round = 0;; round++) {
     // ---- the item after this one: its first blocks ride this item's last steps.
-    const bool more_items = s + 1 < run_end;
-    Item nxt = cur;
-    if (more_items) nxt = item(s + 1);
     w.nxt_end = more_items ? nxt.end : 0;
     w.nxt_k = nxt.k_base;
     w.nxt_v = nxt.v_base;
     w.nxt_bytes = nxt.kv_bytes;
+    // ---- the item after that: wave 0 asks the counter now and passes the answer on through LDS
+    // before the barrier below; every wave reads it after this item's steps.
+    uint32_t answer = 0;
+    const bool asking = more_items && w.wave == 0;
+    if (asking && w.lane == 0)
+      answer = __hip_atomic_fetch_add(&queue->next, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     // ---- this item's Q rows from the stage to registers; the stage is then free for the next
     // item's rows, which have the whole item to arrive.
     {
@@ -1157,6 +1102,7 @@ __global__ __launch_bounds__(NW * 64, 3) void flash_stream_kernel(
       if (on_edge<D, NW, CAUSAL>(w, 0, kbits0)) mask_scores<D, NW, CAUSAL>(w, 0, kbits0, sv);
       bm = row_max(sv);
     }
+    if (asking && w.lane == 0) answers[round & 1] = answer;
     // Step 0 refills the K slot those scores were read from: every wave has read it first.
     __syncthreads();
 
@@ -1200,11 +1146,15 @@ __global__ __launch_bounds__(NW * 64, 3) void flash_stream_kernel(
 #pragma unroll
       for (int db = 0; db < DB; db++) w.acc[db] = zero;
     }
-    if (more_items) {
-      cur = nxt;
-      adopt(cur);
-    }
+    if (!more_items) break;
+    // Every step ends in a barrier and an item has at least one, so wave 0's answer is there.
+    const uint32_t after = 2 * slots + (uint32_t)__builtin_amdgcn_readfirstlane((int)answers[round & 1]);
+    cur = nxt;
+    adopt(cur);
+    more_items = after < total;
+    if (more_items) nxt = item(after);
   }
+  leave();
 #endif  // __HIP_DEVICE_COMPILE__
 }
 
@@ -1212,7 +1162,7 @@ template <int D, int NW, bool CAUSAL, bool F16>
 hipError_t launch_stream(const AttnArgs &a, hipStream_t stream, int64_t slots, const Geometry &geo, int64_t q_row,
                          int64_t kv_row) {
   using TL = Tile<D>;
-  constexpr int smem = TL::kLds + NW * kWaveRows * TL::kRowBytes;
+  constexpr int smem = TL::kLds + NW * kWaveRows * TL::kRowBytes + 16;  // ring, Q stage, two words
   auto kernel = flash_stream_kernel<D, NW, CAUSAL, F16>;
   static std::atomic<uint64_t> configured{0};
   int device = 0;
@@ -1229,7 +1179,8 @@ hipError_t launch_stream(const AttnArgs &a, hipStream_t stream, int64_t slots, c
   hipLaunchKernelGGL(kernel, dim3((uint32_t)(slots * kXcds)), dim3(NW * 64), smem, stream, geo.unit_size, geo.unit_rcp,
                      geo.nqt, geo.nqt_rcp, geo.kv_heads, geo.kvh_rcp, geo.units, heads_group, a.key_lens,
                      (const uint16_t *)a.q, a.t, tk_lens64, (const uint16_t *)a.k, (const uint16_t *)a.v,
-                     (uint16_t *)a.o, a.scale, (int32_t)q_row, (int32_t)kv_row, (uint32_t)slots);
+                     (uint16_t *)a.o, a.scale, (int32_t)q_row, (int32_t)kv_row, (uint32_t)slots,
+                     g_queue_turn.fetch_add(1u, std::memory_order_relaxed) % kQueueSets);
   return hipGetLastError();
 }
 

@@ -1,8 +1,9 @@
-"""The streaming form of the attention kernel (workgroups that walk runs of query tiles, the next
-tile's first key blocks and Q rows fetched under the current tile's steps) against the one-tile
-form: a tile's arithmetic is the same steps in the same order, so the two agree bit for bit
-whatever the runs are.  The knob forces streaming with few workgroups, so that runs are long and
-cross heads, batch rows, one-block tiles, odd and even block counts and idle causal waves."""
+"""The streaming form of the attention kernel (workgroups that walk query tiles one after another,
+the next tile's first key blocks and Q rows fetched under the current tile's steps, tiles handed
+out by a shared counter) against the one-tile form: a tile's arithmetic is the same steps in the
+same order, so the two agree bit for bit whichever workgroup takes which tile.  The knob forces
+streaming with few workgroups, so that walks are long and cross heads, batch rows, one-block
+tiles, odd and even block counts and idle causal waves."""
 import numpy as np
 import pytest
 import torch
@@ -37,7 +38,7 @@ CASES = [
 ]
 
 
-@pytest.mark.parametrize("slots", [1, 2, 5], ids=["1 workgroup an XCD", "2", "5"])
+@pytest.mark.parametrize("slots", [1, 2, 5, 96], ids=["1 workgroup an XCD", "2", "5", "more workgroups than tiles"])
 @pytest.mark.parametrize("name,b,t,tk,h,hkv,causal,lens", CASES, ids=[c[0] for c in CASES])
 def test_streaming_is_the_one_tile_kernel_bit_for_bit(device, name, b, t, tk, h, hkv, causal, lens, slots):
     q, k, v = (bf16_tensor(x, device) for x in case(b, t, tk, h, hkv))
@@ -75,3 +76,41 @@ def test_streaming_f16_and_packed(device):
     torch.cuda.synchronize()
     a, c = (y.detach().cpu().view(torch.int16).numpy() for y in (plain, streamed))
     assert np.array_equal(a, c)
+
+
+def test_counters_are_left_at_zero_for_the_launch_that_meets_them_next(device):
+    """Launches take the sets of shared counters in turn (256 of them): well past one turn of the
+    sets, every launch still hands out every tile once."""
+    q, k, v = (bf16_tensor(x, device) for x in case(3, 260, 200, 4, 2, seed=29))
+    opts = Attn(keys=KeyMask.lens(torch.tensor([200, 77, 129], dtype=torch.int32, device=device)))
+    svod_amd.tune_streaming(-1)
+    plain = bits(svod_amd.attention(q, k, v, opts))
+    svod_amd.tune_streaming(2)
+    out = torch.empty_like(q)
+    for launch in range(600):
+        if launch % 100 == 99:
+            out.zero_()
+        svod_amd.attention(q, k, v, opts, out=out)
+        if launch % 100 == 99:
+            torch.cuda.synchronize()
+            assert np.array_equal(bits(out), plain), launch
+
+
+def test_two_streams_at_once_do_not_share_counters(device):
+    q1, k1, v1 = (bf16_tensor(x, device) for x in case(4, 512, 512, 8, 8, seed=5))
+    q2, k2, v2 = (bf16_tensor(x, device) for x in case(2, 700, 700, 4, 2, seed=6))
+    causal = Attn(causal=True)
+    svod_amd.tune_streaming(-1)
+    want1, want2 = bits(svod_amd.attention(q1, k1, v1)), bits(svod_amd.attention(q2, k2, v2, causal))
+    svod_amd.tune_streaming(3)
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    o1, o2 = torch.empty_like(q1), torch.empty_like(q2)
+    torch.cuda.synchronize()
+    for _ in range(20):
+        with torch.cuda.stream(s1):
+            svod_amd.attention(q1, k1, v1, out=o1)
+        with torch.cuda.stream(s2):
+            svod_amd.attention(q2, k2, v2, causal, out=o2)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(o1), want1)
+    assert np.array_equal(bits(o2), want2)

@@ -73,9 +73,10 @@ typedef enum svodk_key_mask {
 
 /*
  * Attn of tk/src/ops/attention.rs:60-86.  Zero-initialise, then set fields.
- * Options this library has no kernel for (chunk, seg_start, cache, bias) are
- * still validated as the reference validates them and then answered
- * with SVODK_GRAPH_CONFIG.
+ * Windows, chunk masks and segment starts (I32 or I64, non-decreasing along T)
+ * have kernels, alone or together with every other mask.  Options this
+ * library has no kernel for (cache, bias) are still validated as the
+ * reference validates them and then answered with SVODK_GRAPH_CONFIG.
  *
  * `splits` > 1 asks for key splits (tk/src/ops/attention.rs:79, 280-302): the
  * count is capped at the number of 64-key blocks of Tk (split_ranked, :405-410);

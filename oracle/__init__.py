@@ -46,6 +46,33 @@ _f32p = ctypes.POINTER(ctypes.c_float)
 _f64p = ctypes.POINTER(ctypes.c_double)
 _i32p = ctypes.POINTER(ctypes.c_int32)
 _u8p = ctypes.POINTER(ctypes.c_uint8)
+
+
+class _Ranges(ctypes.Structure):
+    """``svod_oracle_ranges``: the chunk mask and the segment starts."""
+
+    _fields_ = [("chunk_size", ctypes.c_int32), ("chunk_has_left", ctypes.c_int32), ("chunk_left", ctypes.c_int32),
+                ("chunk_right", ctypes.c_int32), ("seg_start", ctypes.POINTER(ctypes.c_int32))]
+
+
+_rangesp = ctypes.POINTER(_Ranges)
+
+
+def _ranges(chunk, seg_start):
+    """(pointer or None, what must stay alive) for ``chunk = (size, left or None, right)`` and ``seg_start [B,T]``."""
+    if chunk is None and seg_start is None:
+        return None, None
+    r = _Ranges()
+    seg = None
+    if chunk is not None:
+        size, left, right = chunk
+        r.chunk_size, r.chunk_has_left = int(size), int(left is not None)
+        r.chunk_left, r.chunk_right = int(left or 0), int(right)
+    if seg_start is not None:
+        seg = np.ascontiguousarray(seg_start, dtype=np.int32)
+        r.seg_start = seg.ctypes.data_as(ctypes.POINTER(ctypes.c_int32))
+    return ctypes.pointer(r), (r, seg)
+
 _i32 = ctypes.c_int32
 
 
@@ -69,10 +96,10 @@ def _declare(l: ctypes.CDLL) -> None:
     l.svod_oracle_rope_table.restype = None
     l.svod_oracle_rope_table.argtypes = [ctypes.c_double, _i32, _i32, _f32p, _f32p]
     l.svod_oracle_visible.restype = None
-    l.svod_oracle_visible.argtypes = [_i32, _i32, _i32, _i32, _i32, _i32, _i32p, _i32p, _i32, _u8p]
+    l.svod_oracle_visible.argtypes = [_i32, _i32, _i32, _i32, _i32, _i32, _i32p, _i32p, _i32, _rangesp, _u8p]
     l.svod_oracle_visible_pairs.restype = ctypes.c_int64
     l.svod_oracle_visible_pairs.argtypes = [_i32, _i32, _i32, _i32, _i32p]
-    common = [_i32] * 6 + [_i32, _i32, _i32, ctypes.c_float, _i32p, _i32p, _i32]
+    common = [_i32] * 6 + [_i32, _i32, _i32, ctypes.c_float, _i32p, _i32p, _i32, _rangesp]
     l.svod_oracle_attention_direct.restype = ctypes.c_int
     l.svod_oracle_attention_direct.argtypes = common + [_f32p, _f32p, _f32p, _f64p, _i32]
     l.svod_oracle_attention_graph.restype = ctypes.c_int
@@ -178,6 +205,8 @@ class AttnProblem:
     key_lens: Optional[np.ndarray] = None  # [B] int
     key_mask: Optional[np.ndarray] = None  # [B, Tk] nonzero = visible
     window: Optional[tuple] = None
+    chunk: Optional[tuple] = None  # (size, left or None, right): Chunk of tk/src/ops/attention.rs:39-50
+    seg_start: Optional[np.ndarray] = None  # [B, T] int
     scale: Optional[float] = None
     bf16: bool = True
 
@@ -196,9 +225,10 @@ class AttnProblem:
         lens = None if self.key_lens is None else np.ascontiguousarray(self.key_lens, dtype=np.int32)
         mask = None if self.key_mask is None else np.ascontiguousarray(np.asarray(self.key_mask) != 0, dtype=np.int32)
         wl, wr = (-1, -1) if self.window is None else self.window
-        keep = (lens, mask)
+        ranges, alive = _ranges(self.chunk, self.seg_start)
+        keep = (lens, mask, alive)
         args = [b, t, tk, h, hkv, d, int(self.causal), wl, wr, ctypes.c_float(self.scale_f32()),
-                _ptr(lens, _i32p), _ptr(mask, _i32p), tk]
+                _ptr(lens, _i32p), _ptr(mask, _i32p), tk, ranges]
         return args, keep
 
 
@@ -236,13 +266,14 @@ def attention_flash(p: AttnProblem, bq: int = 64, bkv: int = 64, threads: int = 
     return out
 
 
-def visible(batch, t, tk, causal=False, key_lens=None, key_mask=None, window=None) -> np.ndarray:
+def visible(batch, t, tk, causal=False, key_lens=None, key_mask=None, window=None, chunk=None, seg_start=None) -> np.ndarray:
     """uint8 [B,T,Tk]: 1 where key j is visible to query i (negated ``hidden`` of attention.rs:138-148)."""
     lens = None if key_lens is None else np.ascontiguousarray(key_lens, dtype=np.int32)
     mask = None if key_mask is None else np.ascontiguousarray(np.asarray(key_mask) != 0, dtype=np.int32)
     wl, wr = (-1, -1) if window is None else window
     out = np.empty((batch, t, tk), dtype=np.uint8)
-    lib().svod_oracle_visible(batch, t, tk, int(causal), wl, wr, _ptr(lens, _i32p), _ptr(mask, _i32p), tk, _ptr(out, _u8p))
+    ranges, _alive = _ranges(chunk, seg_start)
+    lib().svod_oracle_visible(batch, t, tk, int(causal), wl, wr, _ptr(lens, _i32p), _ptr(mask, _i32p), tk, ranges, _ptr(out, _u8p))
     return out
 
 

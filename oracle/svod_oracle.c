@@ -18,7 +18,12 @@
  *       pinned by the recurrence constants (tk/src/test/unit/mod.rs:442-445)
  *       and an independent big-integer evaluation in Python.
  *   svod_oracle_visible
- *       pinned by brute-force enumeration of the predicate on tiny shapes.
+ *       pinned by brute-force enumeration of the predicate on tiny shapes,
+ *       the chunk and segment arms also by masks that must equal other masks
+ *       (chunks of one row = a window or a causal mask; one chunk over
+ *       everything and segments from key 0 hide nothing) and by packed
+ *       segments / self-contained chunks giving the attention of each part
+ *       computed alone.
  *   svod_oracle_attention_direct
  *       pinned against torch.nn.functional.scaled_dot_product_attention in
  *       float64 (a library routine, not the reference) and closed forms
@@ -172,6 +177,15 @@ void svod_oracle_rope_table(double theta, int32_t seq_len, int32_t head_dim, flo
 /* ------------------------------------------------------------------ */
 /* the attention problem                                               */
 /* ------------------------------------------------------------------ */
+/* The masks over (query row, key) beyond causal, window and the key masks
+ * (Attn::chunk and Attn::seg_start, tk/src/ops/attention.rs:66-71). */
+typedef struct {
+  int32_t chunk_size;     /* 0: no chunk mask */
+  int32_t chunk_has_left; /* Chunk::left is Some */
+  int32_t chunk_left, chunk_right;
+  const int32_t *seg_start; /* [batch, t] or NULL */
+} svod_oracle_ranges;
+
 typedef struct {
   int32_t batch, t, tk, heads, kv_heads, d;
   int32_t causal;
@@ -181,10 +195,12 @@ typedef struct {
   const int32_t *key_mask; /* [batch, mask_stride], nonzero = visible, or NULL */
   int32_t mask_stride;
   int32_t bf16_stream; /* 1: q/k/v/o are bf16 values; 0: f32 */
+  const svod_oracle_ranges *ranges; /* or NULL */
 } attn_problem;
 
-/* hidden(j) of tk/src/test/unit/attention.rs:138-148, the in-scope arms:
- * j >= len || (causal && j > i) || window || key_mask == 0.
+/* hidden(j) of tk/src/test/unit/attention.rs:133-148, the arms without a cache:
+ * j >= len || (causal && j > i) || window || chunked(j) || key_mask == 0 || j < seg_start[b, i],
+ * chunked(j) = j/size > i/size + right || (left given && j/size + left < i/size).
  * The kernel's keep predicate (tk/src/kernels/attention.rs:641-697) is its
  * negation: col <= row, col < len (len = min(key_lens[b], tk), L533-536),
  * row <= col + left && col <= row + right, key_mask != 0. */
@@ -198,14 +214,25 @@ static inline int hidden(const attn_problem *p, int32_t b, int32_t i, int32_t j)
   if (p->causal && j > i) return 1;
   if (p->window_left >= 0 && (j + p->window_left < i || j > i + p->window_right)) return 1;
   if (p->key_mask && p->key_mask[(int64_t)b * p->mask_stride + j] == 0) return 1;
+  if (p->ranges) {
+    const svod_oracle_ranges *r = p->ranges;
+    if (r->chunk_size > 0) {
+      const int64_t cj = j / r->chunk_size, ci = i / r->chunk_size;
+      if (cj > ci + r->chunk_right) return 1;
+      if (r->chunk_has_left && cj + r->chunk_left < ci) return 1;
+    }
+    /* Rows past t (a tile's overhang) read no segment start: the bounded view gives 0 (L573-576). */
+    if (r->seg_start && i < p->t && j < r->seg_start[(int64_t)b * p->t + i]) return 1;
+  }
   return 0;
 }
 
 /* Visibility of every (b, i, j): out[b][i][j] = 1 where key j is seen by query i. */
 void svod_oracle_visible(int32_t batch, int32_t t, int32_t tk, int32_t causal, int32_t window_left,
                          int32_t window_right, const int32_t *key_lens, const int32_t *key_mask, int32_t mask_stride,
-                         uint8_t *out) {
-  attn_problem p = {batch, t, tk, 1, 1, 1, causal, window_left, window_right, 1.0f, key_lens, key_mask, mask_stride, 0};
+                         const svod_oracle_ranges *ranges, uint8_t *out) {
+  attn_problem p = {batch, t, tk, 1, 1, 1, causal, window_left, window_right, 1.0f, key_lens, key_mask, mask_stride, 0,
+                    ranges};
   for (int32_t b = 0; b < batch; b++)
     for (int32_t i = 0; i < t; i++)
       for (int32_t j = 0; j < tk; j++) out[((int64_t)b * t + i) * tk + j] = (uint8_t)!hidden(&p, b, i, j);
@@ -311,10 +338,11 @@ static int check_problem(const attn_problem *p) {
  * stream is bf16); out [B,T,H,D] f64, unrounded. */
 int svod_oracle_attention_direct(int32_t batch, int32_t t, int32_t tk, int32_t heads, int32_t kv_heads, int32_t d,
                                  int32_t causal, int32_t window_left, int32_t window_right, float scale,
-                                 const int32_t *key_lens, const int32_t *key_mask, int32_t mask_stride, const float *q,
-                                 const float *k, const float *v, double *out, int32_t threads) {
+                                 const int32_t *key_lens, const int32_t *key_mask, int32_t mask_stride,
+                                 const svod_oracle_ranges *ranges, const float *q, const float *k, const float *v,
+                                 double *out, int32_t threads) {
   direct_ctx c = {{batch, t, tk, heads, kv_heads, d, causal, window_left, window_right, scale, key_lens, key_mask,
-                   mask_stride, 0},
+                   mask_stride, 0, ranges},
                   q, k, v, out};
   int rc = check_problem(&c.p);
   if (rc) return rc;
@@ -361,7 +389,7 @@ static void graph_slice(const void *ctxp, int32_t b, int32_t h) {
   for (int32_t i = 0; i < p->t; i++) {
     const float *qi = c->q + ((int64_t)b * p->t + i) * stride + (int64_t)h * d;
     float *oi = c->out + ((int64_t)b * p->t + i) * stride + (int64_t)h * d;
-    int any_mask = p->causal || p->window_left >= 0 || p->key_lens || p->key_mask;
+    int any_mask = p->causal || p->window_left >= 0 || p->key_lens || p->key_mask || p->ranges;
     float mx = -INFINITY;
     for (int32_t j = 0; j < tk; j++) {
       const float *kj = kh + (int64_t)j * d;
@@ -410,10 +438,10 @@ static void graph_slice(const void *ctxp, int32_t b, int32_t h) {
 int svod_oracle_attention_graph(int32_t batch, int32_t t, int32_t tk, int32_t heads, int32_t kv_heads, int32_t d,
                                 int32_t causal, int32_t window_left, int32_t window_right, float scale,
                                 const int32_t *key_lens, const int32_t *key_mask, int32_t mask_stride,
-                                int32_t bf16_stream, const float *q, const float *k, const float *v, float *out,
-                                int32_t threads) {
+                                const svod_oracle_ranges *ranges, int32_t bf16_stream, const float *q, const float *k,
+                                const float *v, float *out, int32_t threads) {
   graph_ctx c = {{batch, t, tk, heads, kv_heads, d, causal, window_left, window_right, scale, key_lens, key_mask,
-                  mask_stride, bf16_stream},
+                  mask_stride, bf16_stream, ranges},
                  q, k, v, out};
   int rc = check_problem(&c.p);
   if (rc) return rc;
@@ -473,6 +501,19 @@ static void flash_slice(const void *ctxp, int32_t b, int32_t h) {
       int32_t lo = (q_off > p->window_left ? q_off : p->window_left) - p->window_left;
       if (lo / bkv > first) first = lo / bkv;
     }
+    const svod_oracle_ranges *rg = p->ranges;
+    /* L580-583: the tile's first and last query chunks. */
+    const int32_t csize = rg ? rg->chunk_size : 0;
+    const int32_t cq0 = csize > 0 ? q_off / csize : 0, cq1 = csize > 0 ? (q_off + (bq - 1)) / csize : 0;
+    if (csize > 0 && rg->chunk_has_left) {
+      int64_t lo = (int64_t)((cq0 > rg->chunk_left ? cq0 : rg->chunk_left) - rg->chunk_left) * csize / bkv;
+      if (lo > first) first = (int32_t)lo;
+    }
+    if (rg && rg->seg_start) {
+      /* L573-579, L594-596: the segment start of the tile's first row. */
+      int32_t lo = rg->seg_start[(int64_t)b * t + q_off] / bkv;
+      if (lo > first) first = lo;
+    }
     if (p->causal) {
       int32_t e = (q_off + bq + bkv - 1) / bkv;
       if (e < end) end = e;
@@ -480,6 +521,10 @@ static void flash_slice(const void *ctxp, int32_t b, int32_t h) {
     if (p->window_left >= 0) {
       int32_t e = (q_off + bq + p->window_right + bkv - 1) / bkv;
       if (e < end) end = e;
+    }
+    if (csize > 0) {
+      int64_t e = ((int64_t)(cq1 + 1 + rg->chunk_right) * csize + (bkv - 1)) / bkv;
+      if (e < end) end = (int32_t)e;
     }
     if (p->key_lens) {
       int32_t e = (len + bkv - 1) / bkv;
@@ -601,10 +646,10 @@ static void flash_slice(const void *ctxp, int32_t b, int32_t h) {
 int svod_oracle_attention_flash(int32_t batch, int32_t t, int32_t tk, int32_t heads, int32_t kv_heads, int32_t d,
                                 int32_t causal, int32_t window_left, int32_t window_right, float scale,
                                 const int32_t *key_lens, const int32_t *key_mask, int32_t mask_stride,
-                                int32_t bf16_stream, int32_t bq, int32_t bkv, const float *q, const float *k,
-                                const float *v, float *out, int32_t threads) {
+                                const svod_oracle_ranges *ranges, int32_t bf16_stream, int32_t bq, int32_t bkv,
+                                const float *q, const float *k, const float *v, float *out, int32_t threads) {
   flash_ctx c = {{batch, t, tk, heads, kv_heads, d, causal, window_left, window_right, scale, key_lens, key_mask,
-                  mask_stride, bf16_stream},
+                  mask_stride, bf16_stream, ranges},
                  bq, bkv, q, k, v, out, 1};
   int rc = check_problem(&c.p);
   if (rc) return rc;
@@ -618,10 +663,11 @@ int svod_oracle_attention_flash(int32_t batch, int32_t t, int32_t tk, int32_t he
 int svod_oracle_attention_flash_split(int32_t batch, int32_t t, int32_t tk, int32_t heads, int32_t kv_heads, int32_t d,
                                       int32_t causal, int32_t window_left, int32_t window_right, float scale,
                                       const int32_t *key_lens, const int32_t *key_mask, int32_t mask_stride,
-                                      int32_t bf16_stream, int32_t bq, int32_t bkv, int32_t splits, const float *q,
-                                      const float *k, const float *v, float *out, int32_t threads) {
+                                      const svod_oracle_ranges *ranges, int32_t bf16_stream, int32_t bq, int32_t bkv,
+                                      int32_t splits, const float *q, const float *k, const float *v, float *out,
+                                      int32_t threads) {
   flash_ctx c = {{batch, t, tk, heads, kv_heads, d, causal, window_left, window_right, scale, key_lens, key_mask,
-                  mask_stride, bf16_stream},
+                  mask_stride, bf16_stream, ranges},
                  bq, bkv, q, k, v, out, splits};
   int rc = check_problem(&c.p);
   if (rc) return rc;

@@ -156,7 +156,7 @@ __device__ __forceinline__ i32x4 make_rsrc(const void *base, int64_t bytes) {
 }
 
 // Everything a wave carries through the key loop.
-template <int D, int NW, bool F16>
+template <int D, int NW, bool F16, bool STREAM, bool RANGED>
 struct Wave {
   static constexpr int KS = D / 16;  // k-steps of the score product
   static constexpr int DB = D / 32;  // 32-row blocks of O^T
@@ -175,10 +175,13 @@ struct Wave {
   int wave_first_row, my_row;
   bool positive;
   float c_exp, unit, limit;
-  // A window (tk/src/ops/attention.rs:64-65): query i sees keys [i - reach_left, i + reach_right].
-  // reach_right is 0 under a causal mask; both are unused unless `windowed`.
-  bool windowed;
-  int reach_left, reach_right;
+  // Per-row key ranges (a window, a chunk mask, segment starts: tk/src/ops/attention.rs:64-71):
+  // this lane's query sees keys [row_lo, row_hi] only, a causal mask already folded into row_hi.
+  // Both are non-decreasing in the row, so the wave's first and last rows bound every row's:
+  // lo_last, hi_first and hi_last are theirs.  All unused unless `ranged`.
+  static constexpr bool ranged = RANGED;
+  int row_lo, row_hi;
+  int lo_last, hi_first, hi_last;
   // per-lane addressing
   int k_src, v_src;  // global byte offsets of this lane's chunk in this wave's first fill of a tile
   int k_read[KS], v_read[DB];
@@ -187,7 +190,7 @@ struct Wave {
   f32x16 acc[DB];
   float m_run, l_run;
   int mask_next;
-  // A streaming workgroup's next item (nxt_end = 0: none, as in the one-item kernel): this item's
+  // A streaming workgroup's next item (STREAM; nxt_end = 0: none): this item's
   // last steps request its first blocks.  The next item's blocks follow this item's at an even
   // position of the ring (end_even = end rounded up), so every item starts in slot 0.
   const uint8_t *nxt_k, *nxt_v;
@@ -199,8 +202,8 @@ struct Wave {
 // it knows about as aliasing every later LDS read and would park the wave on the NEXT tile's
 // fills in the middle of the current tile.  The kernel waits for them itself (vmcnt(0) before
 // the barrier that ends a step).  m0 carries the LDS address of a wave instruction's 1 KiB.
-template <int D, int NW, bool F16>
-__device__ __forceinline__ void fill_tile(const Wave<D, NW, F16> &w, const uint8_t *base, int64_t bytes, int blk,
+template <int D, int NW, bool F16, bool STREAM, bool RANGED>
+__device__ __forceinline__ void fill_tile(const Wave<D, NW, F16, STREAM, RANGED> &w, const uint8_t *base, int64_t bytes, int blk,
                                           int lds_at, int src) {
   // This wave's fills of a tile are NW instructions apart; the swizzle repeats with that period,
   // so they share the lanes' offsets and differ in the descriptor's base.
@@ -208,7 +211,7 @@ __device__ __forceinline__ void fill_tile(const Wave<D, NW, F16> &w, const uint8
   static_assert((NW * kRowsPer) % 16 == 0, "the swizzle repeats from one of a wave's fills to its next");
   const int64_t off = (int64_t)blk * kBkv * w.kv_row_bytes;
 #pragma unroll
-  for (int i = 0; i < Wave<D, NW, F16>::CH; i++) {
+  for (int i = 0; i < Wave<D, NW, F16, STREAM, RANGED>::CH; i++) {
     const int64_t at = off + (int64_t)(NW * i * kRowsPer) * w.kv_row_bytes;
     const i32x4 r = make_rsrc(base + at, bytes - at);
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
@@ -219,27 +222,27 @@ __device__ __forceinline__ void fill_tile(const Wave<D, NW, F16> &w, const uint8
 }
 // Block `n` of the stream of blocks that starts with this item's: the item's own while n < end,
 // then (past the padding to an even count) the next item's.  Nothing past either.
-template <int D, int NW, bool F16>
-__device__ __forceinline__ void fill_k(const Wave<D, NW, F16> &w, int n, int slot) {
+template <int D, int NW, bool F16, bool STREAM, bool RANGED>
+__device__ __forceinline__ void fill_k(const Wave<D, NW, F16, STREAM, RANGED> &w, int n, int slot) {
   const int at = w.lds0 + slot * Tile<D>::kBytes;
   if (n < w.end)
     fill_tile<D, NW>(w, w.k_base, w.kv_bytes, n, at, w.k_src);
-  else if (n >= w.end_even && n - w.end_even < w.nxt_end)
+  else if (STREAM && n >= w.end_even && n - w.end_even < w.nxt_end)
     fill_tile<D, NW>(w, w.nxt_k, w.nxt_bytes, n - w.end_even, at, w.k_src);
 }
-template <int D, int NW, bool F16>
-__device__ __forceinline__ void fill_v(const Wave<D, NW, F16> &w, int n, int slot) {
+template <int D, int NW, bool F16, bool STREAM, bool RANGED>
+__device__ __forceinline__ void fill_v(const Wave<D, NW, F16, STREAM, RANGED> &w, int n, int slot) {
   const int at = w.lds0 + (2 + slot) * Tile<D>::kBytes;
   if (n < w.end)
     fill_tile<D, NW>(w, w.v_base, w.kv_bytes, n, at, w.v_src);
-  else if (n >= w.end_even && n - w.end_even < w.nxt_end)
+  else if (STREAM && n >= w.end_even && n - w.end_even < w.nxt_end)
     fill_tile<D, NW>(w, w.nxt_v, w.nxt_bytes, n - w.end_even, at, w.v_src);
 }
 
 // A key mask row is read 64 keys (one per lane) a block, one block ahead: the load is issued
 // before that block's fills and is long back when the block's step needs it.
-template <int D, int NW, bool F16>
-__device__ __forceinline__ int mask_lane(const Wave<D, NW, F16> &w, int blk) {
+template <int D, int NW, bool F16, bool STREAM, bool RANGED>
+__device__ __forceinline__ int mask_lane(const Wave<D, NW, F16, STREAM, RANGED> &w, int blk) {
   const int key = blk * kBkv + w.lane;
   if (w.key_mask == nullptr || key >= w.tk) return 0;
   const int64_t at = w.mask_row + key;
@@ -248,14 +251,14 @@ __device__ __forceinline__ int mask_lane(const Wave<D, NW, F16> &w, int blk) {
 
 // S^T = K . Q^T of the key block in K slot `slot`, as 32 scalars: sv[16kb + i] is the score of
 // key 32kb + 8(i/4) + 4g + i%4 (sub-registers of the two accumulators: no moves).
-template <int D, int NW, bool F16>
-__device__ __forceinline__ void scores(const Wave<D, NW, F16> &w, const uint8_t *smem, int slot, float (&sv)[32]) {
+template <int D, int NW, bool F16, bool STREAM, bool RANGED>
+__device__ __forceinline__ void scores(const Wave<D, NW, F16, STREAM, RANGED> &w, const uint8_t *smem, int slot, float (&sv)[32]) {
   using TL = Tile<D>;
   const uint8_t *ks_ = smem + slot * TL::kBytes;
   const f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
   f32x16 s0 = zero, s1 = zero;
 #pragma unroll
-  for (int ks = 0; ks < Wave<D, NW, F16>::KS; ks++) {
+  for (int ks = 0; ks < Wave<D, NW, F16, STREAM, RANGED>::KS; ks++) {
     const u32x4 a0 = *reinterpret_cast<const u32x4 *>(ks_ + w.k_read[ks]);
     const u32x4 a1 = *reinterpret_cast<const u32x4 *>(ks_ + w.k_read[ks] + 32 * TL::kRowBytes);
     s0 = mma<F16>(a0, w.qf[ks], s0);
@@ -270,8 +273,8 @@ __device__ __forceinline__ void scores(const Wave<D, NW, F16> &w, const uint8_t 
 
 // The wave-uniform part of block `blk`'s mask: bit j = key 64 blk + j is below the length and
 // kept by the key mask (`word` is this lane's key-mask element of the block).
-template <int D, int NW, bool F16>
-__device__ __forceinline__ uint64_t uniform_bits(const Wave<D, NW, F16> &w, int blk, int word) {
+template <int D, int NW, bool F16, bool STREAM, bool RANGED>
+__device__ __forceinline__ uint64_t uniform_bits(const Wave<D, NW, F16, STREAM, RANGED> &w, int blk, int word) {
   const int k0 = blk * kBkv;
   uint64_t kbits = ~0ull;
   if (w.key_mask != nullptr) kbits = __builtin_amdgcn_ballot_w64(word != 0);
@@ -280,30 +283,30 @@ __device__ __forceinline__ uint64_t uniform_bits(const Wave<D, NW, F16> &w, int 
 }
 
 // Whether a mask edge crosses block `blk` for this wave (L698-733).
-template <int D, int NW, bool CAUSAL, bool F16>
-__device__ __forceinline__ bool on_edge(const Wave<D, NW, F16> &w, int blk, uint64_t kbits) {
+template <int D, int NW, bool CAUSAL, bool F16, bool STREAM, bool RANGED>
+__device__ __forceinline__ bool on_edge(const Wave<D, NW, F16, STREAM, RANGED> &w, int blk, uint64_t kbits) {
   const int k0 = blk * kBkv;
-  if (kbits != ~0ull || (CAUSAL && (k0 + kBkv - 1 > w.wave_first_row))) return true;
-  // L715-719: the window's right edge for the wave's first row, its left edge for the last.
-  return w.windowed && (k0 + kBkv - 1 > w.wave_first_row + w.reach_right ||
-                        k0 < w.wave_first_row + kWaveRows - 1 - w.reach_left);
+  if (kbits != ~0ull) return true;
+  // L715-731: a range's right edge for the wave's first row, its left edge for the last.
+  if (w.ranged) return k0 + kBkv - 1 > w.hi_first || k0 < w.lo_last;
+  return CAUSAL && (k0 + kBkv - 1 > w.wave_first_row);
 }
 
 // Scales (a non-positive scale only) and masks (L641-697) the scores of block `blk`: hidden
 // scores become -inf.  `kbits` is the uniform word; causality adds a per-lane one.
-template <int D, int NW, bool CAUSAL, bool F16>
-__device__ __forceinline__ void mask_scores(const Wave<D, NW, F16> &w, int blk, uint64_t kbits, float (&sv)[32]) {
+template <int D, int NW, bool CAUSAL, bool F16, bool STREAM, bool RANGED>
+__device__ __forceinline__ void mask_scores(const Wave<D, NW, F16, STREAM, RANGED> &w, int blk, uint64_t kbits, float (&sv)[32]) {
   const int k0 = blk * kBkv;
   uint64_t mine = kbits;
-  if ((CAUSAL && (k0 + kBkv - 1 > w.wave_first_row)) || w.windowed) {
-    // Keys k0 .. my_row (+ the window's reach to the right) are seen from above ...
-    const int seen = w.my_row + (CAUSAL ? 0 : w.reach_right) - k0 + 1;
+  if (w.ranged) {
+    // Keys k0 .. row_hi are seen from above and those from row_lo on from below (L659-695).
+    const int seen = w.row_hi - k0 + 1;
     mine &= seen >= 64 ? ~0ull : (seen <= 0 ? 0ull : (~0ull >> (64 - seen)));
-    if (w.windowed) {
-      // ... and those from my_row - reach_left on from below (L659-668).
-      const int below = w.my_row - w.reach_left - k0;
-      mine &= below <= 0 ? ~0ull : (below >= 64 ? 0ull : (~0ull << below));
-    }
+    const int below = w.row_lo - k0;
+    mine &= below <= 0 ? ~0ull : (below >= 64 ? 0ull : (~0ull << below));
+  } else if (CAUSAL && (k0 + kBkv - 1 > w.wave_first_row)) {
+    const int seen = w.my_row - k0 + 1;  // keys k0 .. my_row are seen
+    mine &= seen >= 64 ? ~0ull : (seen <= 0 ? 0ull : (~0ull >> (64 - seen)));
   }
   mine >>= 4 * w.g;
   const uint32_t lo = (uint32_t)mine, hi = (uint32_t)(mine >> 32);
@@ -349,15 +352,15 @@ __device__ __forceinline__ void probabilities(const float *sv, float unit, float
 }
 
 // O^T += V^T . P^T over 32 keys (half a block): chunks c of 16 keys, fragment registers 4c..4c+3.
-template <int D, int NW, bool F16>
-__device__ __forceinline__ void accumulate(Wave<D, NW, F16> &w, const uint8_t *vs_, int half, const uint32_t *pk) {
+template <int D, int NW, bool F16, bool STREAM, bool RANGED>
+__device__ __forceinline__ void accumulate(Wave<D, NW, F16, STREAM, RANGED> &w, const uint8_t *vs_, int half, const uint32_t *pk) {
   using TL = Tile<D>;
 #pragma unroll
   for (int c = 0; c < 2; c++) {
     const u32x4 pw = {pk[4 * c], pk[4 * c + 1], pk[4 * c + 2], pk[4 * c + 3]};
 
 #pragma unroll
-    for (int db = 0; db < Wave<D, NW, F16>::DB; db++) {
+    for (int db = 0; db < Wave<D, NW, F16, STREAM, RANGED>::DB; db++) {
       const uint8_t *at = vs_ + w.v_read[db] + (32 * half + 16 * c) * TL::kRowBytes;
       const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_PTR(s16x4))(at));
       const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_PTR(s16x4))(at + 8 * TL::kRowBytes));
@@ -370,8 +373,8 @@ __device__ __forceinline__ void accumulate(Wave<D, NW, F16> &w, const uint8_t *v
 // The running maximum's update for a block whose row maximum is `bm`: the lazy rescale of
 // L418-431, and the O^T rescale that a wave skips when all its rows kept their maximum
 // (L56-59).  Returns the exponent's offset m*unit; `corr` is the correction of l.
-template <int D, int NW, bool F16>
-__device__ __forceinline__ float adopt_maximum(Wave<D, NW, F16> &w, float bm, float &corr) {
+template <int D, int NW, bool F16, bool STREAM, bool RANGED>
+__device__ __forceinline__ float adopt_maximum(Wave<D, NW, F16, STREAM, RANGED> &w, float bm, float &corr) {
   const float m_max = __builtin_fmaxf(w.m_run, bm);
   const bool grows = w.limit < (m_max - w.m_run);
   const float m_new = grows ? m_max : w.m_run;
@@ -379,7 +382,7 @@ __device__ __forceinline__ float adopt_maximum(Wave<D, NW, F16> &w, float bm, fl
   w.m_run = m_new;
   if (__builtin_amdgcn_ballot_w64(corr != 1.0f) != 0) {
 #pragma unroll
-    for (int db = 0; db < Wave<D, NW, F16>::DB; db++) w.acc[db] *= corr;
+    for (int db = 0; db < Wave<D, NW, F16, STREAM, RANGED>::DB; db++) w.acc[db] *= corr;
   }
   return m_new * w.unit;
 }
@@ -410,11 +413,11 @@ __device__ __forceinline__ uint32_t p_unit(float s_a, float s_b, float unit, flo
 // never waits for the VALU's whole job.  2 KS slots compute S(blk+1) beside the exponentials
 // of keys 0..31; 2 DB slots add P V of keys 0..31 beside the exponentials of keys 32..63;
 // 2 DB slots add P V of keys 32..63 beside the row maximum of S(blk+1).
-template <int D, int NW, int PAR, bool F16>
-__device__ __forceinline__ void hot_step(Wave<D, NW, F16> &w, const uint8_t *smem, int blk, const float (&sv)[32],
+template <int D, int NW, int PAR, bool F16, bool STREAM, bool RANGED>
+__device__ __forceinline__ void hot_step(Wave<D, NW, F16, STREAM, RANGED> &w, const uint8_t *smem, int blk, const float (&sv)[32],
                                          float (&nv)[32], float &bm) {
   using TL = Tile<D>;
-  constexpr int KS = Wave<D, NW, F16>::KS, DB = Wave<D, NW, F16>::DB;
+  constexpr int KS = Wave<D, NW, F16, STREAM, RANGED>::KS, DB = Wave<D, NW, F16, STREAM, RANGED>::DB;
   constexpr int NQK = 2 * KS;  // score slots
   constexpr int NPV = 4 * DB;  // P V slots, half of them per 32 keys
   const uint8_t *ks_ = smem + (PAR ^ 1) * TL::kBytes;
@@ -511,8 +514,8 @@ __device__ __forceinline__ void hot_step(Wave<D, NW, F16> &w, const uint8_t *sme
 // The general step, for the blocks at the edges: any block, a next block or none, masks, any
 // scale.  Slots are picked at run time.  `sv` holds the masked S(blk) and `bm` its row maximum;
 // on exit they hold block blk+1's (when this wave has one).
-template <int D, int NW, bool CAUSAL, bool F16>
-__device__ __forceinline__ void edge_step(Wave<D, NW, F16> &w, const uint8_t *smem, int blk, int my_end, float (&sv)[32],
+template <int D, int NW, bool CAUSAL, bool F16, bool STREAM, bool RANGED>
+__device__ __forceinline__ void edge_step(Wave<D, NW, F16, STREAM, RANGED> &w, const uint8_t *smem, int blk, int my_end, float (&sv)[32],
                                           float &bm) {
   using TL = Tile<D>;
   const int par = blk & 1;
@@ -546,8 +549,8 @@ __device__ __forceinline__ void edge_step(Wave<D, NW, F16> &w, const uint8_t *sm
 }
 
 // A step of a wave with nothing to compute: fills and the barrier only.
-template <int D, int NW, bool F16>
-__device__ __forceinline__ void idle_step(Wave<D, NW, F16> &w, int blk) {
+template <int D, int NW, bool F16, bool STREAM, bool RANGED>
+__device__ __forceinline__ void idle_step(Wave<D, NW, F16, STREAM, RANGED> &w, int blk) {
   const int par = blk & 1;
   fill_v<D, NW>(w, blk + 1, par ^ 1);
   fill_k<D, NW>(w, blk + 2, par);
@@ -577,13 +580,23 @@ struct Splits {
   uint32_t nbatch;
 };
 
-template <int D, int NW, bool CAUSAL, bool SPLIT, bool F16>
+// The per-row masks of a launch that has them (the RANGED instantiations).
+struct Ranges {
+  int32_t win_left, win_right;  // win_left < 0: no window; the host caps both at t + tk
+  int32_t chunk_size;           // 0: no chunk mask (Chunk of tk/src/ops/attention.rs:39-50)
+  int32_t chunk_left;           // < 0: every earlier chunk
+  int32_t chunk_right;          // the host caps it at the chunks of the keys
+  const void *seg_start;        // [B, T] integers or null
+  int32_t seg_i64;
+};
+
+template <int D, int NW, bool CAUSAL, bool SPLIT, bool RANGED, bool F16>
 __global__ __launch_bounds__(NW * 64, D == 64 ? 3 : 2) void flash_fwd_kernel(
     uint32_t unit_size, uint32_t unit_rcp, uint32_t nqt_u, uint32_t nqt_rcp, uint32_t kvh_u, uint32_t kvh_rcp,
     uint32_t units, uint32_t heads_group, const void *__restrict__ key_lens, const uint16_t *__restrict__ q, int32_t t,
     uint32_t tk_lens64, const uint16_t *__restrict__ k, const uint16_t *__restrict__ v,
     uint16_t *__restrict__ o, const void *__restrict__ key_mask, int32_t mask_bytes, float scale, Splits sp,
-    int32_t q_row_elems, int32_t kv_row_elems, int32_t win_left, int32_t win_right) {
+    int32_t q_row_elems, int32_t kv_row_elems, Ranges rg) {
   // The body is device code only: the host pass needs the kernel's handle, not its
   // instructions (and drops the whole instantiation over the LDS-fill instructions).
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -596,7 +609,7 @@ __global__ __launch_bounds__(NW * 64, D == 64 ? 3 : 2) void flash_fwd_kernel(
   const int tk = (int)(tk_lens64 & 0x7fffffffu);
   const bool lens_i64 = (tk_lens64 >> 31) != 0;
   using TL = Tile<D>;
-  using W = Wave<D, NW, F16>;
+  using W = Wave<D, NW, F16, false, RANGED>;
   constexpr int BQ = NW * kWaveRows;
   constexpr int KS = W::KS, DB = W::DB;
   static_assert(TL::kInstrs % NW == 0, "the tile fills in whole wave instructions per wave");
@@ -661,15 +674,45 @@ __global__ __launch_bounds__(NW * 64, D == 64 ? 3 : 2) void flash_fwd_kernel(
     }
   }
 
-  // L584-608: key blocks [first, end) hold every key some query of the tile sees.  A negative
-  // win_left means no window; the host caps both reaches at the sequence lengths.
-  w.windowed = win_left >= 0;
-  w.reach_left = win_left;
-  w.reach_right = CAUSAL ? 0 : win_right;
+  // L584-608: key blocks [first, end) hold every key some query of the tile sees.
   int first = 0, end = (tk + kBkv - 1) / kBkv;
-  if (w.windowed) first = max(q_off - win_left, 0) / kBkv;
   if (CAUSAL) end = min(end, (q_off + BQ + kBkv - 1) / kBkv);
-  if (w.windowed) end = min(end, (q_off + BQ + win_right + kBkv - 1) / kBkv);
+  if (RANGED) {
+    // This lane's row sees keys [lo, hi] (L659-695); rows past t stand in for row t - 1 where a
+    // table is read.  Everything is monotonic in the row, so the tile's first row gives its
+    // first block and its last row the end (L580-606).
+    const int64_t row_abs = q_off + w.wave * kWaveRows + ln;
+    int64_t lo = 0, hi = tk - 1;
+    if (rg.win_left >= 0) {
+      lo = max(lo, row_abs - rg.win_left);
+      hi = min(hi, row_abs + rg.win_right);
+      first = max(q_off - rg.win_left, 0) / kBkv;
+      end = min(end, (q_off + BQ + rg.win_right + kBkv - 1) / kBkv);
+    }
+    if (rg.chunk_size > 0) {
+      const int64_t cq = row_abs / rg.chunk_size;
+      hi = min(hi, (cq + rg.chunk_right + 1) * rg.chunk_size - 1);
+      const int cq1 = (q_off + BQ - 1) / rg.chunk_size;
+      end = (int)min((int64_t)end, ((int64_t)(cq1 + 1 + rg.chunk_right) * rg.chunk_size + (kBkv - 1)) / kBkv);
+      if (rg.chunk_left >= 0) {
+        lo = max(lo, (max(cq, (int64_t)rg.chunk_left) - rg.chunk_left) * rg.chunk_size);
+        const int cq0 = q_off / rg.chunk_size;
+        first = max(first, (int)((int64_t)(max(cq0, rg.chunk_left) - rg.chunk_left) * rg.chunk_size / kBkv));
+      }
+    }
+    if (rg.seg_start != nullptr) {
+      auto start_of = [&](int64_t r) -> int64_t {
+        const int64_t at = (int64_t)b * t + min(r, (int64_t)t - 1);
+        const long long x = rg.seg_i64 ? ((const long long *)rg.seg_start)[at] : (long long)((const int *)rg.seg_start)[at];
+        return x < 0 ? 0 : (x > tk ? tk : x);
+      };
+      lo = max(lo, start_of(row_abs));
+      first = max(first, (int)(start_of(q_off) / kBkv));
+    }
+    if (CAUSAL) hi = min(hi, row_abs);
+    w.row_lo = (int)lo;
+    w.row_hi = (int)max(hi, (int64_t)-1);
+  }
   if (key_lens != nullptr) end = min(end, (len + kBkv - 1) / kBkv);
   end = max(end, first);
   // L609-612: a split takes an even share of those blocks.  From here on the kernel works in
@@ -691,6 +734,13 @@ __global__ __launch_bounds__(NW * 64, D == 64 ? 3 : 2) void flash_fwd_kernel(
   w.mask_bytes = mask_bytes;
   w.wave_first_row = q_off + w.wave * kWaveRows - first_key;
   w.my_row = w.wave_first_row + ln;
+  if (RANGED) {
+    w.row_lo -= first_key;
+    w.row_hi -= first_key;
+    w.lo_last = __builtin_amdgcn_readlane(w.row_lo, kWaveRows - 1);
+    w.hi_first = __builtin_amdgcn_readlane(w.row_hi, 0);
+    w.hi_last = __builtin_amdgcn_readlane(w.row_hi, kWaveRows - 1);
+  }
 
   w.kv_row_bytes = kv_row_elems * 2;
   w.k_base = (const uint8_t *)(k + ((int64_t)b * tk + first_key) * kv_row_elems + (int64_t)kvh * D);
@@ -753,9 +803,9 @@ __global__ __launch_bounds__(NW * 64, D == 64 ? 3 : 2) void flash_fwd_kernel(
   // A causal wave past its last visible key has nothing to add from a block: it only keeps
   // filling and meeting the barriers.  Blocks [0, my_end) are this wave's.
   int my_end = end;
-  if (CAUSAL || w.windowed) {
+  if (RANGED || CAUSAL) {
     // The last key the wave's last row sees; negative: the blocks lie past every row's reach.
-    const int last_seen = w.wave_first_row + kWaveRows - 1 + w.reach_right;
+    const int last_seen = RANGED ? w.hi_last : w.wave_first_row + kWaveRows - 1;
     my_end = min(end, last_seen < 0 ? 0 : last_seen / kBkv + 1);
   }
 
@@ -782,13 +832,16 @@ __global__ __launch_bounds__(NW * 64, D == 64 ? 3 : 2) void flash_fwd_kernel(
   int full = 0;
   if (w.positive && key_mask == nullptr) {
     full = min(my_end, len / kBkv);
-    if (CAUSAL || w.windowed) full = min(full, (w.wave_first_row + w.reach_right + 1) / kBkv);
+    if (RANGED)
+      full = min(full, w.hi_first < 0 ? 0 : (w.hi_first + 1) / kBkv);
+    else if (CAUSAL)
+      full = min(full, (w.wave_first_row + 1) / kBkv);
   }
   int blk = 0;
-  if (w.windowed) {
-    // The window's left edge crosses the blocks below the last row's reach: general steps, an
+  if (RANGED) {
+    // A range's left edge crosses the blocks below the last row's first key: general steps, an
     // even number of them so that the hot pairs start on an even block.
-    const int below = w.wave_first_row + kWaveRows - 1 - w.reach_left;
+    const int below = w.lo_last;
     const int lead = min(my_end, below <= 0 ? 0 : ((below + kBkv - 1) / kBkv + 1) & ~1);
     for (; blk < lead; blk++) edge_step<D, NW, CAUSAL>(w, smem, blk, my_end, sv, bm);
   }
@@ -903,7 +956,7 @@ __global__ __launch_bounds__(NW * 64, 3) void flash_stream_kernel(
   const int tk = (int)(tk_lens64 & 0x7fffffffu);
   const bool lens_i64 = (tk_lens64 >> 31) != 0;
   using TL = Tile<D>;
-  using W = Wave<D, NW, F16>;
+  using W = Wave<D, NW, F16, true, false>;
   constexpr int BQ = NW * kWaveRows;
   constexpr int KS = W::KS, DB = W::DB;
   constexpr int kStageRows = 1024 / TL::kRowBytes;                  // rows a wave instruction stages
@@ -953,9 +1006,6 @@ __global__ __launch_bounds__(NW * 64, 3) void flash_stream_kernel(
   w.mask_row = 0;
   w.mask_bytes = 0;
   w.mask_next = 0;
-  w.windowed = false;
-  w.reach_left = 0;
-  w.reach_right = 0;
   w.kv_row_bytes = kv_row_elems * 2;
   w.lds0 = (int)(uintptr_t)(LDS_PTR(uint8_t))(smem);
   constexpr int kRowsPer = 64 / TL::kCpr;
@@ -1184,7 +1234,7 @@ hipError_t launch_stream(const AttnArgs &a, hipStream_t stream, int64_t slots, c
   return hipGetLastError();
 }
 
-template <int D, int NW, bool CAUSAL, bool SPLIT, bool F16>
+template <int D, int NW, bool CAUSAL, bool SPLIT, bool RANGED, bool F16>
 hipError_t launch(const AttnArgs &a, hipStream_t stream) {
   using TL = Tile<D>;
   constexpr int BQ = NW * kWaveRows;
@@ -1198,7 +1248,7 @@ hipError_t launch(const AttnArgs &a, hipStream_t stream) {
   const int64_t kv_row = a.kv_row_elems > 0 ? a.kv_row_elems : (int64_t)a.kv_heads * a.d;
   // The fills address a (batch, kv head)'s rows with 32-bit byte offsets.
   if ((int64_t)a.tk * kv_row * 2 > 0x7fffffffLL || q_row > 0x7fffffffLL) return hipErrorInvalidValue;
-  auto kernel = flash_fwd_kernel<D, NW, CAUSAL, SPLIT, F16>;
+  auto kernel = flash_fwd_kernel<D, NW, CAUSAL, SPLIT, RANGED, F16>;
   // The LDS ring is above the default limit of a launch: one attribute call per instantiation
   // and device, from whichever thread gets there first (a second call is harmless).
   static std::atomic<uint64_t> configured{0};  // a bit per device ordinal, devices past 63 always ask
@@ -1231,9 +1281,9 @@ hipError_t launch(const AttnArgs &a, hipStream_t stream) {
   // The streaming form, where asked for and where it has a kernel (head size 64, lengths or no
   // key mask, no window, no splits): `knob` workgroups per XCD, each walking its run of tiles.
   // It is never chosen unasked: measured, it has not beaten a workgroup per tile.
-  if constexpr (D == 64 && !SPLIT) {
+  if constexpr (D == 64 && !SPLIT && !RANGED) {
     const int knob = g_stream_slots.load(std::memory_order_relaxed);
-    if (knob > 0 && a.key_mask == nullptr && a.win_left < 0)
+    if (knob > 0 && a.key_mask == nullptr)
       return launch_stream<D, NW, CAUSAL, F16>(a, stream, knob, geo, q_row, kv_row);
   }
   const uint32_t heads_group = (uint32_t)a.heads | geo.group << 16;
@@ -1246,19 +1296,34 @@ hipError_t launch(const AttnArgs &a, hipStream_t stream) {
   sp.l_part = a.l_part;
   sp.nbatch = (uint32_t)a.batch;
   if (splits > 1 && (a.o_part == nullptr || a.m_part == nullptr || a.l_part == nullptr)) return hipErrorInvalidValue;
+  Ranges rg;
+  rg.win_left = a.win_left;
+  rg.win_right = a.win_right;
+  rg.chunk_size = a.chunk_size;
+  rg.chunk_left = a.chunk_left;
+  rg.chunk_right = a.chunk_right;
+  rg.seg_start = a.seg_start;
+  rg.seg_i64 = a.seg_i64;
   hipLaunchKernelGGL(kernel, dim3((uint32_t)grid), dim3(NW * 64), smem, stream, geo.unit_size, geo.unit_rcp, geo.nqt,
                      geo.nqt_rcp, geo.kv_heads, geo.kvh_rcp, geo.units, heads_group, a.key_lens,
                      (const uint16_t *)a.q, a.t, tk_lens64, (const uint16_t *)a.k,
                      (const uint16_t *)a.v, (uint16_t *)a.o, a.key_mask, a.mask_bytes, a.scale, sp, (int32_t)q_row,
-                     (int32_t)kv_row, a.win_left, a.win_right);
+                     (int32_t)kv_row, rg);
   return hipGetLastError();
+}
+
+template <int D, bool RANGED, bool F16>
+hipError_t launch_s(const AttnArgs &a, hipStream_t stream) {
+  if (a.splits > 1)
+    return a.causal ? launch<D, 4, true, true, RANGED, F16>(a, stream) : launch<D, 4, false, true, RANGED, F16>(a, stream);
+  return a.causal ? launch<D, 4, true, false, RANGED, F16>(a, stream) : launch<D, 4, false, false, RANGED, F16>(a, stream);
 }
 
 template <int D, bool F16>
 hipError_t launch_t(const AttnArgs &a, hipStream_t stream) {
-  if (a.splits > 1)
-    return a.causal ? launch<D, 4, true, true, F16>(a, stream) : launch<D, 4, false, true, F16>(a, stream);
-  return a.causal ? launch<D, 4, true, false, F16>(a, stream) : launch<D, 4, false, false, F16>(a, stream);
+  // A window, a chunk mask or segment starts: the instantiations with per-row key ranges.
+  const bool ranged = a.win_left >= 0 || a.chunk_size > 0 || a.seg_start != nullptr;
+  return ranged ? launch_s<D, true, F16>(a, stream) : launch_s<D, false, F16>(a, stream);
 }
 
 template <int D>

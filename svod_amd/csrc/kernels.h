@@ -51,6 +51,14 @@ struct AttnArgs {
   // Attn::window (tk/src/ops/attention.rs:64-65): query i sees keys [i - win_left, i + win_right];
   // win_left < 0 = no window.
   int32_t win_left, win_right;
+  // Attn::chunk (tk/src/ops/attention.rs:39-50, 66-68): query i sees the keys of chunk i / chunk_size,
+  // of the chunk_left chunks before it (< 0 = every earlier one) and the chunk_right after.
+  // chunk_size 0 = no chunk mask.
+  int32_t chunk_size, chunk_left, chunk_right;
+  // Attn::seg_start (tk/src/ops/attention.rs:69-71): [batch, t] i32 or i64 segment starts,
+  // non-decreasing along t; query i does not see keys before seg_start[b, i].  Null = none.
+  const void *seg_start;
+  int32_t seg_i64;
 };
 hipError_t launch_attention(const AttnArgs &a, hipStream_t stream);
 

@@ -333,10 +333,15 @@ static int attend(const svodk_tensor *q, const svodk_tensor *k, const svodk_tens
   if (why != 0) return ran_graph(op, why);
   // Options the reference's kernel holds and this library's does not: no
   // config here holds them (the reference's own use of Fallback::Config, L210-214).
-  if (opts->has_chunk || opts->seg_start != nullptr || opts->has_cache || opts->bias != nullptr)
-    return ran_graph(op, SVODK_GRAPH_CONFIG);
+  if (opts->has_cache || opts->bias != nullptr) return ran_graph(op, SVODK_GRAPH_CONFIG);
   if (opts->has_window && (opts->window_left < 0 || opts->window_right < 0))
     return fail(SVODK_ERR_ARGUMENT, "%s: a negative window reach", op);
+  // Chunk { size, left, right } of tk/src/ops/attention.rs:39-50: usize fields, a size of at least 1.
+  if (opts->has_chunk && (opts->chunk_size <= 0 || opts->chunk_right < 0 || (opts->chunk_has_left && opts->chunk_left < 0)))
+    return fail(SVODK_ERR_ARGUMENT, "%s: a chunk mask needs a positive size and non-negative reaches", op);
+  if (opts->seg_start != nullptr && !(opts->seg_start->dtype == SVODK_I32 || opts->seg_start->dtype == SVODK_I64))
+    return fail(SVODK_ERR_DTYPE, "%s: seg start is %s, the input is Int32 or Int64", op,
+                dtype_name(opts->seg_start->dtype));
   const int64_t t = q->shape[1], tk = k->shape[1], d = q->shape[3];
   if (t > 0x7fffffff || tk > 0x7fffffff || heads > 0x7fffffff || cap > 0x7fffffff)
     return ran_graph(op, SVODK_GRAPH_SHAPE);
@@ -353,9 +358,15 @@ static int attend(const svodk_tensor *q, const svodk_tensor *k, const svodk_tens
                    {"key_mask", bools ? bools->data : nullptr,
                     bools ? (size_t)numel(bools) * dtype_bytes(bools->dtype) : 0, false}};
   if (q->data == nullptr || k->data == nullptr || v->data == nullptr || out->data == nullptr ||
-      (lens && lens->data == nullptr) || (bools && bools->data == nullptr))
+      (lens && lens->data == nullptr) || (bools && bools->data == nullptr) ||
+      (opts->seg_start && opts->seg_start->data == nullptr))
     return fail(SVODK_ERR_ARGUMENT, "%s: a null device pointer", op);
   if (int rc = check_aliasing(op, spans, 6)) return rc;
+  if (opts->seg_start != nullptr) {
+    const svodk_tensor *seg = opts->seg_start;
+    Span pair[2] = {{"seg_start", seg->data, (size_t)numel(seg) * dtype_bytes(seg->dtype), false}, spans[3]};
+    if (int rc = check_aliasing(op, pair, 2)) return rc;
+  }
 
   svodk::AttnArgs a{};
   a.q = q->data;
@@ -381,6 +392,18 @@ static int attend(const svodk_tensor *q, const svodk_tensor *k, const svodk_tens
   if (opts->has_window) {
     a.win_left = (int32_t)std::min<int64_t>(opts->window_left, t + tk);
     a.win_right = (int32_t)std::min<int64_t>(opts->window_right, t + tk);
+  }
+  // The chunk mask's reaches, capped the same way: past the last chunk they hide nothing.
+  if (opts->has_chunk) {
+    const int64_t chunks = (t + tk) / opts->chunk_size + 2;
+    a.chunk_size = (int32_t)std::min<int64_t>(opts->chunk_size, t + tk + 1);
+    a.chunk_left = opts->chunk_has_left ? (int32_t)std::min<int64_t>(opts->chunk_left, chunks) : -1;
+    a.chunk_right = (int32_t)std::min<int64_t>(opts->chunk_right, chunks);
+    if (t + tk > 0x3fffffff) return ran_graph(op, SVODK_GRAPH_SHAPE);  // chunk edges stay 32-bit
+  }
+  if (opts->seg_start != nullptr) {
+    a.seg_start = opts->seg_start->data;
+    a.seg_i64 = opts->seg_start->dtype == SVODK_I64;
   }
   if (packed != nullptr) a.q_row_elems = a.kv_row_elems = (heads + 2 * kv_heads) * d;
   // L280-302: key splits.  The partial tensors live in the caller's workspace.

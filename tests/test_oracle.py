@@ -373,3 +373,92 @@ def test_the_stream_dtype_switch_only_changes_the_rounding():
     assert np.array_equal(oracle.round_f16(f16), f16) and np.array_equal(oracle.round_bf16(bf), bf)
     d = oracle.attention_direct(p)
     assert np.abs(f16 - d).max() < np.abs(bf - d).max()  # f16 keeps three more bits
+
+
+# ---------------------------------------------------------------- chunk masks and segment starts
+def brute_ranges(b, t, tk, chunk, seg):
+    """hidden(j) of tk/src/test/unit/attention.rs:133-148, the chunk and segment arms, one pair at a time."""
+    out = np.ones((b, t, tk), dtype=np.uint8)
+    for bb, i, j in itertools.product(range(b), range(t), range(tk)):
+        if chunk is not None:
+            size, left, right = chunk
+            if j // size > i // size + right or (left is not None and j // size + left < i // size):
+                out[bb, i, j] = 0
+        if seg is not None and j < seg[bb, i]:
+            out[bb, i, j] = 0
+    return out
+
+
+@pytest.mark.parametrize("chunk", [None, (3, 1, 0), (4, None, 1), (2, 0, 0), (5, 2, 2)],
+                         ids=["no chunks", "3s one behind", "4s all behind one ahead", "2s own chunk", "5s two each way"])
+@pytest.mark.parametrize("segments", [False, True])
+def test_chunk_and_segment_visibility_by_brute_force(chunk, segments):
+    b, t, tk = 2, 11, 13
+    seg = np.array([[i - i % 4 for i in range(t)], [0] * 5 + [5] * 6]) if segments else None
+    got = oracle.visible(b, t, tk, chunk=chunk, seg_start=seg)
+    assert np.array_equal(got, brute_ranges(b, t, tk, chunk, seg))
+
+
+def test_masks_that_hide_nothing_and_masks_that_are_other_masks():
+    b, t = 2, 23
+    plain = oracle.visible(b, t, t)
+    assert np.array_equal(oracle.visible(b, t, t, chunk=(t, 0, 0)), plain)               # one chunk holds every row
+    assert np.array_equal(oracle.visible(b, t, t, seg_start=np.zeros((b, t))), plain)     # one segment from key 0
+    assert np.array_equal(oracle.visible(b, t, t, chunk=(1, None, 0)), oracle.visible(b, t, t, causal=True))
+    assert np.array_equal(oracle.visible(b, t, t, chunk=(1, 3, 2)), oracle.visible(b, t, t, window=(3, 2)))
+    starts = np.tile(np.arange(t) - np.arange(t) % 6, (b, 1))
+    assert np.array_equal(oracle.visible(b, t, t, causal=True, seg_start=starts),
+                          oracle.visible(b, t, t, causal=True, chunk=(6, 0, 0)))
+
+
+def ranged_case(b=2, t=100, h=2, hkv=1, d=16, seed=5):
+    g = Lcg(seed)
+    return g.bf16((b, t, h, d)), g.bf16((b, t, hkv, d)), g.bf16((b, t, hkv, d))
+
+
+@pytest.mark.parametrize("path", ["direct", "flash", "graph"])
+def test_packed_segments_are_separate_sequences(path):
+    """Causal attention over rows packed in segments of 40 (the reference's fixture,
+    tk/src/test/unit/attention.rs:31-32,81) is causal attention over each segment alone."""
+    q, k, v = ranged_case()
+    b, t = q.shape[:2]
+    seg = np.tile(np.arange(t) - np.arange(t) % 40, (b, 1))
+    run = {"direct": oracle.attention_direct, "flash": oracle.attention_flash, "graph": oracle.attention_graph}[path]
+    got = run(oracle.AttnProblem(q, k, v, causal=True, seg_start=seg))
+    for s0 in range(0, t, 40):
+        alone = oracle.attention_direct(oracle.AttnProblem(q[:, s0:s0 + 40], k[:, s0:s0 + 40], v[:, s0:s0 + 40], causal=True))
+        assert max_abs(got[:, s0:s0 + 40], alone) < (1e-12 if path == "direct" else 2e-2)
+
+
+@pytest.mark.parametrize("path", ["direct", "flash", "graph"])
+def test_chunks_that_see_only_themselves_are_separate_sequences(path):
+    q, k, v = ranged_case(t=90)
+    run = {"direct": oracle.attention_direct, "flash": oracle.attention_flash, "graph": oracle.attention_graph}[path]
+    got = run(oracle.AttnProblem(q, k, v, chunk=(24, 0, 0)))
+    for s0 in range(0, 90, 24):
+        alone = oracle.attention_direct(oracle.AttnProblem(q[:, s0:s0 + 24], k[:, s0:s0 + 24], v[:, s0:s0 + 24]))
+        assert max_abs(got[:, s0:s0 + 24], alone) < (1e-12 if path == "direct" else 2e-2)
+
+
+RANGED = [
+    ("causal segments", dict(causal=True, segments=True), None),
+    ("chunks with lengths", dict(chunk=(16, 2, 0)), [128, 90]),
+    ("chunks, every earlier one and one ahead", dict(chunk=(24, None, 1)), None),
+    ("every mask at once", dict(causal=True, window=(50, 0), chunk=(32, 3, 0), segments=True, key_mask=True), [128, 100]),
+]
+
+
+@pytest.mark.parametrize("name,masks,lens", RANGED, ids=[r[0] for r in RANGED])
+@pytest.mark.parametrize("tile", [(64, 64), (128, 64), (64, 32)])
+@pytest.mark.parametrize("splits", [1, 2])
+def test_tile_program_skips_only_hidden_blocks(name, masks, lens, tile, splits):
+    """The block range of L584-612 (first..end from window, chunk, segment, causal, lens) leaves out
+    only blocks no query of the tile sees: the program agrees with the direct softmax over the
+    same visibility (tk/src/test/unit/attention.rs:356-358, < 2e-2), whole or split."""
+    masks = dict(masks)
+    b, t = 2, 128
+    q, k, v = ranged_case(b=b, t=t, h=2, hkv=2, d=32)
+    seg = np.tile(np.arange(t) - np.arange(t) % 40, (b, 1)) if masks.pop("segments", False) else None
+    key_mask = (np.add.outer(np.arange(b), np.arange(t)) % 5 != 2) if masks.pop("key_mask", False) else None
+    p = oracle.AttnProblem(q, k, v, key_lens=None if lens is None else np.array(lens), key_mask=key_mask, seg_start=seg, **masks)
+    assert max_abs(oracle.attention_flash(p, bq=tile[0], bkv=tile[1], splits=splits), oracle.attention_direct(p)) < 2e-2

@@ -73,10 +73,11 @@ typedef enum svodk_key_mask {
 
 /*
  * Attn of tk/src/ops/attention.rs:60-86.  Zero-initialise, then set fields.
- * Windows, chunk masks and segment starts (I32 or I64, non-decreasing along T)
- * have kernels, alone or together with every other mask.  Options this
- * library has no kernel for (cache, bias) are still validated as the
- * reference validates them and then answered with SVODK_GRAPH_CONFIG.
+ * Windows, chunk masks, segment starts (I32 or I64, non-decreasing along T)
+ * and an additive bias (of the operands' type, rows unpadded) have kernels,
+ * alone or together with every other option.  A cache, which this library has
+ * no kernel for, is still validated as the reference validates it and then
+ * answered with SVODK_GRAPH_CONFIG.
  *
  * `splits` > 1 asks for key splits (tk/src/ops/attention.rs:79, 280-302): the
  * count is capped at the number of 64-key blocks of Tk (split_ranked, :405-410);

@@ -49,21 +49,27 @@ _u8p = ctypes.POINTER(ctypes.c_uint8)
 
 
 class _Ranges(ctypes.Structure):
-    """``svod_oracle_ranges``: the chunk mask and the segment starts."""
+    """``svod_oracle_extras``: the chunk mask, the segment starts and the bias."""
 
     _fields_ = [("chunk_size", ctypes.c_int32), ("chunk_has_left", ctypes.c_int32), ("chunk_left", ctypes.c_int32),
-                ("chunk_right", ctypes.c_int32), ("seg_start", ctypes.POINTER(ctypes.c_int32))]
+                ("chunk_right", ctypes.c_int32), ("seg_start", ctypes.POINTER(ctypes.c_int32)),
+                ("bias", ctypes.POINTER(ctypes.c_float)), ("bias_per_batch", ctypes.c_int32)]
 
 
 _rangesp = ctypes.POINTER(_Ranges)
 
 
-def _ranges(chunk, seg_start):
-    """(pointer or None, what must stay alive) for ``chunk = (size, left or None, right)`` and ``seg_start [B,T]``."""
-    if chunk is None and seg_start is None:
+def _ranges(chunk, seg_start, bias=None, batch=None):
+    """(pointer or None, what must stay alive) for ``chunk = (size, left or None, right)``, ``seg_start [B,T]``
+    and ``bias [B or 1, H, T, Tk]``."""
+    if chunk is None and seg_start is None and bias is None:
         return None, None
     r = _Ranges()
     seg = None
+    if bias is not None:
+        bias = np.ascontiguousarray(bias, dtype=np.float32)
+        r.bias = bias.ctypes.data_as(ctypes.POINTER(ctypes.c_float))
+        r.bias_per_batch = int(bias.shape[0] != 1 or batch == 1)
     if chunk is not None:
         size, left, right = chunk
         r.chunk_size, r.chunk_has_left = int(size), int(left is not None)
@@ -71,7 +77,7 @@ def _ranges(chunk, seg_start):
     if seg_start is not None:
         seg = np.ascontiguousarray(seg_start, dtype=np.int32)
         r.seg_start = seg.ctypes.data_as(ctypes.POINTER(ctypes.c_int32))
-    return ctypes.pointer(r), (r, seg)
+    return ctypes.pointer(r), (r, seg, bias)
 
 _i32 = ctypes.c_int32
 
@@ -207,6 +213,7 @@ class AttnProblem:
     window: Optional[tuple] = None
     chunk: Optional[tuple] = None  # (size, left or None, right): Chunk of tk/src/ops/attention.rs:39-50
     seg_start: Optional[np.ndarray] = None  # [B, T] int
+    bias: Optional[np.ndarray] = None  # [B or 1, H, T, Tk] float32 (stream-dtype-exact), added to the scaled scores
     scale: Optional[float] = None
     bf16: bool = True
 
@@ -225,7 +232,9 @@ class AttnProblem:
         lens = None if self.key_lens is None else np.ascontiguousarray(self.key_lens, dtype=np.int32)
         mask = None if self.key_mask is None else np.ascontiguousarray(np.asarray(self.key_mask) != 0, dtype=np.int32)
         wl, wr = (-1, -1) if self.window is None else self.window
-        ranges, alive = _ranges(self.chunk, self.seg_start)
+        if self.bias is not None and tuple(self.bias.shape[1:]) != (h, t, tk):
+            raise ValueError(f"bias has shape {self.bias.shape}, expected [{b} | 1, {h}, {t}, {tk}]")
+        ranges, alive = _ranges(self.chunk, self.seg_start, self.bias, b)
         keep = (lens, mask, alive)
         args = [b, t, tk, h, hkv, d, int(self.causal), wl, wr, ctypes.c_float(self.scale_f32()),
                 _ptr(lens, _i32p), _ptr(mask, _i32p), tk, ranges]

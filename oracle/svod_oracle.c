@@ -29,6 +29,10 @@
  *       float64 (a library routine, not the reference) and closed forms
  *       (uniform scores -> mean of visible V; one visible key -> that V row;
  *       fully hidden row -> zeros).
+ *       The bias arm is pinned against the same torch routine with the bias
+ *       (and the masks as -inf) as its attn_mask, and by closed forms
+ *       (a constant row changes nothing; -inf walls are a key mask; zero
+ *       queries give softmax(bias) . v).
  *   svod_oracle_attention_graph, svod_oracle_attention_flash
  *       pinned against svod_oracle_attention_direct within the tolerances the
  *       reference holds itself to (tk/src/test/unit/attention.rs:483,
@@ -177,14 +181,16 @@ void svod_oracle_rope_table(double theta, int32_t seq_len, int32_t head_dim, flo
 /* ------------------------------------------------------------------ */
 /* the attention problem                                               */
 /* ------------------------------------------------------------------ */
-/* The masks over (query row, key) beyond causal, window and the key masks
- * (Attn::chunk and Attn::seg_start, tk/src/ops/attention.rs:66-71). */
+/* The options over (query row, key) beyond causal, window and the key masks
+ * (Attn::chunk, Attn::seg_start and Attn::bias, tk/src/ops/attention.rs:66-71, 82-85). */
 typedef struct {
   int32_t chunk_size;     /* 0: no chunk mask */
   int32_t chunk_has_left; /* Chunk::left is Some */
   int32_t chunk_left, chunk_right;
   const int32_t *seg_start; /* [batch, t] or NULL */
-} svod_oracle_ranges;
+  const float *bias;        /* [batch or 1, heads, t, tk] stream-dtype-exact values, or NULL */
+  int32_t bias_per_batch;   /* Bias::PerBatch (1) or Bias::Shared (0) */
+} svod_oracle_extras;
 
 typedef struct {
   int32_t batch, t, tk, heads, kv_heads, d;
@@ -195,8 +201,22 @@ typedef struct {
   const int32_t *key_mask; /* [batch, mask_stride], nonzero = visible, or NULL */
   int32_t mask_stride;
   int32_t bf16_stream; /* 1: q/k/v/o are bf16 values; 0: f32 */
-  const svod_oracle_ranges *ranges; /* or NULL */
+  const svod_oracle_extras *ranges; /* or NULL */
 } attn_problem;
+
+/* The chunk and segment arms of hidden(j) (tk/src/test/unit/attention.rs:133-137, 147). */
+static inline int hidden_by_ranges(const attn_problem *p, int32_t b, int32_t i, int32_t j) {
+  if (!p->ranges) return 0;
+  const svod_oracle_extras *r = p->ranges;
+  if (r->chunk_size > 0) {
+    const int64_t cj = j / r->chunk_size, ci = i / r->chunk_size;
+    if (cj > ci + r->chunk_right) return 1;
+    if (r->chunk_has_left && cj + r->chunk_left < ci) return 1;
+  }
+  /* Rows past t (a tile's overhang) read no segment start: the bounded view gives 0 (L573-576). */
+  if (r->seg_start && i < p->t && j < r->seg_start[(int64_t)b * p->t + i]) return 1;
+  return 0;
+}
 
 /* hidden(j) of tk/src/test/unit/attention.rs:133-148, the arms without a cache:
  * j >= len || (causal && j > i) || window || chunked(j) || key_mask == 0 || j < seg_start[b, i],
@@ -204,7 +224,7 @@ typedef struct {
  * The kernel's keep predicate (tk/src/kernels/attention.rs:641-697) is its
  * negation: col <= row, col < len (len = min(key_lens[b], tk), L533-536),
  * row <= col + left && col <= row + right, key_mask != 0. */
-static inline int hidden(const attn_problem *p, int32_t b, int32_t i, int32_t j) {
+static inline int hidden_without_ranges(const attn_problem *p, int32_t b, int32_t i, int32_t j) {
   int32_t len = p->tk;
   if (p->key_lens) {
     len = p->key_lens[b];
@@ -214,23 +234,23 @@ static inline int hidden(const attn_problem *p, int32_t b, int32_t i, int32_t j)
   if (p->causal && j > i) return 1;
   if (p->window_left >= 0 && (j + p->window_left < i || j > i + p->window_right)) return 1;
   if (p->key_mask && p->key_mask[(int64_t)b * p->mask_stride + j] == 0) return 1;
-  if (p->ranges) {
-    const svod_oracle_ranges *r = p->ranges;
-    if (r->chunk_size > 0) {
-      const int64_t cj = j / r->chunk_size, ci = i / r->chunk_size;
-      if (cj > ci + r->chunk_right) return 1;
-      if (r->chunk_has_left && cj + r->chunk_left < ci) return 1;
-    }
-    /* Rows past t (a tile's overhang) read no segment start: the bounded view gives 0 (L573-576). */
-    if (r->seg_start && i < p->t && j < r->seg_start[(int64_t)b * p->t + i]) return 1;
-  }
   return 0;
+}
+static inline int hidden(const attn_problem *p, int32_t b, int32_t i, int32_t j) {
+  return hidden_without_ranges(p, b, i, j) || hidden_by_ranges(p, b, i, j);
+}
+
+/* bias[b or 0][h][i][j], or 0 without one (the view of L566-571). */
+static inline float bias_at(const attn_problem *p, int32_t b, int32_t h, int32_t i, int32_t j) {
+  if (!p->ranges || !p->ranges->bias) return 0.0f;
+  const int64_t row = ((int64_t)(p->ranges->bias_per_batch ? b : 0) * p->heads + h) * p->t + i;
+  return p->ranges->bias[row * p->tk + j];
 }
 
 /* Visibility of every (b, i, j): out[b][i][j] = 1 where key j is seen by query i. */
 void svod_oracle_visible(int32_t batch, int32_t t, int32_t tk, int32_t causal, int32_t window_left,
                          int32_t window_right, const int32_t *key_lens, const int32_t *key_mask, int32_t mask_stride,
-                         const svod_oracle_ranges *ranges, uint8_t *out) {
+                         const svod_oracle_extras *ranges, uint8_t *out) {
   attn_problem p = {batch, t, tk, 1, 1, 1, causal, window_left, window_right, 1.0f, key_lens, key_mask, mask_stride, 0,
                     ranges};
   for (int32_t b = 0; b < batch; b++)
@@ -307,7 +327,8 @@ static void direct_slice(const void *ctxp, int32_t b, int32_t h) {
       const float *kj = c->k + ((int64_t)b * p->tk + j) * kv_stride + (int64_t)kv_head * d;
       double dot = 0.0;
       for (int32_t dd = 0; dd < d; dd++) dot += (double)qi[dd] * (double)kj[dd];
-      scores[j] = dot * (double)p->scale;
+      /* attention.rs:152-160: the sum times the scale, plus the bias. */
+      scores[j] = dot * (double)p->scale + (double)bias_at(p, b, h, i, j);
       if (scores[j] > mx) mx = scores[j];
     }
     for (int32_t dd = 0; dd < d; dd++) oi[dd] = 0.0;
@@ -339,7 +360,7 @@ static int check_problem(const attn_problem *p) {
 int svod_oracle_attention_direct(int32_t batch, int32_t t, int32_t tk, int32_t heads, int32_t kv_heads, int32_t d,
                                  int32_t causal, int32_t window_left, int32_t window_right, float scale,
                                  const int32_t *key_lens, const int32_t *key_mask, int32_t mask_stride,
-                                 const svod_oracle_ranges *ranges, const float *q, const float *k, const float *v,
+                                 const svod_oracle_extras *ranges, const float *q, const float *k, const float *v,
                                  double *out, int32_t threads) {
   direct_ctx c = {{batch, t, tk, heads, kv_heads, d, causal, window_left, window_right, scale, key_lens, key_mask,
                    mask_stride, 0, ranges},
@@ -390,6 +411,7 @@ static void graph_slice(const void *ctxp, int32_t b, int32_t h) {
     const float *qi = c->q + ((int64_t)b * p->t + i) * stride + (int64_t)h * d;
     float *oi = c->out + ((int64_t)b * p->t + i) * stride + (int64_t)h * d;
     int any_mask = p->causal || p->window_left >= 0 || p->key_lens || p->key_mask || p->ranges;
+    const int has_bias = p->ranges && p->ranges->bias;
     float mx = -INFINITY;
     for (int32_t j = 0; j < tk; j++) {
       const float *kj = kh + (int64_t)j * d;
@@ -399,8 +421,12 @@ static void graph_slice(const void *ctxp, int32_t b, int32_t h) {
       else
         for (int32_t dd = 0; dd < d; dd++) s += qi[dd] * kj[dd];
       s *= p->scale;
-      keep[j] = (uint8_t)(!any_mask || !hidden(p, b, i, j));
+      /* tk/src/ops/attention.rs:566-574: with a bias the chunk and segment masks fold into it as
+       * its floor (an additive f32::MIN, not part of the keep mask SDPA re-zeroes with). */
+      const int floored = has_bias && hidden_by_ranges(p, b, i, j);
+      keep[j] = (uint8_t)(!any_mask || !(has_bias ? hidden_without_ranges(p, b, i, j) : hidden(p, b, i, j)));
       if (!keep[j]) s = fmin32;
+      if (has_bias) s += floored ? fmin32 : bias_at(p, b, h, i, j);
       row[j] = s;
       if (s > mx) mx = s;
     }
@@ -438,7 +464,7 @@ static void graph_slice(const void *ctxp, int32_t b, int32_t h) {
 int svod_oracle_attention_graph(int32_t batch, int32_t t, int32_t tk, int32_t heads, int32_t kv_heads, int32_t d,
                                 int32_t causal, int32_t window_left, int32_t window_right, float scale,
                                 const int32_t *key_lens, const int32_t *key_mask, int32_t mask_stride,
-                                const svod_oracle_ranges *ranges, int32_t bf16_stream, const float *q, const float *k,
+                                const svod_oracle_extras *ranges, int32_t bf16_stream, const float *q, const float *k,
                                 const float *v, float *out, int32_t threads) {
   graph_ctx c = {{batch, t, tk, heads, kv_heads, d, causal, window_left, window_right, scale, key_lens, key_mask,
                   mask_stride, bf16_stream, ranges},
@@ -501,7 +527,7 @@ static void flash_slice(const void *ctxp, int32_t b, int32_t h) {
       int32_t lo = (q_off > p->window_left ? q_off : p->window_left) - p->window_left;
       if (lo / bkv > first) first = lo / bkv;
     }
-    const svod_oracle_ranges *rg = p->ranges;
+    const svod_oracle_extras *rg = p->ranges;
     /* L580-583: the tile's first and last query chunks. */
     const int32_t csize = rg ? rg->chunk_size : 0;
     const int32_t cq0 = csize > 0 ? q_off / csize : 0, cq1 = csize > 0 ? (q_off + (bq - 1)) / csize : 0;
@@ -556,6 +582,9 @@ static void flash_slice(const void *ctxp, int32_t b, int32_t h) {
           }
           double sv = r32(0.0f + (float)dot);
           sv = r32(sv * scale_log2e);
+          /* biased() of L358-362: one fused multiply-add of the bias by log2(e) onto the scaled score. */
+          if (p->ranges && p->ranges->bias && i < t && j < tk)
+            sv = (double)fmaf(bias_at(p, b, h, i, j), 1.44269504088896340736f, (float)sv);
           /* L641-697: a hidden score is -inf.  Applying the predicate on every
            * block equals applying it on edge blocks only (L698-733): on an
            * interior block every key is kept. */
@@ -646,7 +675,7 @@ static void flash_slice(const void *ctxp, int32_t b, int32_t h) {
 int svod_oracle_attention_flash(int32_t batch, int32_t t, int32_t tk, int32_t heads, int32_t kv_heads, int32_t d,
                                 int32_t causal, int32_t window_left, int32_t window_right, float scale,
                                 const int32_t *key_lens, const int32_t *key_mask, int32_t mask_stride,
-                                const svod_oracle_ranges *ranges, int32_t bf16_stream, int32_t bq, int32_t bkv,
+                                const svod_oracle_extras *ranges, int32_t bf16_stream, int32_t bq, int32_t bkv,
                                 const float *q, const float *k, const float *v, float *out, int32_t threads) {
   flash_ctx c = {{batch, t, tk, heads, kv_heads, d, causal, window_left, window_right, scale, key_lens, key_mask,
                   mask_stride, bf16_stream, ranges},
@@ -663,7 +692,7 @@ int svod_oracle_attention_flash(int32_t batch, int32_t t, int32_t tk, int32_t he
 int svod_oracle_attention_flash_split(int32_t batch, int32_t t, int32_t tk, int32_t heads, int32_t kv_heads, int32_t d,
                                       int32_t causal, int32_t window_left, int32_t window_right, float scale,
                                       const int32_t *key_lens, const int32_t *key_mask, int32_t mask_stride,
-                                      const svod_oracle_ranges *ranges, int32_t bf16_stream, int32_t bq, int32_t bkv,
+                                      const svod_oracle_extras *ranges, int32_t bf16_stream, int32_t bq, int32_t bkv,
                                       int32_t splits, const float *q, const float *k, const float *v, float *out,
                                       int32_t threads) {
   flash_ctx c = {{batch, t, tk, heads, kv_heads, d, causal, window_left, window_right, scale, key_lens, key_mask,

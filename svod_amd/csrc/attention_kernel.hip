@@ -155,8 +155,13 @@ __device__ __forceinline__ i32x4 make_rsrc(const void *base, int64_t bytes) {
   return r;
 }
 
+// What a kernel's wave state is compiled for.
+constexpr unsigned kStream = 1;  // a workgroup walks several query tiles
+constexpr unsigned kRanged = 2;  // per-row key ranges: window, chunk mask, segment starts
+constexpr unsigned kBiased = 4;  // an additive bias joins the scaled scores
+
 // Everything a wave carries through the key loop.
-template <int D, int NW, bool F16, bool STREAM, bool RANGED>
+template <int D, int NW, bool F16, unsigned FLAGS>
 struct Wave {
   static constexpr int KS = D / 16;  // k-steps of the score product
   static constexpr int DB = D / 32;  // 32-row blocks of O^T
@@ -173,13 +178,19 @@ struct Wave {
   int lds0;          // LDS byte address of the ring
   int wave, lane, g;
   int wave_first_row, my_row;
-  bool positive;
+  bool positive;  // the maximum is kept in raw score units: a positive scale and no bias (L368-370)
+  // An additive bias (Attn::bias): this lane's row of it, at the tile's first key, and the keys
+  // (from there) the row holds.  Unused unless `biased`.
+  const uint16_t *bias_row;
+  int bias_keys;
+  bool my_row_ok;  // this lane's query row exists (rows past t read no bias)
   float c_exp, unit, limit;
   // Per-row key ranges (a window, a chunk mask, segment starts: tk/src/ops/attention.rs:64-71):
   // this lane's query sees keys [row_lo, row_hi] only, a causal mask already folded into row_hi.
   // Both are non-decreasing in the row, so the wave's first and last rows bound every row's:
   // lo_last, hi_first and hi_last are theirs.  All unused unless `ranged`.
-  static constexpr bool ranged = RANGED;
+  static constexpr bool ranged = (FLAGS & kRanged) != 0;
+  static constexpr bool biased = (FLAGS & kBiased) != 0;
   int row_lo, row_hi;
   int lo_last, hi_first, hi_last;
   // per-lane addressing
@@ -202,8 +213,8 @@ struct Wave {
 // it knows about as aliasing every later LDS read and would park the wave on the NEXT tile's
 // fills in the middle of the current tile.  The kernel waits for them itself (vmcnt(0) before
 // the barrier that ends a step).  m0 carries the LDS address of a wave instruction's 1 KiB.
-template <int D, int NW, bool F16, bool STREAM, bool RANGED>
-__device__ __forceinline__ void fill_tile(const Wave<D, NW, F16, STREAM, RANGED> &w, const uint8_t *base, int64_t bytes, int blk,
+template <int D, int NW, bool F16, unsigned FLAGS>
+__device__ __forceinline__ void fill_tile(const Wave<D, NW, F16, FLAGS> &w, const uint8_t *base, int64_t bytes, int blk,
                                           int lds_at, int src) {
   // This wave's fills of a tile are NW instructions apart; the swizzle repeats with that period,
   // so they share the lanes' offsets and differ in the descriptor's base.
@@ -211,7 +222,7 @@ __device__ __forceinline__ void fill_tile(const Wave<D, NW, F16, STREAM, RANGED>
   static_assert((NW * kRowsPer) % 16 == 0, "the swizzle repeats from one of a wave's fills to its next");
   const int64_t off = (int64_t)blk * kBkv * w.kv_row_bytes;
 #pragma unroll
-  for (int i = 0; i < Wave<D, NW, F16, STREAM, RANGED>::CH; i++) {
+  for (int i = 0; i < Wave<D, NW, F16, FLAGS>::CH; i++) {
     const int64_t at = off + (int64_t)(NW * i * kRowsPer) * w.kv_row_bytes;
     const i32x4 r = make_rsrc(base + at, bytes - at);
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
@@ -222,27 +233,27 @@ __device__ __forceinline__ void fill_tile(const Wave<D, NW, F16, STREAM, RANGED>
 }
 // Block `n` of the stream of blocks that starts with this item's: the item's own while n < end,
 // then (past the padding to an even count) the next item's.  Nothing past either.
-template <int D, int NW, bool F16, bool STREAM, bool RANGED>
-__device__ __forceinline__ void fill_k(const Wave<D, NW, F16, STREAM, RANGED> &w, int n, int slot) {
+template <int D, int NW, bool F16, unsigned FLAGS>
+__device__ __forceinline__ void fill_k(const Wave<D, NW, F16, FLAGS> &w, int n, int slot) {
   const int at = w.lds0 + slot * Tile<D>::kBytes;
   if (n < w.end)
     fill_tile<D, NW>(w, w.k_base, w.kv_bytes, n, at, w.k_src);
-  else if (STREAM && n >= w.end_even && n - w.end_even < w.nxt_end)
+  else if ((FLAGS & kStream) && n >= w.end_even && n - w.end_even < w.nxt_end)
     fill_tile<D, NW>(w, w.nxt_k, w.nxt_bytes, n - w.end_even, at, w.k_src);
 }
-template <int D, int NW, bool F16, bool STREAM, bool RANGED>
-__device__ __forceinline__ void fill_v(const Wave<D, NW, F16, STREAM, RANGED> &w, int n, int slot) {
+template <int D, int NW, bool F16, unsigned FLAGS>
+__device__ __forceinline__ void fill_v(const Wave<D, NW, F16, FLAGS> &w, int n, int slot) {
   const int at = w.lds0 + (2 + slot) * Tile<D>::kBytes;
   if (n < w.end)
     fill_tile<D, NW>(w, w.v_base, w.kv_bytes, n, at, w.v_src);
-  else if (STREAM && n >= w.end_even && n - w.end_even < w.nxt_end)
+  else if ((FLAGS & kStream) && n >= w.end_even && n - w.end_even < w.nxt_end)
     fill_tile<D, NW>(w, w.nxt_v, w.nxt_bytes, n - w.end_even, at, w.v_src);
 }
 
 // A key mask row is read 64 keys (one per lane) a block, one block ahead: the load is issued
 // before that block's fills and is long back when the block's step needs it.
-template <int D, int NW, bool F16, bool STREAM, bool RANGED>
-__device__ __forceinline__ int mask_lane(const Wave<D, NW, F16, STREAM, RANGED> &w, int blk) {
+template <int D, int NW, bool F16, unsigned FLAGS>
+__device__ __forceinline__ int mask_lane(const Wave<D, NW, F16, FLAGS> &w, int blk) {
   const int key = blk * kBkv + w.lane;
   if (w.key_mask == nullptr || key >= w.tk) return 0;
   const int64_t at = w.mask_row + key;
@@ -251,14 +262,14 @@ __device__ __forceinline__ int mask_lane(const Wave<D, NW, F16, STREAM, RANGED> 
 
 // S^T = K . Q^T of the key block in K slot `slot`, as 32 scalars: sv[16kb + i] is the score of
 // key 32kb + 8(i/4) + 4g + i%4 (sub-registers of the two accumulators: no moves).
-template <int D, int NW, bool F16, bool STREAM, bool RANGED>
-__device__ __forceinline__ void scores(const Wave<D, NW, F16, STREAM, RANGED> &w, const uint8_t *smem, int slot, float (&sv)[32]) {
+template <int D, int NW, bool F16, unsigned FLAGS>
+__device__ __forceinline__ void scores(const Wave<D, NW, F16, FLAGS> &w, const uint8_t *smem, int slot, float (&sv)[32]) {
   using TL = Tile<D>;
   const uint8_t *ks_ = smem + slot * TL::kBytes;
   const f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
   f32x16 s0 = zero, s1 = zero;
 #pragma unroll
-  for (int ks = 0; ks < Wave<D, NW, F16, STREAM, RANGED>::KS; ks++) {
+  for (int ks = 0; ks < Wave<D, NW, F16, FLAGS>::KS; ks++) {
     const u32x4 a0 = *reinterpret_cast<const u32x4 *>(ks_ + w.k_read[ks]);
     const u32x4 a1 = *reinterpret_cast<const u32x4 *>(ks_ + w.k_read[ks] + 32 * TL::kRowBytes);
     s0 = mma<F16>(a0, w.qf[ks], s0);
@@ -273,8 +284,8 @@ __device__ __forceinline__ void scores(const Wave<D, NW, F16, STREAM, RANGED> &w
 
 // The wave-uniform part of block `blk`'s mask: bit j = key 64 blk + j is below the length and
 // kept by the key mask (`word` is this lane's key-mask element of the block).
-template <int D, int NW, bool F16, bool STREAM, bool RANGED>
-__device__ __forceinline__ uint64_t uniform_bits(const Wave<D, NW, F16, STREAM, RANGED> &w, int blk, int word) {
+template <int D, int NW, bool F16, unsigned FLAGS>
+__device__ __forceinline__ uint64_t uniform_bits(const Wave<D, NW, F16, FLAGS> &w, int blk, int word) {
   const int k0 = blk * kBkv;
   uint64_t kbits = ~0ull;
   if (w.key_mask != nullptr) kbits = __builtin_amdgcn_ballot_w64(word != 0);
@@ -282,9 +293,54 @@ __device__ __forceinline__ uint64_t uniform_bits(const Wave<D, NW, F16, STREAM, 
   return kbits;
 }
 
+// The 32 bias elements this lane's scores of block `blk` take, as 16 packed pairs: keys
+// k0 + 32 kb + 8 c + 4 g + {0..3}.  Keys past the row read as zero (their scores are hidden anyway).
+template <int D, int NW, bool F16, unsigned FLAGS>
+__device__ __forceinline__ void load_bias(const Wave<D, NW, F16, FLAGS> &w, int blk, bool row_ok, uint32_t (&bw)[16]) {
+  const int k0 = blk * kBkv + 4 * w.g;
+  const bool aligned = ((uintptr_t)w.bias_row & 7u) == 0;  // wave-uniform when every row is: checked per lane
+#pragma unroll
+  for (int c = 0; c < 8; c++) {
+    const int key = k0 + 32 * (c / 4) + 8 * (c % 4);
+    uint32_t lo = 0, hi = 0;
+    if (row_ok && aligned && key + 3 < w.bias_keys) {
+      const u32x2 x = *reinterpret_cast<const u32x2 *>(w.bias_row + key);
+      lo = x[0];
+      hi = x[1];
+    } else if (row_ok) {
+      const uint32_t e0 = key + 0 < w.bias_keys ? w.bias_row[key + 0] : 0u;
+      const uint32_t e1 = key + 1 < w.bias_keys ? w.bias_row[key + 1] : 0u;
+      const uint32_t e2 = key + 2 < w.bias_keys ? w.bias_row[key + 2] : 0u;
+      const uint32_t e3 = key + 3 < w.bias_keys ? w.bias_row[key + 3] : 0u;
+      lo = e0 | e1 << 16;
+      hi = e2 | e3 << 16;
+    }
+    bw[2 * c] = lo;
+    bw[2 * c + 1] = hi;
+  }
+}
+
+// biased() of L358-362: s = fma(bias, log2(e), s) on the scaled scores, before the masks.
+template <bool F16>
+__device__ __forceinline__ void add_bias(const uint32_t (&bw)[16], float (&sv)[32]) {
+#pragma unroll
+  for (int i = 0; i < 32; i++) {
+    const uint32_t pair = bw[i / 2];
+    const uint16_t e = (uint16_t)((i & 1) ? pair >> 16 : pair & 0xffffu);
+    float x;
+    if (F16) {
+      x = (float)__builtin_bit_cast(_Float16, e);
+    } else {
+      const uint32_t wide = (uint32_t)e << 16;
+      x = __builtin_bit_cast(float, wide);
+    }
+    sv[i] = __builtin_fmaf(x, kLog2e, sv[i]);
+  }
+}
+
 // Whether a mask edge crosses block `blk` for this wave (L698-733).
-template <int D, int NW, bool CAUSAL, bool F16, bool STREAM, bool RANGED>
-__device__ __forceinline__ bool on_edge(const Wave<D, NW, F16, STREAM, RANGED> &w, int blk, uint64_t kbits) {
+template <int D, int NW, bool CAUSAL, bool F16, unsigned FLAGS>
+__device__ __forceinline__ bool on_edge(const Wave<D, NW, F16, FLAGS> &w, int blk, uint64_t kbits) {
   const int k0 = blk * kBkv;
   if (kbits != ~0ull) return true;
   // L715-731: a range's right edge for the wave's first row, its left edge for the last.
@@ -294,8 +350,8 @@ __device__ __forceinline__ bool on_edge(const Wave<D, NW, F16, STREAM, RANGED> &
 
 // Scales (a non-positive scale only) and masks (L641-697) the scores of block `blk`: hidden
 // scores become -inf.  `kbits` is the uniform word; causality adds a per-lane one.
-template <int D, int NW, bool CAUSAL, bool F16, bool STREAM, bool RANGED>
-__device__ __forceinline__ void mask_scores(const Wave<D, NW, F16, STREAM, RANGED> &w, int blk, uint64_t kbits, float (&sv)[32]) {
+template <int D, int NW, bool CAUSAL, bool F16, unsigned FLAGS>
+__device__ __forceinline__ void mask_scores(const Wave<D, NW, F16, FLAGS> &w, int blk, uint64_t kbits, float (&sv)[32]) {
   const int k0 = blk * kBkv;
   uint64_t mine = kbits;
   if (w.ranged) {
@@ -352,15 +408,15 @@ __device__ __forceinline__ void probabilities(const float *sv, float unit, float
 }
 
 // O^T += V^T . P^T over 32 keys (half a block): chunks c of 16 keys, fragment registers 4c..4c+3.
-template <int D, int NW, bool F16, bool STREAM, bool RANGED>
-__device__ __forceinline__ void accumulate(Wave<D, NW, F16, STREAM, RANGED> &w, const uint8_t *vs_, int half, const uint32_t *pk) {
+template <int D, int NW, bool F16, unsigned FLAGS>
+__device__ __forceinline__ void accumulate(Wave<D, NW, F16, FLAGS> &w, const uint8_t *vs_, int half, const uint32_t *pk) {
   using TL = Tile<D>;
 #pragma unroll
   for (int c = 0; c < 2; c++) {
     const u32x4 pw = {pk[4 * c], pk[4 * c + 1], pk[4 * c + 2], pk[4 * c + 3]};
 
 #pragma unroll
-    for (int db = 0; db < Wave<D, NW, F16, STREAM, RANGED>::DB; db++) {
+    for (int db = 0; db < Wave<D, NW, F16, FLAGS>::DB; db++) {
       const uint8_t *at = vs_ + w.v_read[db] + (32 * half + 16 * c) * TL::kRowBytes;
       const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_PTR(s16x4))(at));
       const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_PTR(s16x4))(at + 8 * TL::kRowBytes));
@@ -373,8 +429,8 @@ __device__ __forceinline__ void accumulate(Wave<D, NW, F16, STREAM, RANGED> &w, 
 // The running maximum's update for a block whose row maximum is `bm`: the lazy rescale of
 // L418-431, and the O^T rescale that a wave skips when all its rows kept their maximum
 // (L56-59).  Returns the exponent's offset m*unit; `corr` is the correction of l.
-template <int D, int NW, bool F16, bool STREAM, bool RANGED>
-__device__ __forceinline__ float adopt_maximum(Wave<D, NW, F16, STREAM, RANGED> &w, float bm, float &corr) {
+template <int D, int NW, bool F16, unsigned FLAGS>
+__device__ __forceinline__ float adopt_maximum(Wave<D, NW, F16, FLAGS> &w, float bm, float &corr) {
   const float m_max = __builtin_fmaxf(w.m_run, bm);
   const bool grows = w.limit < (m_max - w.m_run);
   const float m_new = grows ? m_max : w.m_run;
@@ -382,7 +438,7 @@ __device__ __forceinline__ float adopt_maximum(Wave<D, NW, F16, STREAM, RANGED> 
   w.m_run = m_new;
   if (__builtin_amdgcn_ballot_w64(corr != 1.0f) != 0) {
 #pragma unroll
-    for (int db = 0; db < Wave<D, NW, F16, STREAM, RANGED>::DB; db++) w.acc[db] *= corr;
+    for (int db = 0; db < Wave<D, NW, F16, FLAGS>::DB; db++) w.acc[db] *= corr;
   }
   return m_new * w.unit;
 }
@@ -413,11 +469,11 @@ __device__ __forceinline__ uint32_t p_unit(float s_a, float s_b, float unit, flo
 // never waits for the VALU's whole job.  2 KS slots compute S(blk+1) beside the exponentials
 // of keys 0..31; 2 DB slots add P V of keys 0..31 beside the exponentials of keys 32..63;
 // 2 DB slots add P V of keys 32..63 beside the row maximum of S(blk+1).
-template <int D, int NW, int PAR, bool F16, bool STREAM, bool RANGED>
-__device__ __forceinline__ void hot_step(Wave<D, NW, F16, STREAM, RANGED> &w, const uint8_t *smem, int blk, const float (&sv)[32],
+template <int D, int NW, int PAR, bool F16, unsigned FLAGS>
+__device__ __forceinline__ void hot_step(Wave<D, NW, F16, FLAGS> &w, const uint8_t *smem, int blk, const float (&sv)[32],
                                          float (&nv)[32], float &bm) {
   using TL = Tile<D>;
-  constexpr int KS = Wave<D, NW, F16, STREAM, RANGED>::KS, DB = Wave<D, NW, F16, STREAM, RANGED>::DB;
+  constexpr int KS = Wave<D, NW, F16, FLAGS>::KS, DB = Wave<D, NW, F16, FLAGS>::DB;
   constexpr int NQK = 2 * KS;  // score slots
   constexpr int NPV = 4 * DB;  // P V slots, half of them per 32 keys
   const uint8_t *ks_ = smem + (PAR ^ 1) * TL::kBytes;
@@ -514,13 +570,16 @@ __device__ __forceinline__ void hot_step(Wave<D, NW, F16, STREAM, RANGED> &w, co
 // The general step, for the blocks at the edges: any block, a next block or none, masks, any
 // scale.  Slots are picked at run time.  `sv` holds the masked S(blk) and `bm` its row maximum;
 // on exit they hold block blk+1's (when this wave has one).
-template <int D, int NW, bool CAUSAL, bool F16, bool STREAM, bool RANGED>
-__device__ __forceinline__ void edge_step(Wave<D, NW, F16, STREAM, RANGED> &w, const uint8_t *smem, int blk, int my_end, float (&sv)[32],
+template <int D, int NW, bool CAUSAL, bool F16, unsigned FLAGS>
+__device__ __forceinline__ void edge_step(Wave<D, NW, F16, FLAGS> &w, const uint8_t *smem, int blk, int my_end, float (&sv)[32],
                                           float &bm) {
   using TL = Tile<D>;
   const int par = blk & 1;
   const bool more = blk + 1 < my_end;
   const uint64_t kbits_next = uniform_bits<D, NW>(w, blk + 1, w.mask_next);
+  // The next block's bias is asked for first: it has this block's P.V to arrive under.
+  uint32_t bw[16];
+  if (w.biased && more) load_bias<D, NW>(w, blk + 1, w.my_row_ok, bw);
   fill_v<D, NW>(w, blk + 1, par ^ 1);
   if (blk + 2 < w.end) w.mask_next = mask_lane<D, NW>(w, blk + 2);
   fill_k<D, NW>(w, blk + 2, par);
@@ -541,6 +600,7 @@ __device__ __forceinline__ void edge_step(Wave<D, NW, F16, STREAM, RANGED> &w, c
 #pragma unroll
       for (int i = 0; i < 32; i++) sv[i] *= w.c_exp;
     }
+    if (w.biased) add_bias<F16>(bw, sv);
     if (on_edge<D, NW, CAUSAL>(w, blk + 1, kbits_next)) mask_scores<D, NW, CAUSAL>(w, blk + 1, kbits_next, sv);
     bm = row_max(sv);
   }
@@ -549,8 +609,8 @@ __device__ __forceinline__ void edge_step(Wave<D, NW, F16, STREAM, RANGED> &w, c
 }
 
 // A step of a wave with nothing to compute: fills and the barrier only.
-template <int D, int NW, bool F16, bool STREAM, bool RANGED>
-__device__ __forceinline__ void idle_step(Wave<D, NW, F16, STREAM, RANGED> &w, int blk) {
+template <int D, int NW, bool F16, unsigned FLAGS>
+__device__ __forceinline__ void idle_step(Wave<D, NW, F16, FLAGS> &w, int blk) {
   const int par = blk & 1;
   fill_v<D, NW>(w, blk + 1, par ^ 1);
   fill_k<D, NW>(w, blk + 2, par);
@@ -580,7 +640,8 @@ struct Splits {
   uint32_t nbatch;
 };
 
-// The per-row masks of a launch that has them (the RANGED instantiations).
+// The per-row masks (the RANGED instantiations) and the bias (the BIASED ones) of a launch that
+// has them.
 struct Ranges {
   int32_t win_left, win_right;  // win_left < 0: no window; the host caps both at t + tk
   int32_t chunk_size;           // 0: no chunk mask (Chunk of tk/src/ops/attention.rs:39-50)
@@ -588,10 +649,12 @@ struct Ranges {
   int32_t chunk_right;          // the host caps it at the chunks of the keys
   const void *seg_start;        // [B, T] integers or null
   int32_t seg_i64;
+  const uint16_t *bias;         // [B or 1, H, T, Tk] of the operands' type, or null
+  int32_t bias_per_batch;
 };
 
-template <int D, int NW, bool CAUSAL, bool SPLIT, bool RANGED, bool F16>
-__global__ __launch_bounds__(NW * 64, D == 64 ? 3 : 2) void flash_fwd_kernel(
+template <int D, int NW, bool CAUSAL, bool SPLIT, bool RANGED, bool BIASED, bool F16>
+__global__ __launch_bounds__(NW * 64, (D == 64 && !BIASED) ? 3 : 2) void flash_fwd_kernel(
     uint32_t unit_size, uint32_t unit_rcp, uint32_t nqt_u, uint32_t nqt_rcp, uint32_t kvh_u, uint32_t kvh_rcp,
     uint32_t units, uint32_t heads_group, const void *__restrict__ key_lens, const uint16_t *__restrict__ q, int32_t t,
     uint32_t tk_lens64, const uint16_t *__restrict__ k, const uint16_t *__restrict__ v,
@@ -609,7 +672,7 @@ __global__ __launch_bounds__(NW * 64, D == 64 ? 3 : 2) void flash_fwd_kernel(
   const int tk = (int)(tk_lens64 & 0x7fffffffu);
   const bool lens_i64 = (tk_lens64 >> 31) != 0;
   using TL = Tile<D>;
-  using W = Wave<D, NW, F16, false, RANGED>;
+  using W = Wave<D, NW, F16, (RANGED ? kRanged : 0u) | (BIASED ? kBiased : 0u)>;
   constexpr int BQ = NW * kWaveRows;
   constexpr int KS = W::KS, DB = W::DB;
   static_assert(TL::kInstrs % NW == 0, "the tile fills in whole wave instructions per wave");
@@ -734,6 +797,13 @@ __global__ __launch_bounds__(NW * 64, D == 64 ? 3 : 2) void flash_fwd_kernel(
   w.mask_bytes = mask_bytes;
   w.wave_first_row = q_off + w.wave * kWaveRows - first_key;
   w.my_row = w.wave_first_row + ln;
+  w.my_row_ok = row < t;
+  if (BIASED) {
+    // L566-571: the bias of this (batch or 0, head), this lane's row, from the tile's first key on.
+    const int64_t brow = ((int64_t)(rg.bias_per_batch ? b : 0) * heads + h) * t + min(row, t - 1);
+    w.bias_row = rg.bias + brow * tk + first_key;
+    w.bias_keys = tk - first_key;
+  }
   if (RANGED) {
     w.row_lo -= first_key;
     w.row_hi -= first_key;
@@ -784,7 +854,7 @@ __global__ __launch_bounds__(NW * 64, D == 64 ? 3 : 2) void flash_fwd_kernel(
   // ---- online softmax state.  m in RAW score units (raw_max form) when the scale is positive;
   // otherwise the maximum does not commute with it: the scores are scaled first and m lives
   // in the exponent's units (L365-370).
-  w.positive = scale > 0.0f;
+  w.positive = scale > 0.0f && !BIASED;
   w.c_exp = scale * kLog2e;  // L619
   w.unit = w.positive ? w.c_exp : 1.0f;
   w.limit = kRescaleAbove / w.unit;
@@ -814,11 +884,14 @@ __global__ __launch_bounds__(NW * 64, D == 64 ? 3 : 2) void flash_fwd_kernel(
 #pragma unroll
   for (int i = 0; i < 32; i++) sv[i] = nv[i] = 0.0f;
   if (my_end > 0) {
+    uint32_t bw[16];
+    if (BIASED) load_bias<D, NW>(w, 0, row < t, bw);
     scores<D, NW>(w, smem, 0, sv);
     if (!w.positive) {
 #pragma unroll
       for (int i = 0; i < 32; i++) sv[i] *= w.c_exp;
     }
+    if (BIASED) add_bias<F16>(bw, sv);
     const uint64_t kbits0 = uniform_bits<D, NW>(w, 0, word0);
     if (on_edge<D, NW, CAUSAL>(w, 0, kbits0)) mask_scores<D, NW, CAUSAL>(w, 0, kbits0, sv);
     bm = row_max(sv);
@@ -956,7 +1029,7 @@ __global__ __launch_bounds__(NW * 64, 3) void flash_stream_kernel(
   const int tk = (int)(tk_lens64 & 0x7fffffffu);
   const bool lens_i64 = (tk_lens64 >> 31) != 0;
   using TL = Tile<D>;
-  using W = Wave<D, NW, F16, true, false>;
+  using W = Wave<D, NW, F16, kStream>;
   constexpr int BQ = NW * kWaveRows;
   constexpr int KS = W::KS, DB = W::DB;
   constexpr int kStageRows = 1024 / TL::kRowBytes;                  // rows a wave instruction stages
@@ -1234,7 +1307,7 @@ hipError_t launch_stream(const AttnArgs &a, hipStream_t stream, int64_t slots, c
   return hipGetLastError();
 }
 
-template <int D, int NW, bool CAUSAL, bool SPLIT, bool RANGED, bool F16>
+template <int D, int NW, bool CAUSAL, bool SPLIT, bool RANGED, bool BIASED, bool F16>
 hipError_t launch(const AttnArgs &a, hipStream_t stream) {
   using TL = Tile<D>;
   constexpr int BQ = NW * kWaveRows;
@@ -1248,7 +1321,7 @@ hipError_t launch(const AttnArgs &a, hipStream_t stream) {
   const int64_t kv_row = a.kv_row_elems > 0 ? a.kv_row_elems : (int64_t)a.kv_heads * a.d;
   // The fills address a (batch, kv head)'s rows with 32-bit byte offsets.
   if ((int64_t)a.tk * kv_row * 2 > 0x7fffffffLL || q_row > 0x7fffffffLL) return hipErrorInvalidValue;
-  auto kernel = flash_fwd_kernel<D, NW, CAUSAL, SPLIT, RANGED, F16>;
+  auto kernel = flash_fwd_kernel<D, NW, CAUSAL, SPLIT, RANGED, BIASED, F16>;
   // The LDS ring is above the default limit of a launch: one attribute call per instantiation
   // and device, from whichever thread gets there first (a second call is harmless).
   static std::atomic<uint64_t> configured{0};  // a bit per device ordinal, devices past 63 always ask
@@ -1281,7 +1354,7 @@ hipError_t launch(const AttnArgs &a, hipStream_t stream) {
   // The streaming form, where asked for and where it has a kernel (head size 64, lengths or no
   // key mask, no window, no splits): `knob` workgroups per XCD, each walking its run of tiles.
   // It is never chosen unasked: measured, it has not beaten a workgroup per tile.
-  if constexpr (D == 64 && !SPLIT && !RANGED) {
+  if constexpr (D == 64 && !SPLIT && !RANGED && !BIASED) {
     const int knob = g_stream_slots.load(std::memory_order_relaxed);
     if (knob > 0 && a.key_mask == nullptr)
       return launch_stream<D, NW, CAUSAL, F16>(a, stream, knob, geo, q_row, kv_row);
@@ -1304,6 +1377,8 @@ hipError_t launch(const AttnArgs &a, hipStream_t stream) {
   rg.chunk_right = a.chunk_right;
   rg.seg_start = a.seg_start;
   rg.seg_i64 = a.seg_i64;
+  rg.bias = (const uint16_t *)a.bias;
+  rg.bias_per_batch = a.bias_per_batch;
   hipLaunchKernelGGL(kernel, dim3((uint32_t)grid), dim3(NW * 64), smem, stream, geo.unit_size, geo.unit_rcp, geo.nqt,
                      geo.nqt_rcp, geo.kv_heads, geo.kvh_rcp, geo.units, heads_group, a.key_lens,
                      (const uint16_t *)a.q, a.t, tk_lens64, (const uint16_t *)a.k,
@@ -1312,18 +1387,22 @@ hipError_t launch(const AttnArgs &a, hipStream_t stream) {
   return hipGetLastError();
 }
 
-template <int D, bool RANGED, bool F16>
+template <int D, bool RANGED, bool BIASED, bool F16>
 hipError_t launch_s(const AttnArgs &a, hipStream_t stream) {
   if (a.splits > 1)
-    return a.causal ? launch<D, 4, true, true, RANGED, F16>(a, stream) : launch<D, 4, false, true, RANGED, F16>(a, stream);
-  return a.causal ? launch<D, 4, true, false, RANGED, F16>(a, stream) : launch<D, 4, false, false, RANGED, F16>(a, stream);
+    return a.causal ? launch<D, 4, true, true, RANGED, BIASED, F16>(a, stream)
+                    : launch<D, 4, false, true, RANGED, BIASED, F16>(a, stream);
+  return a.causal ? launch<D, 4, true, false, RANGED, BIASED, F16>(a, stream)
+                  : launch<D, 4, false, false, RANGED, BIASED, F16>(a, stream);
 }
 
 template <int D, bool F16>
 hipError_t launch_t(const AttnArgs &a, hipStream_t stream) {
   // A window, a chunk mask or segment starts: the instantiations with per-row key ranges.
   const bool ranged = a.win_left >= 0 || a.chunk_size > 0 || a.seg_start != nullptr;
-  return ranged ? launch_s<D, true, F16>(a, stream) : launch_s<D, false, F16>(a, stream);
+  if (a.bias != nullptr)
+    return ranged ? launch_s<D, true, true, F16>(a, stream) : launch_s<D, false, true, F16>(a, stream);
+  return ranged ? launch_s<D, true, false, F16>(a, stream) : launch_s<D, false, false, F16>(a, stream);
 }
 
 template <int D>

@@ -59,6 +59,10 @@ struct AttnArgs {
   // non-decreasing along t; query i does not see keys before seg_start[b, i].  Null = none.
   const void *seg_start;
   int32_t seg_i64;
+  // Attn::bias (tk/src/ops/attention.rs:82-85): [batch or 1, heads, t, tk] of the operands' type,
+  // rows unpadded, added to the scaled scores before the masks.  Null = none.
+  const void *bias;
+  int32_t bias_per_batch;
 };
 hipError_t launch_attention(const AttnArgs &a, hipStream_t stream);
 

@@ -333,7 +333,7 @@ static int attend(const svodk_tensor *q, const svodk_tensor *k, const svodk_tens
   if (why != 0) return ran_graph(op, why);
   // Options the reference's kernel holds and this library's does not: no
   // config here holds them (the reference's own use of Fallback::Config, L210-214).
-  if (opts->has_cache || opts->bias != nullptr) return ran_graph(op, SVODK_GRAPH_CONFIG);
+  if (opts->has_cache) return ran_graph(op, SVODK_GRAPH_CONFIG);
   if (opts->has_window && (opts->window_left < 0 || opts->window_right < 0))
     return fail(SVODK_ERR_ARGUMENT, "%s: a negative window reach", op);
   // Chunk { size, left, right } of tk/src/ops/attention.rs:39-50: usize fields, a size of at least 1.
@@ -359,7 +359,7 @@ static int attend(const svodk_tensor *q, const svodk_tensor *k, const svodk_tens
                     bools ? (size_t)numel(bools) * dtype_bytes(bools->dtype) : 0, false}};
   if (q->data == nullptr || k->data == nullptr || v->data == nullptr || out->data == nullptr ||
       (lens && lens->data == nullptr) || (bools && bools->data == nullptr) ||
-      (opts->seg_start && opts->seg_start->data == nullptr))
+      (opts->seg_start && opts->seg_start->data == nullptr) || (opts->bias && opts->bias->data == nullptr))
     return fail(SVODK_ERR_ARGUMENT, "%s: a null device pointer", op);
   if (int rc = check_aliasing(op, spans, 6)) return rc;
   if (opts->seg_start != nullptr) {
@@ -400,6 +400,12 @@ static int attend(const svodk_tensor *q, const svodk_tensor *k, const svodk_tens
     a.chunk_left = opts->chunk_has_left ? (int32_t)std::min<int64_t>(opts->chunk_left, chunks) : -1;
     a.chunk_right = (int32_t)std::min<int64_t>(opts->chunk_right, chunks);
     if (t + tk > 0x3fffffff) return ran_graph(op, SVODK_GRAPH_SHAPE);  // chunk edges stay 32-bit
+  }
+  if (opts->bias != nullptr) {
+    Span pair[2] = {{"bias", opts->bias->data, (size_t)numel(opts->bias) * 2, false}, spans[3]};
+    if (int rc = check_aliasing(op, pair, 2)) return rc;
+    a.bias = opts->bias->data;
+    a.bias_per_batch = opts->bias->shape[0] != 1 || cap == 1;
   }
   if (opts->seg_start != nullptr) {
     a.seg_start = opts->seg_start->data;

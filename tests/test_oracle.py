@@ -462,3 +462,55 @@ def test_tile_program_skips_only_hidden_blocks(name, masks, lens, tile, splits):
     key_mask = (np.add.outer(np.arange(b), np.arange(t)) % 5 != 2) if masks.pop("key_mask", False) else None
     p = oracle.AttnProblem(q, k, v, key_lens=None if lens is None else np.array(lens), key_mask=key_mask, seg_start=seg, **masks)
     assert max_abs(oracle.attention_flash(p, bq=tile[0], bkv=tile[1], splits=splits), oracle.attention_direct(p)) < 2e-2
+
+
+# ---------------------------------------------------------------- additive bias
+def biased_case(rows, b=2, t=37, tk=50, h=4, hkv=2, d=16):
+    g = Lcg(5)
+    q, k, v = g.bf16((b, t, h, d)), g.bf16((b, tk, hkv, d)), g.bf16((b, tk, hkv, d))
+    return q, k, v, g.bf16((rows, h, t, tk), mul=2.0)
+
+
+def torch_biased(q, k, v, bias, lens=None, causal=False):
+    """torch's float64 scaled_dot_product_attention with the bias (and the masks as -inf) as its attn_mask."""
+    group = q.shape[2] // k.shape[2]
+    tq = torch.tensor(q, dtype=torch.float64).permute(0, 2, 1, 3)
+    tk_, tv = (torch.tensor(x, dtype=torch.float64).permute(0, 2, 1, 3).repeat_interleave(group, 1) for x in (k, v))
+    m = torch.tensor(bias, dtype=torch.float64).expand(q.shape[0], -1, -1, -1).clone()
+    if lens is not None:
+        m = m.masked_fill(~(torch.arange(k.shape[1])[None, :] < torch.tensor(lens)[:, None])[:, None, None, :], float("-inf"))
+    if causal:
+        m = m.masked_fill(torch.arange(k.shape[1])[None, :] > torch.arange(q.shape[1])[:, None], float("-inf"))
+    return torch.nn.functional.scaled_dot_product_attention(tq, tk_, tv, attn_mask=m).permute(0, 2, 1, 3).numpy()
+
+
+@pytest.mark.parametrize("rows", [1, 2], ids=["shared", "per batch"])
+@pytest.mark.parametrize("lens,causal", [(None, False), ([50, 33], False), (None, True)], ids=["no mask", "lens", "causal"])
+def test_biased_attention_matches_torch_float64(rows, lens, causal):
+    q, k, v, bias = biased_case(rows)
+    want = torch_biased(q, k, v, bias, lens, causal)
+    p = oracle.AttnProblem(q, k, v, bias=bias, causal=causal, key_lens=None if lens is None else np.array(lens))
+    assert max_abs(oracle.attention_direct(p), want) < 1e-12
+    assert max_abs(oracle.attention_flash(p), want) < 2e-2                       # attention.rs:483
+    assert max_abs(oracle.attention_flash(p, bq=128, bkv=64, splits=2), want) < 2e-2
+    assert max_abs(oracle.attention_graph(p), want) < 2e-2
+
+
+def test_bias_closed_forms():
+    q, k, v, bias = biased_case(2)
+    plain = oracle.attention_direct(oracle.AttnProblem(q, k, v))
+    # The same number added to every score of a row leaves its softmax unchanged.
+    flat = np.broadcast_to(np.linspace(-3, 3, q.shape[1], dtype=np.float32)[None, None, :, None], bias.shape)
+    assert max_abs(oracle.attention_direct(oracle.AttnProblem(q, k, v, bias=flat)), plain) < 1e-12
+    # A bias of -inf on a key is a key mask.
+    hide = np.add.outer(np.arange(2), np.arange(k.shape[1])) % 5 == 2
+    walls = np.where(hide[:, None, None, :], -np.inf, 0.0).astype(np.float32) * np.ones_like(bias)
+    masked = oracle.attention_direct(oracle.AttnProblem(q, k, v, key_mask=~hide))
+    for path, tol in ((oracle.attention_direct, 1e-12), (oracle.attention_flash, 2e-2)):
+        assert max_abs(path(oracle.AttnProblem(q, k, v, bias=walls)), masked) < tol
+    # With zero queries the bias alone sets the weights: out = softmax(bias) . v.
+    p = oracle.AttnProblem(np.zeros_like(q), k, v, bias=bias)
+    w = np.exp(bias.astype(np.float64))
+    w /= w.sum(-1, keepdims=True)
+    want = np.einsum("bhij,bjhd->bihd", w, np.repeat(v.astype(np.float64), 2, axis=2))
+    assert max_abs(oracle.attention_direct(p), want) < 1e-12

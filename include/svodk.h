@@ -23,7 +23,7 @@
 extern "C" {
 #endif
 
-#define SVODK_ABI_VERSION 2
+#define SVODK_ABI_VERSION 3
 
 /* Element types of a tensor descriptor. */
 typedef enum svodk_dtype {
@@ -72,12 +72,31 @@ typedef enum svodk_key_mask {
 } svodk_key_mask;
 
 /*
+ * Cache of tk/src/ops/attention.rs:39-56: k and v are caches [rows, Tk, H_all, D]
+ * holding several layers' heads (a decoder step's self or cross attention).
+ * Query head h reads cache head head_start + h / (H / kv_heads) of cache row
+ * row_map[b] (row b without a map).  `k_app`/`v_app` [B, n, kv_heads, D] are keys
+ * and values scored after the cached prefix (the tokens the step projected, not
+ * yet written to the cache): they need SVODK_KEYS_LENS naming the prefix, n is
+ * at most a key block (64) and only the first app_lens[b] of them are seen
+ * (all without app_lens).  Masks other than the key lengths do not reach them.
+ */
+typedef struct svodk_cache {
+  int64_t head_start, kv_heads;
+  const svodk_tensor *row_map;  /* [B] I32 or I64, or NULL */
+  const svodk_tensor *k_app;    /* both or neither */
+  const svodk_tensor *v_app;
+  const svodk_tensor *app_lens; /* [B] I32 or I64, or NULL; needs k_app */
+} svodk_cache;
+
+/*
  * Attn of tk/src/ops/attention.rs:60-86.  Zero-initialise, then set fields.
  * Windows, chunk masks, segment starts (I32 or I64, non-decreasing along T)
- * and an additive bias (of the operands' type, rows unpadded) have kernels,
- * alone or together with every other option.  A cache, which this library has
- * no kernel for, is still validated as the reference validates it and then
- * answered with SVODK_GRAPH_CONFIG.
+ * an additive bias (of the operands' type, rows unpadded; with appended rows
+ * its last dim counts them, their columns last) and a cache have kernels.
+ * Every combination the reference's own tests hold runs; a cache together with
+ * a window, a chunk mask or segment starts, and more than 64 appended rows,
+ * answer SVODK_GRAPH_CONFIG.
  *
  * `splits` > 1 asks for key splits (tk/src/ops/attention.rs:79, 280-302): the
  * count is capped at the number of 64-key blocks of Tk (split_ranked, :405-410);
@@ -99,7 +118,7 @@ typedef struct svodk_attn {
   int32_t chunk_has_left;
   int64_t chunk_left, chunk_right;
   const svodk_tensor *seg_start; /* [B, T] integers or NULL */
-  int32_t has_cache;             /* Cache{..}: never a kernel here */
+  const svodk_cache *cache;      /* or NULL */
   const svodk_tensor *bias;      /* [B|1, H, T, Tk] or NULL */
   int32_t splits;                /* 0 = None */
   int32_t has_scale;

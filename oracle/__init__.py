@@ -10,6 +10,7 @@ share.
 from __future__ import annotations
 
 import ctypes
+import dataclasses
 import os
 import subprocess
 from dataclasses import dataclass
@@ -53,23 +54,37 @@ class _Ranges(ctypes.Structure):
 
     _fields_ = [("chunk_size", ctypes.c_int32), ("chunk_has_left", ctypes.c_int32), ("chunk_left", ctypes.c_int32),
                 ("chunk_right", ctypes.c_int32), ("seg_start", ctypes.POINTER(ctypes.c_int32)),
-                ("bias", ctypes.POINTER(ctypes.c_float)), ("bias_per_batch", ctypes.c_int32)]
+                ("bias", ctypes.POINTER(ctypes.c_float)), ("bias_per_batch", ctypes.c_int32),
+                ("bias_cols", ctypes.c_int32), ("appended", ctypes.c_int32),
+                ("k_app", ctypes.POINTER(ctypes.c_float)), ("v_app", ctypes.POINTER(ctypes.c_float)),
+                ("app_seen", ctypes.POINTER(ctypes.c_int32))]
 
 
 _rangesp = ctypes.POINTER(_Ranges)
 
 
-def _ranges(chunk, seg_start, bias=None, batch=None):
-    """(pointer or None, what must stay alive) for ``chunk = (size, left or None, right)``, ``seg_start [B,T]``
-    and ``bias [B or 1, H, T, Tk]``."""
-    if chunk is None and seg_start is None and bias is None:
+def _ranges(chunk, seg_start, bias=None, batch=None, appended=None):
+    """(pointer or None, what must stay alive) for ``chunk = (size, left or None, right)``, ``seg_start [B,T]``,
+    ``bias [B or 1, H, T, Tk (+ appended rows)]`` and ``appended = (k_app, v_app, seen or None)``."""
+    if chunk is None and seg_start is None and bias is None and appended is None:
         return None, None
     r = _Ranges()
     seg = None
+    if appended is not None:
+        k_app, v_app, seen = appended
+        k_app, v_app = (np.ascontiguousarray(x, dtype=np.float32) for x in (k_app, v_app))
+        seen = None if seen is None else np.ascontiguousarray(seen, dtype=np.int32)
+        r.appended = k_app.shape[1]
+        r.k_app = k_app.ctypes.data_as(ctypes.POINTER(ctypes.c_float))
+        r.v_app = v_app.ctypes.data_as(ctypes.POINTER(ctypes.c_float))
+        if seen is not None:
+            r.app_seen = seen.ctypes.data_as(ctypes.POINTER(ctypes.c_int32))
+        appended = (k_app, v_app, seen)
     if bias is not None:
         bias = np.ascontiguousarray(bias, dtype=np.float32)
         r.bias = bias.ctypes.data_as(ctypes.POINTER(ctypes.c_float))
         r.bias_per_batch = int(bias.shape[0] != 1 or batch == 1)
+        r.bias_cols = bias.shape[3]
     if chunk is not None:
         size, left, right = chunk
         r.chunk_size, r.chunk_has_left = int(size), int(left is not None)
@@ -77,7 +92,7 @@ def _ranges(chunk, seg_start, bias=None, batch=None):
     if seg_start is not None:
         seg = np.ascontiguousarray(seg_start, dtype=np.int32)
         r.seg_start = seg.ctypes.data_as(ctypes.POINTER(ctypes.c_int32))
-    return ctypes.pointer(r), (r, seg, bias)
+    return ctypes.pointer(r), (r, seg, bias, appended)
 
 _i32 = ctypes.c_int32
 
@@ -201,8 +216,19 @@ def rope_table(theta: float, seq_len: int, head_dim: int):
 # attention
 # --------------------------------------------------------------------------
 @dataclass
+class Cache:
+    """``Cache`` of tk/src/ops/attention.rs:39-56: k and v are ``[rows, Tk, H_all, D]`` caches."""
+
+    head_start: int
+    kv_heads: int
+    row_map: Optional[np.ndarray] = None   # [B] cache row a batch lane
+    appended: Optional[tuple] = None       # (k_app, v_app), each [B, n, kv_heads, D]
+    app_lens: Optional[np.ndarray] = None  # [B] visible appended rows
+
+
+@dataclass
 class AttnProblem:
-    """q [B,T,H,D]; k, v [B,Tk,Hkv,D] float32 arrays (bf16-exact when ``bf16``)."""
+    """q [B,T,H,D]; k, v [B,Tk,Hkv,D] float32 arrays (bf16-exact when ``bf16``), or caches with ``cache``."""
 
     q: np.ndarray
     k: np.ndarray
@@ -216,11 +242,42 @@ class AttnProblem:
     bias: Optional[np.ndarray] = None  # [B or 1, H, T, Tk] float32 (stream-dtype-exact), added to the scaled scores
     scale: Optional[float] = None
     bf16: bool = True
+    cache: Optional[Cache] = None
+    appended: Optional[tuple] = None  # (k_app, v_app, seen or None) beside gathered k and v: what ``gathered`` leaves
 
     def dims(self):
         b, t, h, d = self.q.shape
         _, tk, hkv, _ = self.k.shape
         return b, t, tk, h, hkv, d
+
+    def gathered(self) -> "AttnProblem":
+        """The cache read out as the graph reads it (tk/src/ops/attention.rs:498-503): the head range
+        narrowed and the rows selected, k and v ``[B, Tk, kv_heads, D]``; appended rows kept beside them."""
+        c = self.cache
+        if c is None:
+            return self
+        rows = np.arange(self.q.shape[0]) if c.row_map is None else np.asarray(c.row_map, dtype=np.int64)
+        heads = slice(c.head_start, c.head_start + c.kv_heads)
+        k, v = (np.ascontiguousarray(x[rows][:, :, heads]) for x in (self.k, self.v))
+        app = None
+        if c.appended is not None:
+            seen = None if c.app_lens is None else np.minimum(np.asarray(c.app_lens, dtype=np.int64), c.appended[0].shape[1])
+            app = (c.appended[0], c.appended[1], seen)
+        return dataclasses.replace(self, k=k, v=v, cache=None, appended=app)
+
+    def concatenated(self) -> "AttnProblem":
+        """Appended rows joined to the keys they follow and their visibility, with the key lengths',
+        folded into one key mask (tk/src/ops/attention.rs:507-531)."""
+        p = self.gathered()
+        if p.appended is None:
+            return p
+        k_app, v_app, seen = p.appended
+        b, tk, n = p.k.shape[0], p.k.shape[1], k_app.shape[1]
+        lens = np.full(b, tk) if p.key_lens is None else np.minimum(np.asarray(p.key_lens, dtype=np.int64), tk)
+        seen = np.full(b, n) if seen is None else seen
+        mask = np.concatenate([np.arange(tk)[None, :] < lens[:, None], np.arange(n)[None, :] < seen[:, None]], axis=1)
+        return dataclasses.replace(p, k=np.concatenate([p.k, k_app], axis=1), v=np.concatenate([p.v, v_app], axis=1),
+                                   key_lens=None, key_mask=mask, appended=None)
 
     def scale_f32(self) -> float:
         d = self.q.shape[-1]
@@ -232,9 +289,12 @@ class AttnProblem:
         lens = None if self.key_lens is None else np.ascontiguousarray(self.key_lens, dtype=np.int32)
         mask = None if self.key_mask is None else np.ascontiguousarray(np.asarray(self.key_mask) != 0, dtype=np.int32)
         wl, wr = (-1, -1) if self.window is None else self.window
-        if self.bias is not None and tuple(self.bias.shape[1:]) != (h, t, tk):
-            raise ValueError(f"bias has shape {self.bias.shape}, expected [{b} | 1, {h}, {t}, {tk}]")
-        ranges, alive = _ranges(self.chunk, self.seg_start, self.bias, b)
+        if self.cache is not None:
+            raise ValueError("a cached problem is gathered() first")
+        keys = tk + (0 if self.appended is None else self.appended[0].shape[1])
+        if self.bias is not None and tuple(self.bias.shape[1:]) != (h, t, keys):
+            raise ValueError(f"bias has shape {self.bias.shape}, expected [{b} | 1, {h}, {t}, {keys}]")
+        ranges, alive = _ranges(self.chunk, self.seg_start, self.bias, b, self.appended)
         keep = (lens, mask, alive)
         args = [b, t, tk, h, hkv, d, int(self.causal), wl, wr, ctypes.c_float(self.scale_f32()),
                 _ptr(lens, _i32p), _ptr(mask, _i32p), tk, ranges]
@@ -243,6 +303,7 @@ class AttnProblem:
 
 def attention_direct(p: AttnProblem, threads: int = 8) -> np.ndarray:
     """f64 direct softmax (tk/src/test/unit/attention.rs:102-178); unrounded float64 [B,T,H,D]."""
+    p = p.concatenated()
     q, k, v = _f32(p.q), _f32(p.k), _f32(p.v)
     out = np.empty(q.shape, dtype=np.float64)
     args, _keep = p._common()
@@ -254,6 +315,7 @@ def attention_direct(p: AttnProblem, threads: int = 8) -> np.ndarray:
 
 def attention_graph(p: AttnProblem, threads: int = 8) -> np.ndarray:
     """The op's graph fallback (tk/src/ops/attention.rs:496-584); float32 [B,T,H,D]."""
+    p = p.concatenated()
     q, k, v = _f32(p.q), _f32(p.k), _f32(p.v)
     out = np.empty(q.shape, dtype=np.float32)
     args, _keep = p._common()
@@ -265,7 +327,11 @@ def attention_graph(p: AttnProblem, threads: int = 8) -> np.ndarray:
 
 def attention_flash(p: AttnProblem, bq: int = 64, bkv: int = 64, threads: int = 8, splits: int = 1) -> np.ndarray:
     """The tile program under the host interpreter (tk/src/kernels/attention.rs:381-450,466-924);
-    with ``splits > 1`` its keys split and the partial states merged (L609-612, L899-921, L948-1014)."""
+    with ``splits > 1`` its keys split and the partial states merged (L609-612, L899-921, L948-1014).
+    Appended rows are the last split's last step (L827-846)."""
+    p = p.gathered()
+    if p.appended is not None and p.appended[0].shape[1] > bkv:
+        raise ValueError("the appended rows ride one key block")  # L475
     q, k, v = _f32(p.q), _f32(p.k), _f32(p.v)
     out = np.zeros(q.shape, dtype=np.float32)
     args, _keep = p._common()

@@ -33,6 +33,11 @@
  *       (and the masks as -inf) as its attn_mask, and by closed forms
  *       (a constant row changes nothing; -inf walls are a key mask; zero
  *       queries give softmax(bias) . v).
+ *       A cache is a gather plus a concatenation done by the Python layer
+ *       (as the reference's graph does it, tk/src/ops/attention.rs:498-531),
+ *       pinned by an independent numpy evaluation; the tile program's
+ *       appended step is held to the direct softmax within the reference's
+ *       tolerance.
  *   svod_oracle_attention_graph, svod_oracle_attention_flash
  *       pinned against svod_oracle_attention_direct within the tolerances the
  *       reference holds itself to (tk/src/test/unit/attention.rs:483,
@@ -188,8 +193,15 @@ typedef struct {
   int32_t chunk_has_left; /* Chunk::left is Some */
   int32_t chunk_left, chunk_right;
   const int32_t *seg_start; /* [batch, t] or NULL */
-  const float *bias;        /* [batch or 1, heads, t, tk] stream-dtype-exact values, or NULL */
+  const float *bias;        /* [batch or 1, heads, t, bias_cols] stream-dtype-exact values, or NULL */
   int32_t bias_per_batch;   /* Bias::PerBatch (1) or Bias::Shared (0) */
+  int32_t bias_cols;        /* the bias's last dim: tk, plus the appended rows (0 = tk) */
+  /* Cache::appended (tk/src/ops/attention.rs:48-55), the tile program only: rows scored after
+   * the tk keys of k and v, as the last split's last step (tk/src/kernels/attention.rs:739-755,
+   * 827-846).  The cache's row map and head range are a gather the caller has already done. */
+  int32_t appended;         /* rows a batch lane, 0 = none */
+  const float *k_app, *v_app; /* [batch, appended, kv_heads, d] */
+  const int32_t *app_seen;  /* [batch] visible appended rows, or NULL: all of them */
 } svod_oracle_extras;
 
 typedef struct {
@@ -244,7 +256,7 @@ static inline int hidden(const attn_problem *p, int32_t b, int32_t i, int32_t j)
 static inline float bias_at(const attn_problem *p, int32_t b, int32_t h, int32_t i, int32_t j) {
   if (!p->ranges || !p->ranges->bias) return 0.0f;
   const int64_t row = ((int64_t)(p->ranges->bias_per_batch ? b : 0) * p->heads + h) * p->t + i;
-  return p->ranges->bias[row * p->tk + j];
+  return p->ranges->bias[row * (p->ranges->bias_cols > 0 ? p->ranges->bias_cols : p->tk) + j];
 }
 
 /* Visibility of every (b, i, j): out[b][i][j] = 1 where key j is seen by query i. */
@@ -566,29 +578,39 @@ static void flash_slice(const void *ctxp, int32_t b, int32_t h) {
       l[r] = 0.0;
       for (int32_t dd = 0; dd < d; dd++) o[(int64_t)r * d + dd] = 0.0;
     }
-    for (int32_t blk = s_first; blk < s_end; blk++) {
-      const int32_t k0 = blk * bkv;
+    /* L827-846: the appended rows are one more block, which every split scores and all but the
+     * last hide; a hidden block leaves (m, l, o) as they were, so only the last split runs it. */
+    const int32_t app_rows = (rg && rg->appended > 0 && split == splits - 1) ? rg->appended : 0;
+    int32_t app_seen = app_rows;
+    if (app_rows > 0 && rg->app_seen && rg->app_seen[b] < app_seen) app_seen = rg->app_seen[b];
+    for (int32_t blk = s_first; blk < s_end + (app_rows > 0 ? 1 : 0); blk++) {
+      const int is_app = blk == s_end;
+      const int32_t k0 = is_app ? tk : blk * bkv; /* the appended keys' columns come last (L84-85) */
+      const float *k_src = is_app ? rg->k_app + (int64_t)b * app_rows * kv_stride : c->k + (int64_t)b * tk * kv_stride;
+      const float *v_src = is_app ? rg->v_app + (int64_t)b * app_rows * kv_stride : c->v + (int64_t)b * tk * kv_stride;
+      const int32_t k_rows = is_app ? app_rows : tk; /* the view's bound */
       /* s = q . k^T, rows past t and keys past the view's bound read as zero. */
       for (int32_t r = 0; r < bq; r++) {
         const int32_t i = q_off + r;
         for (int32_t cc = 0; cc < bkv; cc++) {
-          const int32_t j = k0 + cc;
+          const int32_t j = k0 + cc, jr = j - (is_app ? tk : 0);
           double dot = 0.0;
-          const int in_k = keys_masked ? (j < len) : 1;
-          if (i < t && in_k && j < tk) {
+          const int in_k = is_app ? 1 : (keys_masked ? (j < len) : 1);
+          if (i < t && in_k && jr < k_rows) {
             const float *qi = c->q + ((int64_t)b * t + i) * stride + (int64_t)h * d;
-            const float *kj = c->k + ((int64_t)b * tk + j) * kv_stride + (int64_t)kv_head * d;
+            const float *kj = k_src + (int64_t)jr * kv_stride + (int64_t)kv_head * d;
             for (int32_t dd = 0; dd < d; dd++) dot += (double)qi[dd] * (double)kj[dd];
           }
           double sv = r32(0.0f + (float)dot);
           sv = r32(sv * scale_log2e);
           /* biased() of L358-362: one fused multiply-add of the bias by log2(e) onto the scaled score. */
-          if (p->ranges && p->ranges->bias && i < t && j < tk)
+          if (p->ranges && p->ranges->bias && i < t && jr < k_rows)
             sv = (double)fmaf(bias_at(p, b, h, i, j), 1.44269504088896340736f, (float)sv);
           /* L641-697: a hidden score is -inf.  Applying the predicate on every
            * block equals applying it on edge blocks only (L698-733): on an
-           * interior block every key is kept. */
-          if (j >= tk || hidden(p, b, i, j)) sv = -INFINITY;
+           * interior block every key is kept.  An appended row is hidden past the
+           * visible count and by nothing else (L832-841). */
+          if (is_app ? (cc >= app_seen) : (j >= tk || hidden(p, b, i, j))) sv = -INFINITY;
           s[(int64_t)r * bkv + cc] = sv;
         }
       }
@@ -617,12 +639,12 @@ static void flash_slice(const void *ctxp, int32_t b, int32_t h) {
         for (int32_t dd = 0; dd < d; dd++) {
           double dot = 0.0;
           for (int32_t cc = 0; cc < bkv; cc++) {
-            const int32_t j = k0 + cc;
-            const int in_k = keys_masked ? (j < len) : 1;
-            if (!in_k || j >= tk) continue;
+            const int32_t j = k0 + cc, jr = j - (is_app ? tk : 0);
+            const int in_k = is_app ? 1 : (keys_masked ? (j < len) : 1);
+            if (!in_k || jr >= k_rows) continue;
             const double pv = p16[(int64_t)r * bkv + cc];
             if (pv == 0.0) continue;
-            dot += pv * (double)c->v[((int64_t)b * tk + j) * kv_stride + (int64_t)kv_head * d + dd];
+            dot += pv * (double)v_src[(int64_t)jr * kv_stride + (int64_t)kv_head * d + dd];
           }
           o[(int64_t)r * d + dd] = (double)((float)o[(int64_t)r * d + dd] + (float)dot);
         }

@@ -9,6 +9,7 @@ only.
 """
 from .ops import (  # noqa: F401
     Attn,
+    Cache,
     Fallback,
     GraphFallback,
     KeyMask,

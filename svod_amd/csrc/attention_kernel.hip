@@ -215,15 +215,15 @@ struct Wave {
 // the barrier that ends a step).  m0 carries the LDS address of a wave instruction's 1 KiB.
 template <int D, int NW, bool F16, unsigned FLAGS>
 __device__ __forceinline__ void fill_tile(const Wave<D, NW, F16, FLAGS> &w, const uint8_t *base, int64_t bytes, int blk,
-                                          int lds_at, int src) {
+                                          int lds_at, int src, int row_bytes) {
   // This wave's fills of a tile are NW instructions apart; the swizzle repeats with that period,
   // so they share the lanes' offsets and differ in the descriptor's base.
   constexpr int kRowsPer = 64 / Tile<D>::kCpr;  // rows a wave instruction covers
   static_assert((NW * kRowsPer) % 16 == 0, "the swizzle repeats from one of a wave's fills to its next");
-  const int64_t off = (int64_t)blk * kBkv * w.kv_row_bytes;
+  const int64_t off = (int64_t)blk * kBkv * row_bytes;
 #pragma unroll
   for (int i = 0; i < Wave<D, NW, F16, FLAGS>::CH; i++) {
-    const int64_t at = off + (int64_t)(NW * i * kRowsPer) * w.kv_row_bytes;
+    const int64_t at = off + (int64_t)(NW * i * kRowsPer) * row_bytes;
     const i32x4 r = make_rsrc(base + at, bytes - at);
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
                  :
@@ -237,17 +237,17 @@ template <int D, int NW, bool F16, unsigned FLAGS>
 __device__ __forceinline__ void fill_k(const Wave<D, NW, F16, FLAGS> &w, int n, int slot) {
   const int at = w.lds0 + slot * Tile<D>::kBytes;
   if (n < w.end)
-    fill_tile<D, NW>(w, w.k_base, w.kv_bytes, n, at, w.k_src);
+    fill_tile<D, NW>(w, w.k_base, w.kv_bytes, n, at, w.k_src, w.kv_row_bytes);
   else if ((FLAGS & kStream) && n >= w.end_even && n - w.end_even < w.nxt_end)
-    fill_tile<D, NW>(w, w.nxt_k, w.nxt_bytes, n - w.end_even, at, w.k_src);
+    fill_tile<D, NW>(w, w.nxt_k, w.nxt_bytes, n - w.end_even, at, w.k_src, w.kv_row_bytes);
 }
 template <int D, int NW, bool F16, unsigned FLAGS>
 __device__ __forceinline__ void fill_v(const Wave<D, NW, F16, FLAGS> &w, int n, int slot) {
   const int at = w.lds0 + (2 + slot) * Tile<D>::kBytes;
   if (n < w.end)
-    fill_tile<D, NW>(w, w.v_base, w.kv_bytes, n, at, w.v_src);
+    fill_tile<D, NW>(w, w.v_base, w.kv_bytes, n, at, w.v_src, w.kv_row_bytes);
   else if ((FLAGS & kStream) && n >= w.end_even && n - w.end_even < w.nxt_end)
-    fill_tile<D, NW>(w, w.nxt_v, w.nxt_bytes, n - w.end_even, at, w.v_src);
+    fill_tile<D, NW>(w, w.nxt_v, w.nxt_bytes, n - w.end_even, at, w.v_src, w.kv_row_bytes);
 }
 
 // A key mask row is read 64 keys (one per lane) a block, one block ahead: the load is issued
@@ -293,11 +293,11 @@ __device__ __forceinline__ uint64_t uniform_bits(const Wave<D, NW, F16, FLAGS> &
   return kbits;
 }
 
-// The 32 bias elements this lane's scores of block `blk` take, as 16 packed pairs: keys
-// k0 + 32 kb + 8 c + 4 g + {0..3}.  Keys past the row read as zero (their scores are hidden anyway).
+// The 32 bias elements this lane's scores of the 64 keys from `first` on take, as 16 packed
+// pairs: keys first + 32 kb + 8 c + 4 g + {0..3}.  Keys past the row read as zero (their scores are hidden anyway).
 template <int D, int NW, bool F16, unsigned FLAGS>
-__device__ __forceinline__ void load_bias(const Wave<D, NW, F16, FLAGS> &w, int blk, bool row_ok, uint32_t (&bw)[16]) {
-  const int k0 = blk * kBkv + 4 * w.g;
+__device__ __forceinline__ void load_bias(const Wave<D, NW, F16, FLAGS> &w, int first, bool row_ok, uint32_t (&bw)[16]) {
+  const int k0 = first + 4 * w.g;
   const bool aligned = ((uintptr_t)w.bias_row & 7u) == 0;  // wave-uniform when every row is: checked per lane
 #pragma unroll
   for (int c = 0; c < 8; c++) {
@@ -348,6 +348,18 @@ __device__ __forceinline__ bool on_edge(const Wave<D, NW, F16, FLAGS> &w, int bl
   return CAUSAL && (k0 + kBkv - 1 > w.wave_first_row);
 }
 
+// Scores whose bit of `mine` is clear become -inf; bit 8 (i / 4) + i % 4 (+ 32 for the second
+// half) is this lane's score i: the key that many places past the lane's first.
+__device__ __forceinline__ void hide_scores(uint64_t mine, float (&sv)[32]) {
+  const uint32_t lo = (uint32_t)mine, hi = (uint32_t)(mine >> 32);
+#pragma unroll
+  for (int i = 0; i < 16; i++) {
+    const int rel = 8 * (i / 4) + (i % 4);  // key k0 + 32kb + 4g + rel
+    sv[i] = ((lo >> rel) & 1u) ? sv[i] : -INFINITY;
+    sv[16 + i] = ((hi >> rel) & 1u) ? sv[16 + i] : -INFINITY;
+  }
+}
+
 // Scales (a non-positive scale only) and masks (L641-697) the scores of block `blk`: hidden
 // scores become -inf.  `kbits` is the uniform word; causality adds a per-lane one.
 template <int D, int NW, bool CAUSAL, bool F16, unsigned FLAGS>
@@ -364,14 +376,7 @@ __device__ __forceinline__ void mask_scores(const Wave<D, NW, F16, FLAGS> &w, in
     const int seen = w.my_row - k0 + 1;  // keys k0 .. my_row are seen
     mine &= seen >= 64 ? ~0ull : (seen <= 0 ? 0ull : (~0ull >> (64 - seen)));
   }
-  mine >>= 4 * w.g;
-  const uint32_t lo = (uint32_t)mine, hi = (uint32_t)(mine >> 32);
-#pragma unroll
-  for (int i = 0; i < 16; i++) {
-    const int rel = 8 * (i / 4) + (i % 4);  // key k0 + 32kb + 4g + rel
-    sv[i] = ((lo >> rel) & 1u) ? sv[i] : -INFINITY;
-    sv[16 + i] = ((hi >> rel) & 1u) ? sv[16 + i] : -INFINITY;
-  }
+  hide_scores(mine >> (4 * w.g), sv);
 }
 
 // The row maximum of a block's scores: in-lane tree of three-way folds, then the other
@@ -579,7 +584,7 @@ __device__ __forceinline__ void edge_step(Wave<D, NW, F16, FLAGS> &w, const uint
   const uint64_t kbits_next = uniform_bits<D, NW>(w, blk + 1, w.mask_next);
   // The next block's bias is asked for first: it has this block's P.V to arrive under.
   uint32_t bw[16];
-  if (w.biased && more) load_bias<D, NW>(w, blk + 1, w.my_row_ok, bw);
+  if (w.biased && more) load_bias<D, NW>(w, (blk + 1) * kBkv, w.my_row_ok, bw);
   fill_v<D, NW>(w, blk + 1, par ^ 1);
   if (blk + 2 < w.end) w.mask_next = mask_lane<D, NW>(w, blk + 2);
   fill_k<D, NW>(w, blk + 2, par);
@@ -649,11 +654,20 @@ struct Ranges {
   int32_t chunk_right;          // the host caps it at the chunks of the keys
   const void *seg_start;        // [B, T] integers or null
   int32_t seg_i64;
-  const uint16_t *bias;         // [B or 1, H, T, Tk] of the operands' type, or null
+  const uint16_t *bias;         // [B or 1, H, T, bias_cols] of the operands' type, or null
   int32_t bias_per_batch;
+  int32_t bias_cols;            // Tk, plus the appended rows
+  // The cache of a launch that has one (the CACHED instantiations; tk/src/ops/attention.rs:39-56).
+  int32_t kv_head_start;        // the first of the launch's kv heads in a cache row
+  const void *row_map;          // [B] cache row per batch lane, or null: row b
+  int32_t row_map_i64;
+  const uint16_t *k_app, *v_app;  // [B, app_rows, kv_heads, D] scored after the cached keys, or null
+  int32_t app_rows;             // at most a key block
+  const void *app_lens;         // [B] visible appended rows, or null: all
+  int32_t app_lens_i64;
 };
 
-template <int D, int NW, bool CAUSAL, bool SPLIT, bool RANGED, bool BIASED, bool F16>
+template <int D, int NW, bool CAUSAL, bool SPLIT, bool RANGED, bool BIASED, bool CACHED, bool F16>
 __global__ __launch_bounds__(NW * 64, (D == 64 && !BIASED) ? 3 : 2) void flash_fwd_kernel(
     uint32_t unit_size, uint32_t unit_rcp, uint32_t nqt_u, uint32_t nqt_rcp, uint32_t kvh_u, uint32_t kvh_rcp,
     uint32_t units, uint32_t heads_group, const void *__restrict__ key_lens, const uint16_t *__restrict__ q, int32_t t,
@@ -801,8 +815,8 @@ __global__ __launch_bounds__(NW * 64, (D == 64 && !BIASED) ? 3 : 2) void flash_f
   if (BIASED) {
     // L566-571: the bias of this (batch or 0, head), this lane's row, from the tile's first key on.
     const int64_t brow = ((int64_t)(rg.bias_per_batch ? b : 0) * heads + h) * t + min(row, t - 1);
-    w.bias_row = rg.bias + brow * tk + first_key;
-    w.bias_keys = tk - first_key;
+    w.bias_row = rg.bias + brow * rg.bias_cols + first_key;
+    w.bias_keys = rg.bias_cols - first_key;
   }
   if (RANGED) {
     w.row_lo -= first_key;
@@ -813,8 +827,16 @@ __global__ __launch_bounds__(NW * 64, (D == 64 && !BIASED) ? 3 : 2) void flash_f
   }
 
   w.kv_row_bytes = kv_row_elems * 2;
-  w.k_base = (const uint8_t *)(k + ((int64_t)b * tk + first_key) * kv_row_elems + (int64_t)kvh * D);
-  w.v_base = (const uint8_t *)(v + ((int64_t)b * tk + first_key) * kv_row_elems + (int64_t)kvh * D);
+  // L544-550: a cache is read at the batch lane's row of it, from the launch's first head on.
+  int64_t kv_row = b;
+  int kv_col = kvh;
+  if (CACHED) {
+    if (rg.row_map != nullptr)
+      kv_row = rg.row_map_i64 ? ((const long long *)rg.row_map)[b] : (long long)((const int *)rg.row_map)[b];
+    kv_col += rg.kv_head_start;
+  }
+  w.k_base = (const uint8_t *)(k + (kv_row * tk + first_key) * kv_row_elems + (int64_t)kv_col * D);
+  w.v_base = (const uint8_t *)(v + (kv_row * tk + first_key) * kv_row_elems + (int64_t)kv_col * D);
   w.kv_bytes = len > 0 ? (int64_t)(len - 1) * w.kv_row_bytes + D * 2 : 0;
   w.lds0 = (int)(uintptr_t)(LDS_PTR(uint8_t))(smem);
 
@@ -924,6 +946,53 @@ __global__ __launch_bounds__(NW * 64, (D == 64 && !BIASED) ? 3 : 2) void flash_f
   }
   for (; blk < my_end; blk++) edge_step<D, NW, CAUSAL>(w, smem, blk, my_end, sv, bm);
   for (; blk < end; blk++) idle_step<D, NW>(w, blk);
+
+  // ---- the appended rows (L739-755, L827-846): one more block of keys, from their own tensors,
+  // which only the last split scores; the first `seen` of them are visible and no other mask
+  // reaches them.  Every wave is past the last step's barrier, so the ring is free.
+  if (CACHED) {
+    if (rg.k_app != nullptr && (!SPLIT || split == (int)sp.count - 1)) {
+      int seen = rg.app_rows;
+      if (rg.app_lens != nullptr) {
+        const long long n = rg.app_lens_i64 ? ((const long long *)rg.app_lens)[b] : (long long)((const int *)rg.app_lens)[b];
+        seen = (int)(n < 0 ? 0 : (n < seen ? n : seen));
+      }
+      const int app_row_bytes = (int)geo.kv_heads * D * 2;
+      const int64_t at = ((int64_t)b * rg.app_rows * geo.kv_heads + kvh) * D;
+      const int64_t bytes = seen > 0 ? (int64_t)(seen - 1) * app_row_bytes + D * 2 : 0;  // hidden rows read as zeros
+      {
+        const int frow = w.wave * kRowsPer + w.lane / TL::kCpr;
+        const int pc = w.lane % TL::kCpr;
+        const int k_src = frow * app_row_bytes + ((pc ^ TL::swz_k(frow)) << 4);
+        const int v_src = frow * app_row_bytes + ((pc ^ (TL::swz_v(frow) << 2)) << 4);
+        fill_tile<D, NW>(w, (const uint8_t *)(rg.k_app + at), bytes, 0, w.lds0, k_src, app_row_bytes);
+        fill_tile<D, NW>(w, (const uint8_t *)(rg.v_app + at), bytes, 0, w.lds0 + 2 * TL::kBytes, v_src, app_row_bytes);
+      }
+      uint32_t bw[16];
+      if (BIASED) load_bias<D, NW>(w, tk - first_key, row < t, bw);  // their columns come last (L84-85)
+      __builtin_amdgcn_s_waitcnt(0x0f70);
+      __syncthreads();
+      scores<D, NW>(w, smem, 0, sv);
+      if (!w.positive) {
+#pragma unroll
+        for (int i = 0; i < 32; i++) sv[i] *= w.c_exp;
+      }
+      if (BIASED) add_bias<F16>(bw, sv);
+      const uint64_t visible = seen >= 64 ? ~0ull : ((1ull << seen) - 1);
+      if (visible != ~0ull) hide_scores(visible >> (4 * w.g), sv);
+      bm = row_max(sv);
+      float corr;
+      const float m_exp = adopt_maximum<D, NW>(w, bm, corr);
+      const uint8_t *vs_ = smem + 2 * TL::kBytes;
+      float bs[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+      uint32_t pk[16];
+      probabilities<F16>(sv, w.unit, m_exp, bs, pk);
+      probabilities<F16>(sv + 16, w.unit, m_exp, bs, pk + 8);
+      accumulate<D, NW>(w, vs_, 0, pk);
+      accumulate<D, NW>(w, vs_, 1, pk + 8);
+      w.l_run = w.l_run * corr + ((bs[0] + bs[1]) + (bs[2] + bs[3]));
+    }
+  }
 
   const Pair lp = both_halves(w.l_run);
   const float l_tot = lp.a + lp.b;
@@ -1307,7 +1376,7 @@ hipError_t launch_stream(const AttnArgs &a, hipStream_t stream, int64_t slots, c
   return hipGetLastError();
 }
 
-template <int D, int NW, bool CAUSAL, bool SPLIT, bool RANGED, bool BIASED, bool F16>
+template <int D, int NW, bool CAUSAL, bool SPLIT, bool RANGED, bool BIASED, bool CACHED, bool F16>
 hipError_t launch(const AttnArgs &a, hipStream_t stream) {
   using TL = Tile<D>;
   constexpr int BQ = NW * kWaveRows;
@@ -1321,7 +1390,7 @@ hipError_t launch(const AttnArgs &a, hipStream_t stream) {
   const int64_t kv_row = a.kv_row_elems > 0 ? a.kv_row_elems : (int64_t)a.kv_heads * a.d;
   // The fills address a (batch, kv head)'s rows with 32-bit byte offsets.
   if ((int64_t)a.tk * kv_row * 2 > 0x7fffffffLL || q_row > 0x7fffffffLL) return hipErrorInvalidValue;
-  auto kernel = flash_fwd_kernel<D, NW, CAUSAL, SPLIT, RANGED, BIASED, F16>;
+  auto kernel = flash_fwd_kernel<D, NW, CAUSAL, SPLIT, RANGED, BIASED, CACHED, F16>;
   // The LDS ring is above the default limit of a launch: one attribute call per instantiation
   // and device, from whichever thread gets there first (a second call is harmless).
   static std::atomic<uint64_t> configured{0};  // a bit per device ordinal, devices past 63 always ask
@@ -1354,7 +1423,7 @@ hipError_t launch(const AttnArgs &a, hipStream_t stream) {
   // The streaming form, where asked for and where it has a kernel (head size 64, lengths or no
   // key mask, no window, no splits): `knob` workgroups per XCD, each walking its run of tiles.
   // It is never chosen unasked: measured, it has not beaten a workgroup per tile.
-  if constexpr (D == 64 && !SPLIT && !RANGED && !BIASED) {
+  if constexpr (D == 64 && !SPLIT && !RANGED && !BIASED && !CACHED) {
     const int knob = g_stream_slots.load(std::memory_order_relaxed);
     if (knob > 0 && a.key_mask == nullptr)
       return launch_stream<D, NW, CAUSAL, F16>(a, stream, knob, geo, q_row, kv_row);
@@ -1379,6 +1448,15 @@ hipError_t launch(const AttnArgs &a, hipStream_t stream) {
   rg.seg_i64 = a.seg_i64;
   rg.bias = (const uint16_t *)a.bias;
   rg.bias_per_batch = a.bias_per_batch;
+  rg.bias_cols = a.tk + a.app_rows;
+  rg.kv_head_start = a.kv_head_start;
+  rg.row_map = a.row_map;
+  rg.row_map_i64 = a.row_map_i64;
+  rg.k_app = (const uint16_t *)a.k_app;
+  rg.v_app = (const uint16_t *)a.v_app;
+  rg.app_rows = a.app_rows;
+  rg.app_lens = a.app_lens;
+  rg.app_lens_i64 = a.app_lens_i64;
   hipLaunchKernelGGL(kernel, dim3((uint32_t)grid), dim3(NW * 64), smem, stream, geo.unit_size, geo.unit_rcp, geo.nqt,
                      geo.nqt_rcp, geo.kv_heads, geo.kvh_rcp, geo.units, heads_group, a.key_lens,
                      (const uint16_t *)a.q, a.t, tk_lens64, (const uint16_t *)a.k,
@@ -1387,22 +1465,26 @@ hipError_t launch(const AttnArgs &a, hipStream_t stream) {
   return hipGetLastError();
 }
 
-template <int D, bool RANGED, bool BIASED, bool F16>
+template <int D, bool RANGED, bool BIASED, bool CACHED, bool F16>
 hipError_t launch_s(const AttnArgs &a, hipStream_t stream) {
   if (a.splits > 1)
-    return a.causal ? launch<D, 4, true, true, RANGED, BIASED, F16>(a, stream)
-                    : launch<D, 4, false, true, RANGED, BIASED, F16>(a, stream);
-  return a.causal ? launch<D, 4, true, false, RANGED, BIASED, F16>(a, stream)
-                  : launch<D, 4, false, false, RANGED, BIASED, F16>(a, stream);
+    return a.causal ? launch<D, 4, true, true, RANGED, BIASED, CACHED, F16>(a, stream)
+                    : launch<D, 4, false, true, RANGED, BIASED, CACHED, F16>(a, stream);
+  return a.causal ? launch<D, 4, true, false, RANGED, BIASED, CACHED, F16>(a, stream)
+                  : launch<D, 4, false, false, RANGED, BIASED, CACHED, F16>(a, stream);
 }
 
 template <int D, bool F16>
 hipError_t launch_t(const AttnArgs &a, hipStream_t stream) {
   // A window, a chunk mask or segment starts: the instantiations with per-row key ranges.
   const bool ranged = a.win_left >= 0 || a.chunk_size > 0 || a.seg_start != nullptr;
-  if (a.bias != nullptr)
-    return ranged ? launch_s<D, true, true, F16>(a, stream) : launch_s<D, false, true, F16>(a, stream);
-  return ranged ? launch_s<D, true, false, F16>(a, stream) : launch_s<D, false, false, F16>(a, stream);
+  const bool biased = a.bias != nullptr;
+  if (a.cached) {
+    if (ranged) return hipErrorInvalidValue;  // not instantiated: the op layer keeps the graph
+    return biased ? launch_s<D, false, true, true, F16>(a, stream) : launch_s<D, false, false, true, F16>(a, stream);
+  }
+  if (biased) return ranged ? launch_s<D, true, true, false, F16>(a, stream) : launch_s<D, false, true, false, F16>(a, stream);
+  return ranged ? launch_s<D, true, false, false, F16>(a, stream) : launch_s<D, false, false, false, F16>(a, stream);
 }
 
 template <int D>

@@ -63,6 +63,18 @@ struct AttnArgs {
   // rows unpadded, added to the scaled scores before the masks.  Null = none.
   const void *bias;
   int32_t bias_per_batch;
+  // Cache (tk/src/ops/attention.rs:39-56).  kv_head_start: the first of this attention's kv_heads
+  // in a cache row of kv_row_elems / d heads.  row_map: [batch] i32 or i64 cache row per batch
+  // lane, null = row b.  k_app / v_app: [batch, app_rows, kv_heads, d] scored after the tk cached
+  // keys, the first app_lens[b] of them visible (all without app_lens); app_rows <= 64.
+  int32_t cached;
+  int32_t kv_head_start;
+  const void *row_map;
+  int32_t row_map_i64;
+  const void *k_app, *v_app;
+  int32_t app_rows;
+  const void *app_lens;
+  int32_t app_lens_i64;
 };
 hipError_t launch_attention(const AttnArgs &a, hipStream_t stream);
 

@@ -257,12 +257,17 @@ static int attend(const svodk_tensor *q, const svodk_tensor *k, const svodk_tens
   // L131: q is [B, T, H, D].
   if (q->rank != 4)
     return fail(SVODK_ERR_SHAPE, "%s: q has shape %s, expected [B, T, H, D]", op, fmt_shape(q).c_str());
-  // L136-138: k is [B, Tk, H_kv, D]; v has k's shape.  (A cache with a row map
-  // relaxes the batch; a cache never takes a kernel here, but the check stands.)
-  const bool batch_fits = k->rank == 4 && (k->shape[0] == q->shape[0] || opts->has_cache);
-  if (!(k->rank == 4 && batch_fits && k->shape[3] == q->shape[3]))
+  // L132-138: k is [B, Tk, H_kv, D] ([rows, ...] under a cache's row map); v has k's shape.
+  const svodk_cache *cache = opts->cache;
+  const bool mapped = cache != nullptr && cache->row_map != nullptr;
+  const bool batch_fits = k->rank == 4 && (k->shape[0] == q->shape[0] || mapped);
+  if (!(k->rank == 4 && batch_fits && k->shape[3] == q->shape[3])) {
+    if (mapped)
+      return fail(SVODK_ERR_SHAPE, "%s: k has shape %s, expected [rows, Tk, H_kv, %lld]", op, fmt_shape(k).c_str(),
+                  (long long)q->shape[3]);
     return fail(SVODK_ERR_SHAPE, "%s: k has shape %s, expected [%lld, Tk, H_kv, %lld]", op, fmt_shape(k).c_str(),
                 (long long)q->shape[0], (long long)q->shape[3]);
+  }
   if (!same_shape(v, k))
     return fail(SVODK_ERR_SHAPE, "%s: v has shape %s, expected %s", op, fmt_shape(v).c_str(), fmt_shape(k).c_str());
   // L139-141: k and v share q's type.
@@ -271,10 +276,59 @@ static int attend(const svodk_tensor *q, const svodk_tensor *k, const svodk_tens
   if (v->dtype != q->dtype)
     return fail(SVODK_ERR_DTYPE, "%s: v is %s, the input is %s", op, dtype_name(v->dtype), dtype_name(q->dtype));
   // L142-145: whole groups of query heads per KV head.
-  const int64_t heads = q->shape[2], kv_heads = k->shape[2];
-  if (!opts->has_cache && !(kv_heads > 0 && heads % kv_heads == 0))
+  const int64_t heads = q->shape[2], kv_heads = cache ? cache->kv_heads : k->shape[2];
+  if (!(kv_heads > 0 && heads % kv_heads == 0))
     return fail(SVODK_ERR_HEADS, "%s: %lld query heads are not a multiple of %lld key/value heads", op,
                 (long long)heads, (long long)kv_heads);
+  // L146-170: the cache's head range lies in the row; its map, appended rows and their counts fit the batch.
+  int64_t appended = 0;
+  if (cache != nullptr) {
+    if (!(cache->head_start >= 0 && cache->head_start + cache->kv_heads <= k->shape[2]))
+      return fail(SVODK_ERR_SHAPE, "%s: k has shape %s, expected [rows, Tk, >= %lld, %lld]", op, fmt_shape(k).c_str(),
+                  (long long)(cache->head_start + cache->kv_heads), (long long)q->shape[3]);
+    if (cache->row_map != nullptr) {
+      if (!well_formed(cache->row_map)) return fail(SVODK_ERR_ARGUMENT, "%s: row map descriptor malformed", op);
+      if (!(cache->row_map->rank == 1 && cache->row_map->shape[0] == q->shape[0]))
+        return fail(SVODK_ERR_SHAPE, "%s: row map has shape %s, expected [%lld]", op,
+                    fmt_shape(cache->row_map).c_str(), (long long)q->shape[0]);
+      if (!is_int(cache->row_map->dtype))
+        return fail(SVODK_ERR_DTYPE, "%s: row map is %s, the input is an integer type", op,
+                    dtype_name(cache->row_map->dtype));
+    }
+    if ((cache->k_app != nullptr) != (cache->v_app != nullptr))
+      return fail(SVODK_ERR_ARGUMENT, "%s: appended keys and values come together", op);
+    if (cache->k_app != nullptr) {
+      const svodk_tensor *both[2] = {cache->k_app, cache->v_app};
+      const char *names[2] = {"appended k", "appended v"};
+      if (!well_formed(both[0]) || !well_formed(both[1]))
+        return fail(SVODK_ERR_ARGUMENT, "%s: appended rows descriptor malformed", op);
+      const int64_t rows = both[0]->rank == 4 && both[0]->shape[1] > 0 ? both[0]->shape[1] : 0;
+      for (int i = 0; i < 2; i++) {
+        const svodk_tensor *x = both[i];
+        const bool fits = rows > 0 && x->rank == 4 && x->shape[0] == q->shape[0] && x->shape[1] == rows &&
+                          x->shape[2] == kv_heads && x->shape[3] == q->shape[3];
+        if (!fits)
+          return fail(SVODK_ERR_SHAPE, "%s: %s has shape %s, expected [%lld, %lld, %lld, %lld]", op, names[i],
+                      fmt_shape(x).c_str(), (long long)q->shape[0], (long long)(rows > 0 ? rows : 1),
+                      (long long)kv_heads, (long long)q->shape[3]);
+        if (x->dtype != q->dtype)
+          return fail(SVODK_ERR_DTYPE, "%s: %s is %s, the input is %s", op, names[i], dtype_name(x->dtype),
+                      dtype_name(q->dtype));
+      }
+      if (opts->key_kind != SVODK_KEYS_LENS)
+        return fail(SVODK_ERR_SHAPE, "%s: key lens has shape [], expected [B] with appended rows", op);
+      appended = rows;
+    }
+    if (cache->app_lens != nullptr) {
+      if (!well_formed(cache->app_lens)) return fail(SVODK_ERR_ARGUMENT, "%s: appended lens descriptor malformed", op);
+      if (!(cache->k_app != nullptr && cache->app_lens->rank == 1 && cache->app_lens->shape[0] == q->shape[0]))
+        return fail(SVODK_ERR_SHAPE, "%s: appended lens has shape %s, expected [%lld] with appended rows", op,
+                    fmt_shape(cache->app_lens).c_str(), (long long)q->shape[0]);
+      if (!is_int(cache->app_lens->dtype))
+        return fail(SVODK_ERR_DTYPE, "%s: appended lens is %s, the input is an integer type", op,
+                    dtype_name(cache->app_lens->dtype));
+    }
+  }
   // L174-186: the key mask's shape.
   const svodk_tensor *lens = nullptr, *bools = nullptr;
   if (opts->key_kind == SVODK_KEYS_LENS) {
@@ -305,11 +359,11 @@ static int attend(const svodk_tensor *q, const svodk_tensor *k, const svodk_tens
     if (!well_formed(opts->bias)) return fail(SVODK_ERR_ARGUMENT, "%s: bias descriptor malformed", op);
     const svodk_tensor *bt = opts->bias;
     const bool fits = bt->rank == 4 && (bt->shape[0] == q->shape[0] || bt->shape[0] == 1) && bt->shape[1] == heads &&
-                      bt->shape[2] == q->shape[1] && bt->shape[3] == k->shape[1];
+                      bt->shape[2] == q->shape[1] && bt->shape[3] == k->shape[1] + appended;
     if (!fits)
       return fail(SVODK_ERR_SHAPE, "%s: bias has shape %s, expected [%lld | 1, %lld, %lld, %lld]", op,
                   fmt_shape(bt).c_str(), (long long)q->shape[0], (long long)heads, (long long)q->shape[1],
-                  (long long)k->shape[1]);
+                  (long long)(k->shape[1] + appended));
   }
   // The output the reference op allocates itself (tk/src/ops/mod.rs:423-429):
   // here the caller's, so its shape and type are checked like an operand's.
@@ -333,7 +387,11 @@ static int attend(const svodk_tensor *q, const svodk_tensor *k, const svodk_tens
   if (why != 0) return ran_graph(op, why);
   // Options the reference's kernel holds and this library's does not: no
   // config here holds them (the reference's own use of Fallback::Config, L210-214).
-  if (opts->has_cache) return ran_graph(op, SVODK_GRAPH_CONFIG);
+  // L209-214: no config holds more appended rows than a key block; and this library has no
+  // kernel for a cache under per-row key ranges.
+  if (appended > 64) return ran_graph(op, SVODK_GRAPH_CONFIG);
+  if (cache != nullptr && (opts->has_window || opts->has_chunk || opts->seg_start != nullptr))
+    return ran_graph(op, SVODK_GRAPH_CONFIG);
   if (opts->has_window && (opts->window_left < 0 || opts->window_right < 0))
     return fail(SVODK_ERR_ARGUMENT, "%s: a negative window reach", op);
   // Chunk { size, left, right } of tk/src/ops/attention.rs:39-50: usize fields, a size of at least 1.
@@ -412,6 +470,33 @@ static int attend(const svodk_tensor *q, const svodk_tensor *k, const svodk_tens
     a.seg_i64 = opts->seg_start->dtype == SVODK_I64;
   }
   if (packed != nullptr) a.q_row_elems = a.kv_row_elems = (heads + 2 * kv_heads) * d;
+  if (cache != nullptr) {
+    a.cached = 1;
+    a.kv_row_elems = k->shape[2] * d;  // a cache row holds every layer's heads
+    a.kv_head_start = (int32_t)cache->head_start;
+    if (cache->row_map != nullptr) {
+      if (cache->row_map->data == nullptr) return fail(SVODK_ERR_ARGUMENT, "%s: a null device pointer", op);
+      a.row_map = cache->row_map->data;
+      a.row_map_i64 = cache->row_map->dtype == SVODK_I64;
+    }
+    if (cache->k_app != nullptr) {
+      if (cache->k_app->data == nullptr || cache->v_app->data == nullptr ||
+          (cache->app_lens != nullptr && cache->app_lens->data == nullptr))
+        return fail(SVODK_ERR_ARGUMENT, "%s: a null device pointer", op);
+      const svodk_tensor *apps[2] = {cache->k_app, cache->v_app};
+      for (const svodk_tensor *x : apps) {
+        Span pair[2] = {{"appended rows", x->data, (size_t)numel(x) * 2, false}, spans[3]};
+        if (int rc = check_aliasing(op, pair, 2)) return rc;
+      }
+      a.k_app = cache->k_app->data;
+      a.v_app = cache->v_app->data;
+      a.app_rows = (int32_t)appended;
+      if (cache->app_lens != nullptr) {
+        a.app_lens = cache->app_lens->data;
+        a.app_lens_i64 = cache->app_lens->dtype == SVODK_I64;
+      }
+    }
+  }
   // L280-302: key splits.  The partial tensors live in the caller's workspace.
   a.splits = split_count(opts->splits, tk);
   if (a.splits > 1) {
@@ -467,7 +552,7 @@ int svodk_attention_packed(const svodk_tensor *qkv, int32_t heads, int32_t kv_he
   const int64_t slots = (int64_t)heads + 2 * kv_heads;
   if (!(qkv->rank == 3 && qkv->shape[2] > 0 && qkv->shape[2] % slots == 0))
     return fail(SVODK_ERR_SHAPE, "%s: qkv has shape %s, expected [B, T, slots·D]", op, fmt_shape(qkv).c_str());
-  if (opts->has_cache)
+  if (opts->cache != nullptr)
     return fail(SVODK_ERR_SHAPE, "%s: qkv has shape %s, expected [B, T, slots·D] with no cache", op,
                 fmt_shape(qkv).c_str());
   // L115-121: the three views of the fused row.

@@ -32,13 +32,19 @@ class _Tensor(ctypes.Structure):
                 ("shape", ctypes.c_int64 * 4)]
 
 
+class _Cache(ctypes.Structure):
+    _fields_ = [("head_start", ctypes.c_int64), ("kv_heads", ctypes.c_int64), ("row_map", ctypes.POINTER(_Tensor)),
+                ("k_app", ctypes.POINTER(_Tensor)), ("v_app", ctypes.POINTER(_Tensor)),
+                ("app_lens", ctypes.POINTER(_Tensor))]
+
+
 class _Attn(ctypes.Structure):
     _fields_ = [
         ("causal", ctypes.c_int32), ("key_kind", ctypes.c_int32), ("keys", ctypes.POINTER(_Tensor)),
         ("has_window", ctypes.c_int32), ("window_left", ctypes.c_int64), ("window_right", ctypes.c_int64),
         ("has_chunk", ctypes.c_int32), ("chunk_size", ctypes.c_int64), ("chunk_has_left", ctypes.c_int32),
         ("chunk_left", ctypes.c_int64), ("chunk_right", ctypes.c_int64),
-        ("seg_start", ctypes.POINTER(_Tensor)), ("has_cache", ctypes.c_int32), ("bias", ctypes.POINTER(_Tensor)),
+        ("seg_start", ctypes.POINTER(_Tensor)), ("cache", ctypes.POINTER(_Cache)), ("bias", ctypes.POINTER(_Tensor)),
         ("splits", ctypes.c_int32), ("has_scale", ctypes.c_int32), ("scale", ctypes.c_float),
         ("batch_live", ctypes.c_int32), ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_int64),
     ]
@@ -183,6 +189,17 @@ class KeyMask:
 
 
 @dataclass
+class Cache:
+    """``Cache`` of tk/src/ops/attention.rs:39-56: k and v are caches ``[rows, Tk, H_all, D]``."""
+
+    head_start: int
+    kv_heads: int
+    row_map: Optional[torch.Tensor] = None
+    appended: Optional[Tuple[torch.Tensor, torch.Tensor]] = None
+    app_lens: Optional[torch.Tensor] = None
+
+
+@dataclass
 class Attn:
     """``Attn`` of tk/src/ops/attention.rs:60-86.  ``batch_live`` stands for a bound
     batch variable (``Batch::Var``): only the first ``batch_live`` batches run."""
@@ -192,7 +209,7 @@ class Attn:
     window: Optional[Tuple[int, int]] = None
     chunk: Optional[Tuple[int, Optional[int], int]] = None  # (size, left, right)
     seg_start: Optional[torch.Tensor] = None
-    cache: bool = False
+    cache: Optional["Cache"] = None
     splits: Optional[int] = None
     scale: Optional[float] = None
     bias: Optional[torch.Tensor] = None
@@ -225,7 +242,15 @@ def _attn_options(opts: Attn, keep: list) -> _Attn:
         a.has_chunk, a.chunk_size, a.chunk_right = 1, size, right
         a.chunk_has_left, a.chunk_left = (0, 0) if left is None else (1, left)
     a.seg_start = _ref(keep, opts.seg_start)
-    a.has_cache = int(bool(opts.cache))
+    if opts.cache is not None:
+        c = _Cache()
+        c.head_start, c.kv_heads = int(opts.cache.head_start), int(opts.cache.kv_heads)
+        c.row_map = _ref(keep, opts.cache.row_map)
+        if opts.cache.appended is not None:
+            c.k_app, c.v_app = _ref(keep, opts.cache.appended[0]), _ref(keep, opts.cache.appended[1])
+        c.app_lens = _ref(keep, opts.cache.app_lens)
+        keep.append(c)
+        a.cache = ctypes.pointer(c)
     a.bias = _ref(keep, opts.bias)
     a.splits = opts.splits or 0
     if opts.scale is not None:

@@ -25,7 +25,7 @@ def test_every_declared_symbol_is_exported():
     lib = svod_amd.load_library()
     for n in sorted(names):
         assert hasattr(lib, n), n
-    assert lib.svodk_abi_version() == 2
+    assert lib.svodk_abi_version() == 3
 
 
 def test_status_names():
@@ -176,7 +176,7 @@ def test_packed_attention_validates_its_operand():
         svod_amd.attention_packed(t([2, 16, 12 * 64]), 5, 2)
     assert e.value.kind == "Heads"
     with pytest.raises(OpError) as e:
-        svod_amd.attention_packed(t([2, 16, 12 * 64]), 4, 4, Attn(cache=True))
+        svod_amd.attention_packed(t([2, 16, 12 * 64]), 4, 4, Attn(cache=svod_amd.Cache(0, 4)))
     assert e.value.kind == "Shape"
 
 
@@ -192,3 +192,27 @@ def test_the_split_workspace_is_the_partial_tensors():
         import ctypes
         got = lib.svodk_attention_workspace(ctypes.byref(qd), ctypes.byref(kd), ctypes.byref(a))
         assert got == want * 2 * 100 * 8 * (64 + 2) * 4
+
+
+# ---- a cache: tk/src/ops/attention.rs:146-170
+def test_a_cache_is_validated_as_the_reference_validates_it():
+    from svod_amd import Cache
+    q, cache_kv = t([2, 3, 4, 64]), t([5, 20, 12, 64])
+    lens = KeyMask.lens(t([2], I32))
+    kind, msg = kind_of(lambda: svod_amd.attention(q, cache_kv, cache_kv, Attn(cache=Cache(4, 4))))
+    assert kind == "Shape" and "k has shape" in msg                      # five rows, two lanes, no row map
+    kind, msg = kind_of(lambda: svod_amd.attention(q, cache_kv, cache_kv, Attn(cache=Cache(10, 4, row_map=t([2], I32)))))
+    assert kind == "Shape" and ">= 14" in msg                            # heads 10..14 of 12
+    kind, msg = kind_of(lambda: svod_amd.attention(q, cache_kv, cache_kv, Attn(cache=Cache(0, 3, row_map=t([2], I32)))))
+    assert kind == "Heads"
+    kind, msg = kind_of(lambda: svod_amd.attention(q, cache_kv, cache_kv, Attn(cache=Cache(0, 4, row_map=t([3], I32)))))
+    assert kind == "Shape" and "row map" in msg
+    app, short = t([2, 1, 4, 64]), t([2, 1, 2, 64])
+    kind, msg = kind_of(lambda: svod_amd.attention(q, cache_kv, cache_kv, Attn(keys=lens, cache=Cache(0, 4, t([2], I32), (app, short)))))
+    assert kind == "Shape" and "appended v" in msg
+    kind, msg = kind_of(lambda: svod_amd.attention(q, cache_kv, cache_kv, Attn(cache=Cache(0, 4, t([2], I32), (app, app)))))
+    assert kind == "Shape" and "key lens" in msg                         # appended rows need the prefix lengths
+    kind, msg = kind_of(lambda: svod_amd.attention(q, cache_kv, cache_kv, Attn(keys=lens, cache=Cache(0, 4, t([2], I32), app_lens=t([2], I32)))))
+    assert kind == "Shape" and "appended lens" in msg                    # counts without rows
+    kind, msg = kind_of(lambda: svod_amd.attention(q, cache_kv, cache_kv, Attn(keys=lens, bias=t([2, 4, 3, 20]), cache=Cache(0, 4, t([2], I32), (app, app)))))
+    assert kind == "Shape" and "bias" in msg and "21" in msg             # the bias counts the appended row

@@ -1,0 +1,120 @@
+"""Attention over a cache (Cache of tk/src/ops/attention.rs:39-56; tk/src/kernels/attention.rs:544-550,
+739-755, 827-846): k and v hold several layers' heads, batch lanes map to cache rows, and the rows a decoder
+step has just projected are scored after the cached prefix.  The cases are the reference's own
+(tk/src/test/unit/ops.rs:585-627: five lanes over two cache rows of three layers, lengths tk, 1, 37, tk-1, 0)
+at the head sizes this library has kernels for."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import svod_amd
+from svod_amd import Attn, Cache, KeyMask
+from util import Lcg, assert_bf16_parity, bf16_tensor, bits, max_abs, to_np
+
+pytestmark = pytest.mark.gpu
+
+B, ROWS, LAYERS = 5, 2, 3
+
+
+def operands(t, d, h, tk, appended, seed=40):
+    g = Lcg(seed)
+    q = g.bf16((B, t, h, d))
+    k, v = g.bf16((ROWS, tk, LAYERS * h, d)), g.bf16((ROWS, tk, LAYERS * h, d))
+    k_app, v_app = g.bf16((B, appended, h, d)), g.bf16((B, appended, h, d))
+    bias = g.bf16((B, h, t, tk + appended), mul=2.0)
+    lens = np.array([tk, 1, 37, tk - 1, 0])
+    row_map = np.array([0, 1, 1, 0, 1])
+    seen = np.array([max(appended - lane % 3, 1) for lane in range(B)])
+    return q, k, v, k_app, v_app, bias, lens, row_map, seen
+
+
+def run(device, t, d, h, tk, splits, appended, counted, biased, int_dtype=torch.int32, mapped=True):
+    q, k, v, k_app, v_app, bias, lens, row_map, seen = operands(t, d, h, tk, appended)
+    if not mapped:
+        k, v = (np.ascontiguousarray(x[row_map]) for x in (k, v))  # a cache row a lane
+    ints = lambda a: torch.from_numpy(np.asarray(a)).to(int_dtype).to(device)
+    cache = Cache(head_start=h, kv_heads=h, row_map=ints(row_map) if mapped else None,
+                  appended=(bf16_tensor(k_app, device), bf16_tensor(v_app, device)),
+                  app_lens=ints(seen) if counted else None)
+    opts = Attn(keys=KeyMask.lens(ints(lens)), cache=cache, splits=splits,
+                bias=bf16_tensor(bias, device) if biased else None)
+    got = svod_amd.attention(bf16_tensor(q, device), bf16_tensor(k, device), bf16_tensor(v, device), opts)
+    torch.cuda.synchronize()
+    assert svod_amd.chosen().startswith('Kernel { op: "attention"'), svod_amd.chosen()
+    p = oracle.AttnProblem(q, k, v, key_lens=lens, bias=bias if biased else None,
+                           cache=oracle.Cache(h, h, row_map if mapped else None, (k_app, v_app), seen if counted else None))
+    return got, p
+
+
+# ([t, d, h, tk], splits, appended, counted, biased): ops.rs:585-591, d 48 run at 64
+CASES = [
+    ("one query, 1500 keys, four splits", [1, 64, 20, 1500], 4, 1, False, False),
+    ("d 128 unsplit", [1, 128, 8, 300], None, 1, False, False),
+    ("three queries, two splits", [3, 64, 4, 200], 2, 1, False, False),
+    ("biased, three queries, two splits", [3, 64, 4, 200], 2, 1, False, True),
+    ("a streaming chunk: eight queries, eight appended", [8, 64, 16, 128], None, 8, False, False),
+    ("sixteen counted appended, two splits", [16, 64, 16, 128], 2, 16, True, False),
+    ("biased, counted appended", [8, 64, 4, 128], None, 8, True, True),
+    ("a full block of appended rows, d 128, biased", [5, 128, 4, 333], None, 64, True, True),
+    ("many queries over a long cache", [200, 64, 4, 700], None, 3, True, False),
+]
+
+
+@pytest.mark.parametrize("name,dims,splits,appended,counted,biased", CASES, ids=[c[0] for c in CASES])
+def test_cached_attention_matches_a_direct_softmax(device, name, dims, splits, appended, counted, biased):
+    t, d, h, tk = dims
+    got, p = run(device, t, d, h, tk, splits, appended, counted, biased)
+    direct = oracle.attention_direct(p)
+    program = oracle.attention_flash(p, bq=128, bkv=64, splits=min(splits or 1, (tk + 63) // 64))
+    assert_bf16_parity(name, to_np(got), direct, program)
+
+
+def test_a_lane_with_no_cached_keys_sees_only_the_appended_rows(device):
+    """Lane 4 of the fixture has length 0: its output is the softmax over its appended rows alone."""
+    t, d, h, tk, appended = 3, 64, 4, 200, 4
+    got, p = run(device, t, d, h, tk, None, appended, False, False)
+    q, k_app, v_app = p.q[4], p.cache.appended[0][4], p.cache.appended[1][4]
+    s = np.einsum("thd,nhd->htn", q.astype(np.float64), k_app.astype(np.float64)) / np.sqrt(d)
+    w = np.exp(s - s.max(-1, keepdims=True))
+    w /= w.sum(-1, keepdims=True)
+    want = np.einsum("htn,nhd->thd", w, v_app.astype(np.float64))
+    assert max_abs(to_np(got)[4], want) < 2e-2
+
+
+def test_the_row_map_is_a_gather_and_its_integers_may_be_64_bit(device):
+    t, d, h, tk = 5, 64, 4, 150
+    mapped, _ = run(device, t, d, h, tk, None, 2, True, False)
+    wide, _ = run(device, t, d, h, tk, None, 2, True, False, int_dtype=torch.int64)
+    gathered, _ = run(device, t, d, h, tk, None, 2, True, False, mapped=False)
+    assert np.array_equal(bits(mapped), bits(wide))
+    assert np.array_equal(bits(mapped), bits(gathered))
+
+
+def test_a_cache_without_appended_rows_is_a_view_of_its_heads(device):
+    """head_start and kv_heads alone: the same bits as attention over the narrowed, gathered tensors."""
+    t, d, h, tk = 40, 64, 4, 300
+    q, k, v, _, _, _, lens, row_map, _ = operands(t, d, h, tk, 1)
+    dev = lambda x: bf16_tensor(x, device)
+    ints = lambda a: torch.tensor(a, dtype=torch.int32, device=device)
+    for causal in (False, True):
+        cached = svod_amd.attention(dev(q), dev(k), dev(v), Attn(causal=causal, keys=KeyMask.lens(ints(lens)),
+                                                                 cache=Cache(2 * h, h, row_map=ints(row_map))))
+        plain = svod_amd.attention(dev(q), dev(np.ascontiguousarray(k[row_map][:, :, 2 * h:3 * h])),
+                                   dev(np.ascontiguousarray(v[row_map][:, :, 2 * h:3 * h])),
+                                   Attn(causal=causal, keys=KeyMask.lens(ints(lens))))
+        assert np.array_equal(bits(cached), bits(plain))
+
+
+def test_what_the_cache_has_no_kernel_for_keeps_the_graph(device):
+    t, d, h, tk = 4, 64, 4, 100
+    q, k, v, _, _, _, lens, row_map, _ = operands(t, d, h, tk, 1)
+    dev = lambda x: bf16_tensor(x, device)
+    ints = lambda a: torch.tensor(a, dtype=torch.int32, device=device)
+    g = Lcg(3)
+    many = (dev(g.bf16((B, 65, h, d))), dev(g.bf16((B, 65, h, d))))
+    for opts in (Attn(keys=KeyMask.lens(ints(lens)), cache=Cache(h, h, ints(row_map), appended=many)),
+                 Attn(keys=KeyMask.lens(ints(lens)), cache=Cache(h, h, ints(row_map)), window=(10, 0))):
+        with pytest.raises(svod_amd.GraphFallback) as e:
+            svod_amd.attention(dev(q), dev(k), dev(v), opts)
+        assert e.value.why == svod_amd.Fallback.Config

@@ -38,8 +38,8 @@ def parse():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="bge_m3",
-                    choices=["bge_m3", "bge_m3_bool", "qwen3_attention", "qwen3_prologue", "whisper", "long",
-                             "hbm_copy"],
+                    choices=["bge_m3", "bge_m3_bool", "qwen3_attention", "qwen3_prologue", "qwen3_add_rms_norm",
+                             "whisper", "long", "hbm_copy"],
                     help="hbm_copy is a plain 256 MiB device copy: the known-size kernel the HBM counters "
                          "(FETCH_SIZE, WRITE_SIZE) are calibrated on")
     ap.add_argument("--layers", type=int, default=24, help="calls per step for the bge_m3 workloads")
@@ -111,6 +111,20 @@ def main():
         workload = "Qwen3-Embedding prologue bf16 qkv[8,2048,4096] -> q,k,v (RMSNorm eps 1e-6 + RoPE theta 1e6)"
         cpu_sample = ("heads", p)
         kernel_name, bound = "heads_kernel<128>", "hbm"
+    elif args.workload == "qwen3_add_rms_norm":
+        # The residual add + RMSNorm between Qwen3-Embedding's layers: hidden size 16 heads x 128 = 2048.
+        g = torch.Generator(device=dev).manual_seed(0x5EED0030)
+        shape = (8, 2048, 2048)
+        xs = [torch.randn(shape, generator=g, device=dev).to(torch.bfloat16) for _ in range(4)]
+        rs = [torch.randn(shape, generator=g, device=dev).to(torch.bfloat16) for _ in range(4)]
+        wn = (0.8 + 0.4 * torch.rand(2048, generator=g, device=dev)).to(torch.bfloat16)
+        outs = [(torch.empty_like(xs[0]), torch.empty_like(xs[0])) for _ in range(4)]
+        for i in range(args.calls):
+            calls.append(lambda i=i: svod_amd.add_rms_norm(xs[i % 4], rs[i % 4], wn, 1e-6, out=outs[i % 4]))
+        bytes_min = 4 * xs[0].numel() * 2 + 2 * 2048  # x and residual read, sum and out written, the weight
+        workload = "Qwen3-Embedding residual add + RMSNorm bf16 x,residual [8,2048,2048] -> sum, out (eps 1e-6)"
+        cpu_sample = ("norm", (xs[0], rs[0], wn))
+        kernel_name, bound = "rows_kernel<4, rms, residual>", "hbm"
     else:
         if args.workload == "qwen3_attention":
             p = W.config3_prologue(device=dev)
@@ -221,7 +235,9 @@ def main():
                 "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": HBM_TRAFFIC_BYTES.get(args.workload),
                 "traffic_unit": "bytes per launch", "kernel": kernel_name,
                 "kernel_us": round(kernel_us, 3), "bytes_per_launch": bytes_min}
-        metric, unit = "attention prologue GB/s on 1 MI355X", "GB/s"
+        metric = ("row norm GB/s on 1 MI355X" if args.workload == "qwen3_add_rms_norm" else
+                  "attention prologue GB/s on 1 MI355X")
+        unit = "GB/s"
 
     # ---- CPU baseline: the oracle's restatement of the reference graph path, bounded sample.
     cpu = None
@@ -251,6 +267,20 @@ def cpu_baseline(sample, seconds, bound):
 
     kind, w = sample
     cores = min(os.cpu_count() or 1, 16)
+    if kind == "norm":
+        rows = 4096
+        x, r = (a.reshape(-1, a.shape[-1])[:rows].float().cpu().numpy() for a in w[:2])
+        wn = w[2].float().cpu().numpy()
+        t0 = time.perf_counter()
+        reps = 0
+        while time.perf_counter() - t0 < min(seconds, 5.0):
+            oracle.norm_f32(oracle.RMS, x, wn, residual=r, eps=1e-6)
+            reps += 1
+        dt = (time.perf_counter() - t0) / reps
+        nbytes = 4 * x.size * 2
+        return {"value": round(nbytes / dt / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": f"{rows} rows of one call (x, residual [{rows},2048]), f32 restatement of the graph path, "
+                          f"scalar C, {reps} reps"}
     if kind == "heads":
         rows = 256
         qkv = w.qkv[:1, :rows].float().cpu().numpy()

@@ -178,6 +178,25 @@ int svodk_heads(const svodk_tensor *qkv, const svodk_qkv *opts, const svodk_tens
                 const svodk_tensor *v, void *hip_stream);
 
 /*
+ * ops::layer_norm, add_layer_norm, rms_norm, add_rms_norm (tk/src/ops/norm.rs:16-42 -> norm, :44-98):
+ *   layer: (x - mean) * rsqrt(var + eps) * w + b      rms: x * rsqrt(mean(x^2) + eps) * w
+ * over the last dim of x [..., D], in f32, rounded once to x's type.  The add_ forms normalize
+ * x + residual and also write that sum, rounded to x's type first, to `sum`.  w and b are [D];
+ * b may be NULL; every operand has x's 16-bit type.  D is a multiple of 256 in 256..4096 (the
+ * reference stops at 2048); other widths answer SVODK_GRAPH_SHAPE.  `batch_live` is as in
+ * the attention options: <= 0 runs every batch.
+ */
+int svodk_layer_norm(const svodk_tensor *x, const svodk_tensor *w, const svodk_tensor *b, double eps, int32_t batch_live,
+                     const svodk_tensor *out, void *hip_stream);
+int svodk_add_layer_norm(const svodk_tensor *x, const svodk_tensor *residual, const svodk_tensor *w,
+                         const svodk_tensor *b, double eps, int32_t batch_live, const svodk_tensor *sum,
+                         const svodk_tensor *out, void *hip_stream);
+int svodk_rms_norm(const svodk_tensor *x, const svodk_tensor *w, double eps, int32_t batch_live, const svodk_tensor *out,
+                   void *hip_stream);
+int svodk_add_rms_norm(const svodk_tensor *x, const svodk_tensor *residual, const svodk_tensor *w, double eps,
+                       int32_t batch_live, const svodk_tensor *sum, const svodk_tensor *out, void *hip_stream);
+
+/*
  * The shape gates as pure functions, no device needed
  * (shape::attention, tk/src/ops/shape.rs:189-206; shape::heads, :209-218;
  * gate, :92-99).  `has_target` stands for "the default device has kernels".
@@ -188,6 +207,8 @@ int svodk_plan_attention(int32_t has_target, const int32_t *dtypes, int32_t n_dt
                          const int64_t *k_dims, int32_t causal, int32_t bias);
 int svodk_plan_heads(int32_t has_target, const int32_t *dtypes, int32_t n_dtypes, const int64_t *x_dims, int32_t x_rank,
                      int32_t head_dim);
+/* shape::norm (tk/src/ops/shape.rs:221-231). */
+int svodk_plan_norm(int32_t has_target, const int32_t *dtypes, int32_t n_dtypes, const int64_t *x_dims, int32_t x_rank);
 
 /*
  * A tuning knob in place of the reference's per-shape tuner (tk/src/tune.rs): attention calls

@@ -116,6 +116,10 @@ def _declare(l: ctypes.CDLL) -> None:
     l.svod_oracle_normal_fill.argtypes = [_f32p, ctypes.c_int64, ctypes.c_uint64, ctypes.c_double, ctypes.c_int]
     l.svod_oracle_rope_table.restype = None
     l.svod_oracle_rope_table.argtypes = [ctypes.c_double, _i32, _i32, _f32p, _f32p]
+    l.svod_oracle_norm_direct.restype = ctypes.c_int
+    l.svod_oracle_norm_direct.argtypes = [_i32, ctypes.c_int64, _i32, ctypes.c_double, _f32p, _f32p, _f32p, _f32p, _f64p, _f32p]
+    l.svod_oracle_norm_f32.restype = ctypes.c_int
+    l.svod_oracle_norm_f32.argtypes = [_i32, ctypes.c_int64, _i32, ctypes.c_double, _f32p, _f32p, _f32p, _f32p, _f32p, _f32p]
     l.svod_oracle_visible.restype = None
     l.svod_oracle_visible.argtypes = [_i32, _i32, _i32, _i32, _i32, _i32, _i32p, _i32p, _i32, _rangesp, _u8p]
     l.svod_oracle_visible_pairs.restype = ctypes.c_int64
@@ -419,3 +423,46 @@ def heads_kernel(p: HeadsProblem):
 def heads_graph(p: HeadsProblem):
     """The op's graph fallback (tk/src/ops/heads.rs:115-134)."""
     return _heads("svod_oracle_heads_graph", p)
+
+
+# --------------------------------------------------------------------------
+# row norms
+# --------------------------------------------------------------------------
+LAYER, RMS = 0, 1
+
+
+def _norm_args(x, residual, w, b):
+    x = _f32(x)
+    d = x.shape[-1]
+    rows = x.size // d
+    residual = None if residual is None else _f32(residual)
+    w = _f32(w)
+    b = None if b is None else _f32(b)
+    if w.shape != (d,) or (b is not None and b.shape != (d,)) or (residual is not None and residual.shape != x.shape):
+        raise ValueError("norm operands do not fit")
+    return x, residual, w, b, rows, d
+
+
+def norm_direct(kind: int, x, w, b=None, residual=None, eps: float = 1e-5):
+    """The f64 reference of tk/src/test/unit/rows.rs:169-197: ``(out float64 unrounded, sum float32 or None)``."""
+    x, residual, w, b, rows, d = _norm_args(x, residual, w, b)
+    out = np.empty(x.shape, dtype=np.float64)
+    total = None if residual is None else np.empty(x.shape, dtype=np.float32)
+    rc = lib().svod_oracle_norm_direct(kind, rows, d, float(eps), _ptr(x, _f32p), _ptr(residual, _f32p), _ptr(w, _f32p),
+                                       _ptr(b, _f32p), _ptr(out, _f64p), _ptr(total, _f32p))
+    if rc:
+        raise ValueError(f"oracle norm_direct rejected the problem (rc={rc})")
+    return out, total
+
+
+def norm_f32(kind: int, x, w, b=None, residual=None, eps: float = 1e-5):
+    """The kernel's and the graph's f32 arithmetic (tk/src/kernels/rows.rs:73-114, tk/src/ops/norm.rs:113-127),
+    rounded once to the stream dtype: ``(out float32, sum float32 or None)``."""
+    x, residual, w, b, rows, d = _norm_args(x, residual, w, b)
+    out = np.empty(x.shape, dtype=np.float32)
+    total = None if residual is None else np.empty(x.shape, dtype=np.float32)
+    rc = lib().svod_oracle_norm_f32(kind, rows, d, float(eps), _ptr(x, _f32p), _ptr(residual, _f32p), _ptr(w, _f32p),
+                                    _ptr(b, _f32p), _ptr(out, _f32p), _ptr(total, _f32p))
+    if rc:
+        raise ValueError(f"oracle norm_f32 rejected the problem (rc={rc})")
+    return out, total

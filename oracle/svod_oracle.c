@@ -51,6 +51,16 @@
  *   svod_oracle_heads_kernel, svod_oracle_heads_graph
  *       pinned against svod_oracle_heads_direct within 2e-2 / 1e-2
  *       (tk/src/test/unit/heads.rs:124,159); v is bit-exact.
+ *   svod_oracle_norm_direct
+ *       pinned against torch.nn.functional.layer_norm / rms_norm in float64
+ *       (library routines, not the reference) and closed forms (a constant
+ *       row, zero mean and var/(var+eps) variance, scale invariance); the
+ *       fused sum against torch's bf16 add, exactly.
+ *   svod_oracle_norm_f32
+ *       pinned against svod_oracle_norm_direct within the reference's 1e-2
+ *       (tk/src/test/unit/rows.rs:223); the ORDER of its row sums is this
+ *       file's own (neither the kernel nor the graph fixes one), so its bit
+ *       patterns are "parity unpinned" below that tolerance.
  *   svod_oracle_rope_table
  *       restates tensor/src/transformer.rs:130-164 with libm powf/cosf/sinf;
  *       the reference evaluates pow/cos/sin through its own f32 graph
@@ -906,4 +916,90 @@ int64_t svod_oracle_visible_pairs(int32_t batch, int32_t t, int32_t tk, int32_t 
     }
   }
   return pairs;
+}
+
+/* ------------------------------------------------------------------ */
+/* row norms: tk/src/kernels/rows.rs:41-115, tk/src/ops/norm.rs         */
+/*   kind 0: (x - mean) * rsqrt(var + eps) * w + b   (LayerNorm)       */
+/*   kind 1: x * rsqrt(mean(x^2) + eps) * w          (RMSNorm)         */
+/* x, residual, out, sum [rows, d]; w, b [d]; stream-dtype-exact f32.   */
+/* With a residual the sum x + residual is rounded to the stream dtype, */
+/* written out, and it is that rounded sum which is normalized          */
+/* (rows.rs:77-86).                                                    */
+/* ------------------------------------------------------------------ */
+
+/* The f64 reference of tk/src/test/unit/rows.rs:169-197: out and sum as f64, out unrounded here
+ * (the caller rounds where the reference's round_to does). */
+int svod_oracle_norm_direct(int32_t kind, int64_t rows, int32_t d, double eps, const float *x, const float *residual,
+                            const float *w, const float *b, double *out, float *sum) {
+  if (rows < 0 || d <= 0 || (kind != 0 && kind != 1)) return -1;
+  double *row = (double *)malloc(sizeof(double) * (size_t)d);
+  for (int64_t i = 0; i < rows; i++) {
+    for (int32_t c = 0; c < d; c++) {
+      const int64_t e = i * d + c;
+      if (residual) {
+        const float s = round_stream(x[e] + residual[e]); /* L183-184 */
+        if (sum) sum[e] = s;
+        row[c] = (double)s;
+      } else {
+        row[c] = (double)x[e];
+      }
+    }
+    double mean = 0.0;
+    if (kind == 0) {
+      for (int32_t c = 0; c < d; c++) mean += row[c];
+      mean /= (double)d;
+    }
+    double var = 0.0;
+    for (int32_t c = 0; c < d; c++) var += (row[c] - mean) * (row[c] - mean);
+    var /= (double)d;
+    const double inv = 1.0 / sqrt(var + eps);
+    for (int32_t c = 0; c < d; c++)
+      out[i * d + c] = (row[c] - mean) * inv * (double)w[c] + ((kind == 0 && b) ? (double)b[c] : 0.0);
+  }
+  free(row);
+  return 0;
+}
+
+/* The kernel's arithmetic (rows.rs:73-114) and the graph's (tk/src/ops/norm.rs:113-127 ->
+ * tensor/src/nn/norm.rs:62-75,146-168): everything in f32, one rounding to the stream dtype at
+ * the end; the two differ only in the order of the row sums, which neither source fixes.
+ * mean = sum * (1/d) with 1/d rounded to f32 (affine, rows.rs:88-91); var + eps in f32. */
+int svod_oracle_norm_f32(int32_t kind, int64_t rows, int32_t d, double eps, const float *x, const float *residual,
+                         const float *w, const float *b, float *out, float *sum) {
+  if (rows < 0 || d <= 0 || (kind != 0 && kind != 1)) return -1;
+  float *row = (float *)malloc(sizeof(float) * (size_t)d);
+  const float inv_d = (float)(1.0 / (double)d), feps = (float)eps;
+  for (int64_t i = 0; i < rows; i++) {
+    for (int32_t c = 0; c < d; c++) {
+      const int64_t e = i * d + c;
+      if (residual) {
+        const float s = round_stream(x[e] + residual[e]);
+        if (sum) sum[e] = s;
+        row[c] = s;
+      } else {
+        row[c] = x[e];
+      }
+    }
+    float mean = 0.0f;
+    if (kind == 0) {
+      float acc = 0.0f;
+      for (int32_t c = 0; c < d; c++) acc += row[c];
+      mean = acc * inv_d;
+    }
+    float acc = 0.0f;
+    for (int32_t c = 0; c < d; c++) {
+      const float ctr = row[c] - mean;
+      acc += ctr * ctr;
+    }
+    const float var = acc * inv_d + feps;
+    const float inv = 1.0f / sqrtf(var);
+    for (int32_t c = 0; c < d; c++) {
+      float y = ((row[c] - mean) * inv) * w[c];
+      if (kind == 0 && b) y += b[c];
+      out[i * d + c] = round_stream(y);
+    }
+  }
+  free(row);
+  return 0;
 }

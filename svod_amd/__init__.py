@@ -15,14 +15,19 @@ from .ops import (  # noqa: F401
     KeyMask,
     OpError,
     Qkv,
+    add_layer_norm,
+    add_rms_norm,
     attention,
     attention_packed,
     tune_streaming,
     chosen,
     heads,
+    layer_norm,
     library_path,
     load_library,
     plan_attention,
     plan_heads,
+    plan_norm,
+    rms_norm,
     supported,
 )

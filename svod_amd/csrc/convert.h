@@ -1,0 +1,56 @@
+// Widening and narrowing between the operands' 16-bit float types and f32, shared by the
+// row-wise kernels (the attention prologue and the row norms).
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+namespace svodk {
+
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+
+// Round to nearest even, NaN quieted: the rule of tk/src/interp.rs:37-44.
+__device__ __forceinline__ uint32_t to_bf16_bits(float x) {
+  uint32_t bits = __float_as_uint(x);
+  uint32_t rounded = (bits + 0x7fffu + ((bits >> 16) & 1u)) >> 16;
+  return (x != x) ? ((bits | 0x00400000u) >> 16) : rounded;
+}
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+  return to_bf16_bits(lo) | (to_bf16_bits(hi) << 16);
+}
+
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+
+// Eight 16-bit values of the operands' type, widened exactly.
+template <bool F16>
+__device__ __forceinline__ void widen(const u32x4 &w, float (&x)[8]) {
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    if constexpr (F16) {
+      const uint32_t pair = w[i];  // a copy: the cast below wants an object of its own, not a vector's element
+      const f32x2 f = __builtin_convertvector(__builtin_bit_cast(f16x2, pair), f32x2);
+      x[2 * i] = f[0];
+      x[2 * i + 1] = f[1];
+    } else {
+      x[2 * i] = bf16_lo(w[i]);
+      x[2 * i + 1] = bf16_hi(w[i]);
+    }
+  }
+}
+
+// Two f32 values rounded to the operands' type, nearest even (tk/src/interp.rs:37-50).
+template <bool F16>
+__device__ __forceinline__ uint32_t narrow(float lo, float hi) {
+  if constexpr (F16) {
+    const f32x2 f = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, f16x2));
+  } else {
+    return pack_bf16(lo, hi);
+  }
+}
+
+}  // namespace svodk

@@ -25,6 +25,24 @@ hipError_t launch_heads(const HeadsArgs &a, hipStream_t stream);
 // Head sizes the prologue kernel is built for.
 bool heads_supports(int32_t d);
 
+// Row norms: tk/src/kernels/rows.rs:41-115 (norm_body).
+struct NormArgs {
+  const void *x;         // [rows, d]
+  const void *residual;  // [rows, d] or null: normalize x + residual, the sum written to `sum`
+  const void *w;         // [d]
+  const void *b;         // [d] or null (LayerNorm only)
+  void *out;             // [rows, d]
+  void *sum;             // [rows, d] with a residual
+  int64_t rows;          // live rows
+  int32_t d;
+  double eps;
+  int32_t layer;  // LayerNorm (1) or RMSNorm (0)
+  int32_t f16;    // every operand is f16, not bf16
+};
+hipError_t launch_norm(const NormArgs &a, hipStream_t stream);
+// Row widths the norm kernel is built for.
+bool norm_supports(int64_t d);
+
 // Flash attention forward: tk/src/kernels/attention.rs:466-924 (attention_body).
 struct AttnArgs {
   const void *q;  // [batch, t, heads, d] bf16

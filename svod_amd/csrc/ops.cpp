@@ -197,6 +197,19 @@ int plan_heads(bool has_target, const int32_t *dtypes, int n, const int64_t *x, 
   return 0;
 }
 
+// shape::norm (L221-231) with norm_candidates (tk/src/ops/config/norm.rs:19-24): the reduced dim a
+// multiple of 256 from 256 on, no empty dim.  The reference stops at 2048 (64 elements a lane of
+// its 32-lane warp); a 64-lane wave holds 4096 the same way, so the kernel here goes that far.
+int plan_norm(bool has_target, const int32_t *dtypes, int n, const int64_t *x, int rank) {
+  if (int why = gate(has_target, dtypes, n)) return why;
+  if (x == nullptr) return SVODK_GRAPH_SYMBOLIC;
+  if (rank < 1) return SVODK_GRAPH_SHAPE;
+  for (int i = 0; i < rank; i++)
+    if (x[i] == 0) return SVODK_GRAPH_SHAPE;
+  if (!svodk::norm_supports(x[rank - 1])) return SVODK_GRAPH_SHAPE;
+  return 0;
+}
+
 const char *OP_ATTN = "attention";
 const char *OP_HEADS = "heads";
 
@@ -693,6 +706,117 @@ int svodk_heads(const svodk_tensor *qkv, const svodk_qkv *opts, const svodk_tens
   const hipError_t e = svodk::launch_heads(a, (hipStream_t)hip_stream);
   if (e != hipSuccess) return fail(SVODK_ERR_LAUNCH, "%s: %s", op, hipGetErrorString(e));
   return SVODK_KERNEL;
+}
+
+// norm (tk/src/ops/norm.rs:44-98): LayerNorm or RMSNorm over the last dim of x, after a residual
+// add when there is one.
+static int norm(bool layer, const svodk_tensor *x, const svodk_tensor *residual, const svodk_tensor *w,
+                const svodk_tensor *b, double eps, int32_t batch_live, const svodk_tensor *sum, const svodk_tensor *out,
+                void *hip_stream) {
+  const char *op = layer ? "layer_norm" : "rms_norm";
+  if (!well_formed(x) || !well_formed(w) || !well_formed(out) || (b && !well_formed(b)) ||
+      (residual && !well_formed(residual)) || (sum && !well_formed(sum)))
+    return fail(SVODK_ERR_ARGUMENT, "%s: a null or malformed tensor descriptor", op);
+  if ((residual != nullptr) != (sum != nullptr))
+    return fail(SVODK_ERR_ARGUMENT, "%s: the sum comes with a residual and only with one", op);
+  // L54-60: x is [..., D]; w and b are [D].
+  if (x->rank < 1) return fail(SVODK_ERR_SHAPE, "%s: x has shape %s, expected [..., D]", op, fmt_shape(x).c_str());
+  const int64_t d = x->shape[x->rank - 1];
+  const svodk_tensor *vecs[2] = {w, b};
+  const char *vec_names[2] = {"w", "b"};
+  for (int i = 0; i < 2; i++)
+    if (vecs[i] != nullptr && !(vecs[i]->rank == 1 && vecs[i]->shape[0] == d))
+      return fail(SVODK_ERR_SHAPE, "%s: %s has shape %s, expected [%lld]", op, vec_names[i], fmt_shape(vecs[i]).c_str(),
+                  (long long)d);
+  // L61-64: the residual has x's shape.
+  if (residual != nullptr && !same_shape(residual, x))
+    return fail(SVODK_ERR_SHAPE, "%s: residual has shape %s, expected %s", op, fmt_shape(residual).c_str(),
+                fmt_shape(x).c_str());
+  // The outputs the reference op allocates itself (L88-89): here the caller's.
+  const svodk_tensor *outs[2] = {out, sum};
+  const char *out_names[2] = {"out", "sum"};
+  for (int i = 0; i < 2; i++) {
+    if (outs[i] == nullptr) continue;
+    if (!same_shape(outs[i], x))
+      return fail(SVODK_ERR_SHAPE, "%s: %s has shape %s, expected %s", op, out_names[i], fmt_shape(outs[i]).c_str(),
+                  fmt_shape(x).c_str());
+    if (outs[i]->dtype != x->dtype)
+      return fail(SVODK_ERR_DTYPE, "%s: %s is %s, the input is %s", op, out_names[i], dtype_name(outs[i]->dtype),
+                  dtype_name(x->dtype));
+  }
+  const int64_t cap = x->shape[0];
+  if (batch_live > cap)
+    return fail(SVODK_ERR_SHAPE, "%s: live batch %d exceeds the capacity %lld", op, batch_live, (long long)cap);
+
+  // L66-71: the plan over every operand's type.
+  int32_t dtypes[4];
+  int n = 0;
+  dtypes[n++] = x->dtype;
+  if (residual) dtypes[n++] = residual->dtype;
+  dtypes[n++] = w->dtype;
+  if (b) dtypes[n++] = b->dtype;
+  const int why = plan_norm(current_device_has_kernels(), dtypes, n, x->shape, x->rank);
+  if (why != 0) return ran_graph(op, why);
+
+  const size_t bytes = (size_t)numel(x) * 2;
+  Span spans[6] = {{"x", x->data, bytes, false},
+                   {"residual", residual ? residual->data : nullptr, residual ? bytes : 0, false},
+                   {"w", w->data, (size_t)d * 2, false},
+                   {"b", b ? b->data : nullptr, b ? (size_t)d * 2 : 0, false},
+                   {"out", out->data, bytes, true},
+                   {"sum", sum ? sum->data : nullptr, sum ? bytes : 0, true}};
+  if (x->data == nullptr || w->data == nullptr || out->data == nullptr || (b && b->data == nullptr) ||
+      (residual && residual->data == nullptr) || (sum && sum->data == nullptr))
+    return fail(SVODK_ERR_ARGUMENT, "%s: a null device pointer", op);
+  if (int rc = check_aliasing(op, spans, 6)) return rc;
+
+  svodk::NormArgs a{};
+  a.x = x->data;
+  a.residual = residual ? residual->data : nullptr;
+  a.w = w->data;
+  a.b = (layer && b) ? b->data : nullptr;
+  a.out = out->data;
+  a.sum = sum ? sum->data : nullptr;
+  // L74-76: the rows are every dim before the last; a bound leading batch runs its live part.
+  const int64_t per_batch = x->rank > 1 ? numel(x) / (cap * d) : 1;
+  a.rows = x->rank > 1 ? (batch_live > 0 ? batch_live : cap) * per_batch : 1;
+  a.d = (int32_t)d;
+  a.eps = eps;
+  a.layer = layer;
+  a.f16 = x->dtype == SVODK_F16;
+  ran(op, op, "NormCfg { br: 4 }");
+  const hipError_t e = svodk::launch_norm(a, (hipStream_t)hip_stream);
+  if (e != hipSuccess) return fail(SVODK_ERR_LAUNCH, "%s: %s", op, hipGetErrorString(e));
+  return SVODK_KERNEL;
+}
+
+int svodk_layer_norm(const svodk_tensor *x, const svodk_tensor *w, const svodk_tensor *b, double eps, int32_t batch_live,
+                     const svodk_tensor *out, void *hip_stream) {
+  return norm(true, x, nullptr, w, b, eps, batch_live, nullptr, out, hip_stream);
+}
+
+int svodk_add_layer_norm(const svodk_tensor *x, const svodk_tensor *residual, const svodk_tensor *w,
+                         const svodk_tensor *b, double eps, int32_t batch_live, const svodk_tensor *sum,
+                         const svodk_tensor *out, void *hip_stream) {
+  if (residual == nullptr || sum == nullptr)
+    return fail(SVODK_ERR_ARGUMENT, "layer_norm: add_layer_norm needs a residual and a sum");
+  return norm(true, x, residual, w, b, eps, batch_live, sum, out, hip_stream);
+}
+
+int svodk_rms_norm(const svodk_tensor *x, const svodk_tensor *w, double eps, int32_t batch_live, const svodk_tensor *out,
+                   void *hip_stream) {
+  return norm(false, x, nullptr, w, nullptr, eps, batch_live, nullptr, out, hip_stream);
+}
+
+int svodk_add_rms_norm(const svodk_tensor *x, const svodk_tensor *residual, const svodk_tensor *w, double eps,
+                       int32_t batch_live, const svodk_tensor *sum, const svodk_tensor *out, void *hip_stream) {
+  if (residual == nullptr || sum == nullptr)
+    return fail(SVODK_ERR_ARGUMENT, "rms_norm: add_rms_norm needs a residual and a sum");
+  return norm(false, x, residual, w, nullptr, eps, batch_live, sum, out, hip_stream);
+}
+
+int svodk_plan_norm(int32_t has_target, const int32_t *dtypes, int32_t n_dtypes, const int64_t *x_dims, int32_t x_rank) {
+  return plan_norm(has_target != 0, dtypes, n_dtypes, x_dims, x_rank);
 }
 
 }  // extern "C"

@@ -87,6 +87,14 @@ def load_library() -> ctypes.CDLL:
     lib.svodk_plan_attention.argtypes = [ctypes.c_int32, i32p, ctypes.c_int32, i64p, i64p, ctypes.c_int32, ctypes.c_int32]
     lib.svodk_plan_heads.restype = ctypes.c_int
     lib.svodk_plan_heads.argtypes = [ctypes.c_int32, i32p, ctypes.c_int32, i64p, ctypes.c_int32, ctypes.c_int32]
+    for name, n_tensors_before_eps in (("svodk_layer_norm", 3), ("svodk_add_layer_norm", 4), ("svodk_rms_norm", 2),
+                                       ("svodk_add_rms_norm", 3)):
+        fn = getattr(lib, name)
+        fn.restype = ctypes.c_int
+        n_outputs = 2 if "add_" in name else 1
+        fn.argtypes = [tp] * n_tensors_before_eps + [ctypes.c_double, ctypes.c_int32] + [tp] * n_outputs + [ctypes.c_void_p]
+    lib.svodk_plan_norm.restype = ctypes.c_int
+    lib.svodk_plan_norm.argtypes = [ctypes.c_int32, i32p, ctypes.c_int32, i64p, ctypes.c_int32]
     lib.svodk_tune_streaming.restype = None
     lib.svodk_tune_streaming.argtypes = [ctypes.c_int32]
     lib.svodk_supported.restype = ctypes.c_int
@@ -349,6 +357,61 @@ def heads(qkv: torch.Tensor, opts: Qkv, out: Optional[Tuple[torch.Tensor, torch.
                              ctypes.c_void_p(_stream(qkv)))
     _finish("heads", status)
     return out
+
+
+def _norm(name: str, x, residual, w, b, eps, batch_live, out):
+    lib = load_library()
+    keep: list = []
+    fused = residual is not None
+    if out is None:
+        out = (torch.empty_like(x), torch.empty_like(x)) if fused else torch.empty_like(x)
+    none = ctypes.POINTER(_Tensor)()
+    args = [_ref(keep, x)]
+    if fused:
+        args.append(_ref(keep, residual))
+    args.append(_ref(keep, w))
+    if "layer" in name:
+        args.append(_ref(keep, b) if b is not None else none)
+    args += [ctypes.c_double(float(eps)), ctypes.c_int32(batch_live or 0)]
+    args += [_ref(keep, out[0]), _ref(keep, out[1])] if fused else [_ref(keep, out)]
+    status = getattr(lib, "svodk_" + name)(*args, ctypes.c_void_p(_stream(x)))
+    _finish("layer_norm" if "layer" in name else "rms_norm", status)
+    return out
+
+
+def layer_norm(x: torch.Tensor, w: torch.Tensor, b: Optional[torch.Tensor] = None, eps: float = 1e-5,
+               out: Optional[torch.Tensor] = None, batch_live: Optional[int] = None) -> torch.Tensor:
+    """``(x - mean)·rsqrt(var + eps)·w + b`` over the last dim of ``x`` (tk/src/ops/norm.rs:16-19)."""
+    return _norm("layer_norm", x, None, w, b, eps, batch_live, out)
+
+
+def add_layer_norm(x: torch.Tensor, residual: torch.Tensor, w: torch.Tensor, b: Optional[torch.Tensor] = None,
+                   eps: float = 1e-5, out: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
+                   batch_live: Optional[int] = None):
+    """``(x + residual, layer_norm(x + residual))``, the sum rounded to the input type first
+    (tk/src/ops/norm.rs:21-31); ``out`` is ``(sum, y)``."""
+    return _norm("add_layer_norm", x, residual, w, b, eps, batch_live, out)
+
+
+def rms_norm(x: torch.Tensor, w: torch.Tensor, eps: float = 1e-5, out: Optional[torch.Tensor] = None,
+             batch_live: Optional[int] = None) -> torch.Tensor:
+    """``x·rsqrt(mean(x²) + eps)·w`` over the last dim of ``x`` (tk/src/ops/norm.rs:33-36)."""
+    return _norm("rms_norm", x, None, w, None, eps, batch_live, out)
+
+
+def add_rms_norm(x: torch.Tensor, residual: torch.Tensor, w: torch.Tensor, eps: float = 1e-5,
+                 out: Optional[Tuple[torch.Tensor, torch.Tensor]] = None, batch_live: Optional[int] = None):
+    """``(x + residual, rms_norm(x + residual))``, the sum rounded to the input type first
+    (tk/src/ops/norm.rs:38-42); ``out`` is ``(sum, y)``."""
+    return _norm("add_rms_norm", x, residual, w, None, eps, batch_live, out)
+
+
+def plan_norm(has_target: bool, dtypes, x_dims) -> Optional[Fallback]:
+    """``shape::norm`` (tk/src/ops/shape.rs:221-231) as a pure function."""
+    lib = load_library()
+    dt = (ctypes.c_int32 * len(dtypes))(*[_DTYPES[d] for d in dtypes])
+    xd = None if x_dims is None else (ctypes.c_int64 * len(x_dims))(*x_dims)
+    return _plan(lib.svodk_plan_norm(int(has_target), dt, len(dtypes), xd, 0 if x_dims is None else len(x_dims)))
 
 
 def chosen() -> str:

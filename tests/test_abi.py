@@ -216,3 +216,39 @@ def test_a_cache_is_validated_as_the_reference_validates_it():
     assert kind == "Shape" and "appended lens" in msg                    # counts without rows
     kind, msg = kind_of(lambda: svod_amd.attention(q, cache_kv, cache_kv, Attn(keys=lens, bias=t([2, 4, 3, 20]), cache=Cache(0, 4, t([2], I32), (app, app)))))
     assert kind == "Shape" and "bias" in msg and "21" in msg             # the bias counts the appended row
+
+
+# ---- norms: tk/src/ops/norm.rs:54-64 and tk/src/ops/config/norm.rs:19-24
+@pytest.mark.parametrize("d,want", [(256, None), (768, None), (2048, None), (4096, None), (128, Fallback.Shape),
+                                    (1000, Fallback.Shape), (8192, Fallback.Shape)])
+def test_norm_plan(d, want):
+    assert svod_amd.plan_norm(True, [BF16, BF16], [4, 37, d]) == want
+
+
+def test_norm_plan_gates():
+    assert svod_amd.plan_norm(False, [BF16, BF16], [37, 512]) == Fallback.Target
+    assert svod_amd.plan_norm(True, [BF16, F16], [37, 512]) == Fallback.Dtype
+    assert svod_amd.plan_norm(True, [torch.float32, torch.float32], [37, 512]) == Fallback.Dtype
+    assert svod_amd.plan_norm(True, [BF16, BF16], None) == Fallback.Symbolic
+    assert svod_amd.plan_norm(True, [BF16, BF16], [0, 512]) == Fallback.Shape
+
+
+def test_norms_reject_what_the_graph_would_reject():
+    x = t([2, 10, 512])
+    kind, msg = kind_of(lambda: svod_amd.rms_norm(x, t([256])))
+    assert kind == "Shape" and msg.startswith("rms_norm: w has shape")
+    kind, msg = kind_of(lambda: svod_amd.layer_norm(x, t([512]), t([2, 512])))
+    assert kind == "Shape" and msg.startswith("layer_norm: b has shape")
+    kind, msg = kind_of(lambda: svod_amd.add_rms_norm(x, t([2, 9, 512]), t([512])))
+    assert kind == "Shape" and "residual has shape" in msg
+    kind, msg = kind_of(lambda: svod_amd.add_layer_norm(x, t([2, 10, 512]), t([512]), out=(t([2, 10, 512]), t([2, 10, 256]))))
+    assert kind == "Shape" and "out has shape" in msg
+
+
+def test_without_a_device_a_norm_names_the_graph():
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present: the Target fallback is the no-device outcome")
+    with pytest.raises(GraphFallback) as e:
+        svod_amd.layer_norm(t([4, 512]), t([512]))
+    assert e.value.why == Fallback.Target
+    assert svod_amd.chosen() == 'Graph { op: "layer_norm", why: Target }'

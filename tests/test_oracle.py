@@ -514,3 +514,59 @@ def test_bias_closed_forms():
     w /= w.sum(-1, keepdims=True)
     want = np.einsum("bhij,bjhd->bihd", w, np.repeat(v.astype(np.float64), 2, axis=2))
     assert max_abs(oracle.attention_direct(p), want) < 1e-12
+
+
+# ---------------------------------------------------------------- row norms
+def norm_case(rows, d, seed=5):
+    """norm_inputs of tk/src/test/unit/rows.rs:147-165: x = 2u + 1.5 (a mean away from zero), r = u, w = 1 + u/2, b = u/2."""
+    g = Lcg(seed)
+    return g.bf16((rows, d), mul=2.0, add=1.5), g.bf16((rows, d)), g.bf16((d,), mul=0.5, add=1.0), g.bf16((d,), mul=0.5)
+
+
+@pytest.mark.parametrize("d", [256, 768, 2048])
+def test_norms_match_torch_float64(d):
+    x, r, w, b = norm_case(37, d)
+    t64 = lambda a: torch.tensor(a, dtype=torch.float64)
+    want = torch.nn.functional.layer_norm(t64(x), (d,), t64(w), t64(b), 1e-5).numpy()
+    assert max_abs(oracle.norm_direct(oracle.LAYER, x, w, b, eps=1e-5)[0], want) < 1e-12
+    want = torch.nn.functional.layer_norm(t64(x), (d,), t64(w), None, 1e-5).numpy()
+    assert max_abs(oracle.norm_direct(oracle.LAYER, x, w, eps=1e-5)[0], want) < 1e-12
+    want = torch.nn.functional.rms_norm(t64(x), (d,), t64(w), 1e-6).numpy()
+    assert max_abs(oracle.norm_direct(oracle.RMS, x, w, eps=1e-6)[0], want) < 1e-12
+    # The fused residual: the sum is rounded to bf16 first (tk/src/kernels/rows.rs:77-86), exactly.
+    total = (torch.tensor(x) + torch.tensor(r)).to(torch.bfloat16)
+    got, got_sum = oracle.norm_direct(oracle.RMS, x, w, residual=r, eps=1e-6)
+    assert np.array_equal(got_sum, total.to(torch.float32).numpy())
+    assert max_abs(got, torch.nn.functional.rms_norm(total.to(torch.float64), (d,), t64(w), 1e-6).numpy()) < 1e-12
+
+
+@pytest.mark.parametrize("kind,residual,bias", [(0, False, True), (0, True, False), (1, False, False), (1, True, False)])
+def test_the_f32_norm_is_within_the_references_tolerance_of_float64(kind, residual, bias):
+    """tk/src/test/unit/rows.rs:223, 250-251: rel 1e-2 against the f64 reference rounded to bf16."""
+    x, r, w, b = norm_case(37, 1024)
+    args = dict(residual=r if residual else None, eps=1e-5)
+    got, got_sum = oracle.norm_f32(kind, x, w, b if bias else None, **args)
+    want, want_sum = oracle.norm_direct(kind, x, w, b if bias else None, **args)
+    assert np.all(np.abs(got - want) <= 1e-2 * np.maximum(np.abs(want), 1.0))
+    if residual:
+        assert np.array_equal(got_sum, want_sum)
+
+
+def test_norm_closed_forms():
+    d = 512
+    ones = np.ones(d, dtype=np.float32)
+    # A constant row: RMSNorm gives c / sqrt(c^2 + eps); LayerNorm gives the bias (the centred row is zero).
+    row = np.full((1, d), 3.0, dtype=np.float32)
+    assert max_abs(oracle.norm_direct(oracle.RMS, row, ones, eps=1e-6)[0], np.full((1, d), 3.0 / np.sqrt(9.0 + 1e-6))) < 1e-12
+    assert max_abs(oracle.norm_direct(oracle.LAYER, row, ones, 0.25 * ones, eps=1e-5)[0], np.full((1, d), 0.25)) < 1e-12
+    # Unit weights, no bias: a LayerNorm row has mean 0 and variance var / (var + eps).
+    x = norm_case(9, d)[0]
+    y = oracle.norm_direct(oracle.LAYER, x, ones, eps=1e-5)[0]
+    assert np.abs(y.mean(-1)).max() < 1e-12
+    var = x.astype(np.float64).var(-1)
+    assert np.abs(y.var(-1) - var / (var + 1e-5)).max() < 1e-12
+    # Scaling a row by 2^k leaves a LayerNorm unchanged up to eps, and RMSNorm's mean square is 1 - eps-ish.
+    y2 = oracle.norm_direct(oracle.LAYER, 4.0 * x, ones, eps=0.0)[0]
+    assert max_abs(y2, oracle.norm_direct(oracle.LAYER, x, ones, eps=0.0)[0]) < 1e-12
+    z = oracle.norm_direct(oracle.RMS, x, ones, eps=0.0)[0]
+    assert np.abs((z * z).mean(-1) - 1.0).max() < 1e-12

@@ -98,14 +98,17 @@ typedef struct svodk_cache {
  * a window, a chunk mask or segment starts, and more than 64 appended rows,
  * answer SVODK_GRAPH_CONFIG.
  *
- * `splits` > 1 asks for key splits (tk/src/ops/attention.rs:79, 280-302): the
+ * `splits` > 1 asks for key splits (tk/src/ops/attention.rs:76-79, 280-302): the
  * count is capped at the number of 64-key blocks of Tk (split_ranked, :405-410);
  * each split leaves a partial state in `workspace` and combine_splits
  * (tk/src/kernels/attention.rs:984-1014) merges them into `out`.  The reference
  * op allocates those partial tensors itself; this library allocates nothing,
  * so the caller lends `workspace` (svodk_attention_workspace says how many
- * bytes).  Without a large enough workspace a split call answers
- * SVODK_GRAPH_CONFIG.
+ * bytes).  A named count without a large enough workspace answers
+ * SVODK_GRAPH_CONFIG.  `splits` = 1 keeps the keys whole.  `splits` = 0 (None)
+ * lets the library choose, as the reference's tuner would: it splits calls with
+ * few query tiles and many keys (a decoder step) when the workspace
+ * svodk_attention_workspace asks for is lent, and keeps the keys whole without it.
  */
 typedef struct svodk_attn {
   int32_t causal;
@@ -120,7 +123,7 @@ typedef struct svodk_attn {
   const svodk_tensor *seg_start; /* [B, T] integers or NULL */
   const svodk_cache *cache;      /* or NULL */
   const svodk_tensor *bias;      /* [B|1, H, T, Tk] or NULL */
-  int32_t splits;                /* 0 = None */
+  int32_t splits;                /* 0 = None: the library chooses */
   int32_t has_scale;
   float scale; /* used when has_scale; else 1/sqrt(D) */
   /* Batch::Var of tk/src/kernels/mod.rs:221-259: buffers hold `q.shape[0]`

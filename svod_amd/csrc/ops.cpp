@@ -253,11 +253,27 @@ int svodk_plan_heads(int32_t has_target, const int32_t *dtypes, int32_t n_dtypes
 }
 
 // split_ranked of tk/src/ops/attention.rs:405-410 for this library's one tile shape: a named
-// count is capped at the 64-key blocks of tk; none, or one, leaves the keys unsplit.
-static int split_count(int32_t asked, int64_t tk) {
+// count is capped at the 64-key blocks of tk; one leaves the keys unsplit.  With none named the
+// reference lets its tuner choose "among one, two, the counts around two blocks per SM and the
+// block count" (tk/src/ops/attention.rs:76-79) by measurement; here a rule stands where the
+// tuner would: enough splits for about two workgroups a CU (512 on an MI355X), each with at
+// least 8 key blocks.  Measured on decode and short-query shapes (kernel + merge, microseconds,
+// unsplit -> rule's count): 16 workgroups x 128 blocks 101.6 -> 24.2 (16 splits), 32 x 128
+// 151.5 -> 29.8 (16), 64 x 32 28.7 -> 16.8 (4), 64 x 64 82.7 -> 37.6 (8), 256 x 64 86.2 -> 67.4
+// (2), 320 x 24 32.7 -> 28.6 (2); from 640 workgroups on the rule answers one, which is fastest.
+// A window, a chunk mask or segment starts leave a tile few of the keys: the rule keeps those whole.
+static int split_count(const svodk_attn *opts, int64_t batch, int64_t t, int64_t heads, int64_t tk) {
+  const int32_t asked = opts->splits;
   const int64_t most = tk > 0 ? (tk + 63) / 64 : 1;
-  if (asked <= 1) return 1;
-  return (int)(asked < most ? asked : most);
+  if (asked == 1) return 1;
+  if (asked > 1) return (int)(asked < most ? asked : most);
+  if (opts->has_window || opts->has_chunk || opts->seg_start != nullptr) return 1;
+  const int64_t workgroups = (t + 127) / 128 * heads * batch;
+  if (workgroups <= 0) return 1;
+  const int64_t wanted = (512 + workgroups / 2) / workgroups;  // rounded
+  const int64_t fits = most / 8;
+  const int64_t n = wanted < fits ? wanted : fits;
+  return (int)(n < 1 ? 1 : (n > 64 ? 64 : n));
 }
 
 // attend (tk/src/ops/attention.rs:126-303): attention of q, k and v, or of the `packed` operand
@@ -511,11 +527,18 @@ static int attend(const svodk_tensor *q, const svodk_tensor *k, const svodk_tens
     }
   }
   // L280-302: key splits.  The partial tensors live in the caller's workspace.
-  a.splits = split_count(opts->splits, tk);
+  a.splits = split_count(opts, a.batch, t, heads, tk);
+  if (a.splits > 1) {
+    const int64_t rows = (int64_t)a.batch * t * heads;
+    int64_t need = (int64_t)a.splits * rows * (d + 2) * 4;
+    const bool lent = opts->workspace != nullptr && opts->workspace_bytes >= need;
+    // Splits the caller named need their workspace; splits of the rule's own are dropped without it.
+    if (!lent && opts->splits > 1) return ran_graph(op, SVODK_GRAPH_CONFIG);
+    if (!lent) a.splits = 1, need = 0;
+  }
   if (a.splits > 1) {
     const int64_t rows = (int64_t)a.batch * t * heads;
     const int64_t need = (int64_t)a.splits * rows * (d + 2) * 4;
-    if (opts->workspace == nullptr || opts->workspace_bytes < need) return ran_graph(op, SVODK_GRAPH_CONFIG);
     Span ws[2] = {{"workspace", opts->workspace, (size_t)need, true}, {"o", out->data, (size_t)numel(out) * 2, true}};
     if (int rc = check_aliasing(op, ws, 2)) return rc;
     for (int i = 0; i < 3; i++) {
@@ -583,9 +606,9 @@ void svodk_tune_streaming(int32_t workgroups_per_xcd) { svodk::attention_stream_
 // The workspace of a split call (tk/src/ops/attention.rs:285-293).
 int64_t svodk_attention_workspace(const svodk_tensor *q, const svodk_tensor *k, const svodk_attn *opts) {
   if (!well_formed(q) || !well_formed(k) || opts == nullptr || q->rank != 4 || k->rank != 4) return 0;
-  const int splits = split_count(opts->splits, k->shape[1]);
-  if (splits <= 1) return 0;
   const int64_t batch = opts->batch_live > 0 ? opts->batch_live : q->shape[0];
+  const int splits = split_count(opts, batch, q->shape[1], q->shape[2], k->shape[1]);
+  if (splits <= 1) return 0;
   return (int64_t)splits * batch * q->shape[1] * q->shape[2] * (q->shape[3] + 2) * 4;
 }
 

@@ -270,7 +270,7 @@ def _attn_options(opts: Attn, keep: list) -> _Attn:
 def _lend_workspace(lib, a: _Attn, qd: _Tensor, kd: _Tensor, device, workspace, keep: list) -> None:
     """The partial tensors of a split call, which the reference op allocates itself
     (tk/src/ops/attention.rs:285-293): here the harness does, like the output."""
-    if a.splits <= 1:
+    if a.splits == 1:
         return
     need = int(lib.svodk_attention_workspace(ctypes.byref(qd), ctypes.byref(kd), ctypes.byref(a)))
     if workspace is None and need > 0:

@@ -144,3 +144,23 @@ def test_packed_attention_is_the_split_call_bit_for_bit(device, b, t, h, hkv, d,
     assert np.array_equal(bits(packed), bits(split))
     p = oracle.AttnProblem(to_np(q), to_np(k), to_np(v), causal=causal, key_lens=None if lens is None else np.asarray(lens))
     assert max_abs(to_np(packed), oracle.attention_direct(p)) < 2e-2
+
+
+def test_a_decoder_step_is_split_unasked_when_the_workspace_is_lent(device):
+    """One query row against 8192 keys: with no count named the library splits the keys (and merges),
+    given the workspace it asks for; without one it keeps them whole.  Both agree with the direct softmax."""
+    b, t, tk, h, hkv, d = 1, 1, 8192, 8, 2, 64
+    g = Lcg(17)
+    q, k, v = g.bf16((b, t, h, d)), g.bf16((b, tk, hkv, d)), g.bf16((b, tk, hkv, d))
+    dq, dk, dv = (bf16_tensor(x, device) for x in (q, k, v))
+    want = oracle.attention_direct(oracle.AttnProblem(q, k, v))
+    split = svod_amd.attention(dq, dk, dv)  # the wrapper lends what svodk_attention_workspace asks for
+    assert "combine_splits" in svod_amd.chosen()
+    whole = svod_amd.attention(dq, dk, dv, workspace=torch.empty(16, dtype=torch.uint8, device=device))
+    assert "combine_splits" not in svod_amd.chosen() and "flash_attention" in svod_amd.chosen()
+    one = svod_amd.attention(dq, dk, dv, Attn(splits=1))
+    assert "combine_splits" not in svod_amd.chosen()
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(whole), bits(one))
+    for got in (split, whole):
+        assert max_abs(to_np(got), want) < 2e-2

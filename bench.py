@@ -47,6 +47,8 @@ def parse():
                     help="calls per step for the other workloads, rotating over 4 copies of the operands so that "
                          "none is served from the Infinity Cache")
     ap.add_argument("--no-graph", action="store_true", help="enqueue eagerly instead of replaying a HIP graph")
+    ap.add_argument("--no-row-order", action="store_true",
+                    help="bge_m3: take the batch rows as they come instead of ordering them by length once per step")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="rough budget of the CPU baseline sample")
     return ap.parse_args()
@@ -77,18 +79,27 @@ def main():
 
     # ---- build the step: a list of closures launching on the current stream.
     calls, flops_vis, flops_nom, bytes_min, kernel_name, bound = [], 0.0, 0.0, 0, "", "mfma"
+    extra_calls = []  # launches of a step that are not calls of the op being measured
     cpu_sample = None
     if args.workload in ("bge_m3", "bge_m3_bool"):
         sets = [W.config2(layer=l, device=dev) for l in range(args.layers)]
+        # The lengths belong to the batch, not to a layer (every set has the same ones): as a model would,
+        # the step orders the batch rows by length once (one small launch, inside the timed region) and
+        # hands the order to its 24 layer calls.  --no-row-order runs the rows as they come.
+        order = None
+        if args.workload == "bge_m3" and not args.no_row_order:
+            order = torch.empty(sets[0].key_lens.shape, dtype=torch.int32, device=dev)
+            extra_calls.append(lambda: svod_amd.order_rows(sets[0].key_lens, out=order))
         for w in sets:
             keys = KeyMask.lens(w.key_lens) if args.workload == "bge_m3" else KeyMask.bool(w.key_mask())
             out = torch.empty_like(w.q)
             calls.append((lambda w=w, keys=keys, out=out: svod_amd.attention(
-                w.q, w.k, w.v, Attn(keys=keys, scale=w.scale), out=out)))
+                w.q, w.k, w.v, Attn(keys=keys, scale=w.scale, row_order=order), out=out)))
         w0 = sets[0]
         flops_vis, flops_nom, bytes_min = w0.visible_flops(), w0.nominal_flops(), w0.min_bytes()
-        workload = "BGE-M3 encoder self-attention bf16 B32 H16 D64 S512 key-padding U[64,512], %d layer calls/step%s" % (
-            args.layers, " (KeyMask::Bool)" if args.workload == "bge_m3_bool" else " (KeyMask::Lens)")
+        workload = "BGE-M3 encoder self-attention bf16 B32 H16 D64 S512 key-padding U[64,512], %d layer calls/step%s%s" % (
+            args.layers, " (KeyMask::Bool)" if args.workload == "bge_m3_bool" else " (KeyMask::Lens)",
+            ", batch rows ordered by length once per step (svodk_order_rows, in the timed region)" if order is not None else "")
         cpu_sample = ("attention", w0)
         kernel_name = "flash_fwd_kernel<64>"
     elif args.workload == "hbm_copy":
@@ -150,6 +161,8 @@ def main():
         cpu_sample = ("attention", w)
 
     def step():
+        for c in extra_calls:
+            c()
         for c in calls:
             c()
 

@@ -25,6 +25,7 @@ from .ops import (  # noqa: F401
     layer_norm,
     library_path,
     load_library,
+    order_rows,
     plan_attention,
     plan_heads,
     plan_norm,

@@ -670,16 +670,16 @@ struct Ranges {
 template <int D, int NW, bool CAUSAL, bool SPLIT, bool RANGED, bool BIASED, bool CACHED, bool F16>
 __global__ __launch_bounds__(NW * 64, (D == 64 && !BIASED) ? 3 : 2) void flash_fwd_kernel(
     uint32_t unit_size, uint32_t unit_rcp, uint32_t nqt_u, uint32_t nqt_rcp, uint32_t kvh_u, uint32_t kvh_rcp,
-    uint32_t units, uint32_t heads_group, const void *__restrict__ key_lens, const uint16_t *__restrict__ q, int32_t t,
-    uint32_t tk_lens64, const uint16_t *__restrict__ k, const uint16_t *__restrict__ v,
-    uint16_t *__restrict__ o, const void *__restrict__ key_mask, int32_t mask_bytes, float scale, Splits sp,
-    int32_t q_row_elems, int32_t kv_row_elems, Ranges rg) {
+    uint32_t units, uint32_t heads_group, const void *__restrict__ key_lens, const int32_t *__restrict__ row_order,
+    int32_t t, uint32_t tk_lens64, const uint16_t *__restrict__ q, const uint16_t *__restrict__ k,
+    const uint16_t *__restrict__ v, uint16_t *__restrict__ o, const void *__restrict__ key_mask, int32_t mask_bytes,
+    float scale, Splits sp, int32_t q_row_elems, int32_t kv_row_elems, Ranges rg) {
   // The body is device code only: the host pass needs the kernel's handle, not its
   // instructions (and drops the whole instantiation over the LDS-fill instructions).
 #if defined(__HIP_DEVICE_COMPILE__)
   // The first 14 dwords of the arguments (up to tk_lens64) arrive in registers with the wave
   // (kernarg preload, scalars and pointers only): they are what the workgroup's coordinates,
-  // its length and the Q loads need, so none of those waits for an argument load.  Two of them
+  // its batch row and its length need, so none of those waits for an argument load.  Two of them
   // are packed to fit: heads | group << 16, and tk | (key_lens is 64-bit) << 31.
   const Geometry geo = {unit_size, unit_rcp, nqt_u, nqt_rcp, kvh_u, kvh_rcp, heads_group >> 16, units};
   const int heads = (int)(heads_group & 0xffffu);
@@ -706,9 +706,17 @@ __global__ __launch_bounds__(NW * 64, (D == 64 && !BIASED) ? 3 : 2) void flash_f
   const uint32_t within = local - round * geo.unit_size;
   const uint32_t head_in_group = div_by(within, geo.nqt, geo.nqt_rcp);
   const int order = (int)(within - head_in_group * geo.nqt);
-  const int b = (int)div_by(unit, geo.kv_heads, geo.kvh_rcp);
-  const int kvh = (int)(unit - (uint32_t)b * geo.kv_heads);  // L548: query head h reads KV head h / (heads / kv_heads)
+  const int b_place = (int)div_by(unit, geo.kv_heads, geo.kvh_rcp);
+  const int kvh = (int)(unit - (uint32_t)b_place * geo.kv_heads);  // L548: query head h reads KV head h / (heads / kv_heads)
   const int h = kvh * (int)geo.group + (int)head_in_group;
+  // Which batch row a workgroup takes is free (the reference's grid fixes what is computed, not
+  // when): with an order from the caller, place p of the launch works on row row_order[p], so
+  // that rows with more keys can go first and the launch ends on its short tiles.
+  int b = b_place;
+  if (row_order != nullptr) {
+    const int nbatch = (int)div_by(geo.units, geo.kv_heads, geo.kvh_rcp);
+    b = min(max(row_order[b_place], 0), nbatch - 1);
+  }
   // Grid x of the reference is order * splits + split (L523); geo.nqt counts those.
   int split = 0, tile = order, nqt = (int)geo.nqt;
   if (SPLIT) {
@@ -1425,7 +1433,7 @@ hipError_t launch(const AttnArgs &a, hipStream_t stream) {
   // It is never chosen unasked: measured, it has not beaten a workgroup per tile.
   if constexpr (D == 64 && !SPLIT && !RANGED && !BIASED && !CACHED) {
     const int knob = g_stream_slots.load(std::memory_order_relaxed);
-    if (knob > 0 && a.key_mask == nullptr)
+    if (knob > 0 && a.key_mask == nullptr && a.row_order == nullptr)
       return launch_stream<D, NW, CAUSAL, F16>(a, stream, knob, geo, q_row, kv_row);
   }
   const uint32_t heads_group = (uint32_t)a.heads | geo.group << 16;
@@ -1459,7 +1467,7 @@ hipError_t launch(const AttnArgs &a, hipStream_t stream) {
   rg.app_lens_i64 = a.app_lens_i64;
   hipLaunchKernelGGL(kernel, dim3((uint32_t)grid), dim3(NW * 64), smem, stream, geo.unit_size, geo.unit_rcp, geo.nqt,
                      geo.nqt_rcp, geo.kv_heads, geo.kvh_rcp, geo.units, heads_group, a.key_lens,
-                     (const uint16_t *)a.q, a.t, tk_lens64, (const uint16_t *)a.k,
+                     (const int32_t *)a.row_order, a.t, tk_lens64, (const uint16_t *)a.q, (const uint16_t *)a.k,
                      (const uint16_t *)a.v, (uint16_t *)a.o, a.key_mask, a.mask_bytes, a.scale, sp, (int32_t)q_row,
                      (int32_t)kv_row, rg);
   return hipGetLastError();
@@ -1492,7 +1500,35 @@ hipError_t launch_d(const AttnArgs &a, hipStream_t stream) {
   return a.f16 ? launch_t<D, true>(a, stream) : launch_t<D, false>(a, stream);
 }
 
+// The batch rows in descending order of their key lengths, ties by row: order[p] = the row with
+// the p-th most keys.  One workgroup; a thread ranks its rows against all of them in LDS.
+__global__ __launch_bounds__(256) void order_rows_kernel(const void *__restrict__ key_lens, int32_t lens_i64, int32_t n,
+                                                         int32_t *__restrict__ order) {
+  extern __shared__ int32_t lens_sh[];
+  for (int i = threadIdx.x; i < n; i += 256) {
+    const long long x = lens_i64 ? ((const long long *)key_lens)[i] : (long long)((const int *)key_lens)[i];
+    lens_sh[i] = (int32_t)(x < 0 ? 0 : (x > 0x7fffffffLL ? 0x7fffffffLL : x));
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < n; i += 256) {
+    const int32_t mine = lens_sh[i];
+    int ahead = 0;
+    for (int j = 0; j < n; j++) {
+      const int32_t other = lens_sh[j];
+      ahead += (other > mine || (other == mine && j < i)) ? 1 : 0;
+    }
+    order[ahead] = i;
+  }
+}
+
 }  // namespace
+
+hipError_t launch_order_rows(const void *key_lens, int32_t lens_i64, int32_t n, int32_t *order, hipStream_t stream) {
+  if (n <= 0) return hipSuccess;
+  if (n > kMaxOrderedRows) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(order_rows_kernel, dim3(1), dim3(256), (size_t)n * 4, stream, key_lens, lens_i64, n, order);
+  return hipGetLastError();
+}
 
 bool attention_supports(int32_t d) { return d == 64 || d == 128; }
 

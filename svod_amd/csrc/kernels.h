@@ -52,6 +52,9 @@ struct AttnArgs {
   const void *key_lens;  // [batch] i32/i64 or null
   const void *key_mask;  // [batch, tk] u8/i32 or null
   int32_t lens_i64;      // key_lens holds 64-bit integers
+  // [batch] i32 or null: place p of the launch works on batch row row_order[p] (a permutation;
+  // out-of-range entries are clamped).  Results do not depend on it; the order of work does.
+  const void *row_order;
   int32_t mask_bytes;    // element size of key_mask: 1 or 4
   int32_t batch;         // live batches
   int32_t t, tk, heads, kv_heads, d;
@@ -106,6 +109,9 @@ struct CombineArgs {
 };
 hipError_t launch_combine(const CombineArgs &a, hipStream_t stream);
 bool attention_supports(int32_t d);
+// order[p] = the batch row with the p-th most keys (ties by row), for AttnArgs::row_order.
+constexpr int32_t kMaxOrderedRows = 8192;
+hipError_t launch_order_rows(const void *key_lens, int32_t lens_i64, int32_t n, int32_t *order, hipStream_t stream);
 // Tuning of the streaming form (workgroups that walk runs of query tiles): see svodk_tune_streaming.
 void attention_stream_slots(int32_t slots);
 // Text of the tile configuration launch_attention picks for `a` (for chosen()).

@@ -498,6 +498,20 @@ static int attend(const svodk_tensor *q, const svodk_tensor *k, const svodk_tens
     a.seg_start = opts->seg_start->data;
     a.seg_i64 = opts->seg_start->dtype == SVODK_I64;
   }
+  if (opts->row_order != nullptr) {
+    const svodk_tensor *ro = opts->row_order;
+    if (!well_formed(ro)) return fail(SVODK_ERR_ARGUMENT, "%s: row order descriptor malformed", op);
+    if (!(ro->rank == 1 && ro->shape[0] == q->shape[0]))
+      return fail(SVODK_ERR_SHAPE, "%s: row order has shape %s, expected [%lld]", op, fmt_shape(ro).c_str(),
+                  (long long)q->shape[0]);
+    if (ro->dtype != SVODK_I32)
+      return fail(SVODK_ERR_DTYPE, "%s: row order is %s, the input is Int32", op, dtype_name(ro->dtype));
+    if (ro->data == nullptr) return fail(SVODK_ERR_ARGUMENT, "%s: a null device pointer", op);
+    Span pair[2] = {{"row_order", ro->data, (size_t)numel(ro) * 4, false}, spans[3]};
+    if (int rc = check_aliasing(op, pair, 2)) return rc;
+    // Under a bound batch the order must name live rows only: an order of the whole capacity does not.
+    if (a.batch == cap) a.row_order = ro->data;
+  }
   if (packed != nullptr) a.q_row_elems = a.kv_row_elems = (heads + 2 * kv_heads) * d;
   if (cache != nullptr) {
     a.cached = 1;
@@ -604,6 +618,31 @@ int svodk_attention_packed(const svodk_tensor *qkv, int32_t heads, int32_t kv_he
 void svodk_tune_streaming(int32_t workgroups_per_xcd) { svodk::attention_stream_slots(workgroups_per_xcd); }
 
 // The workspace of a split call (tk/src/ops/attention.rs:285-293).
+int svodk_order_rows(const svodk_tensor *key_lens, const svodk_tensor *order, void *hip_stream) {
+  const char *op = "order_rows";
+  if (!well_formed(key_lens) || !well_formed(order))
+    return fail(SVODK_ERR_ARGUMENT, "%s: a null or malformed tensor descriptor", op);
+  if (!(key_lens->rank == 1 && order->rank == 1 && order->shape[0] == key_lens->shape[0]))
+    return fail(SVODK_ERR_SHAPE, "%s: key lens %s and order %s, expected [B] and [B]", op, fmt_shape(key_lens).c_str(),
+                fmt_shape(order).c_str());
+  if (!is_int(key_lens->dtype))
+    return fail(SVODK_ERR_DTYPE, "%s: key lens is %s, the input is an integer type", op, dtype_name(key_lens->dtype));
+  if (order->dtype != SVODK_I32)
+    return fail(SVODK_ERR_DTYPE, "%s: order is %s, the output is Int32", op, dtype_name(order->dtype));
+  if (key_lens->shape[0] > svodk::kMaxOrderedRows)
+    return fail(SVODK_ERR_SHAPE, "%s: %lld rows, at most %d", op, (long long)key_lens->shape[0], svodk::kMaxOrderedRows);
+  if (!current_device_has_kernels()) return ran_graph(op, SVODK_GRAPH_TARGET);
+  if (key_lens->data == nullptr || order->data == nullptr) return fail(SVODK_ERR_ARGUMENT, "%s: a null device pointer", op);
+  Span spans[2] = {{"key_lens", key_lens->data, (size_t)numel(key_lens) * dtype_bytes(key_lens->dtype), false},
+                   {"order", order->data, (size_t)numel(order) * 4, true}};
+  if (int rc = check_aliasing(op, spans, 2)) return rc;
+  ran(op, "order_rows", "one workgroup");
+  const hipError_t e = svodk::launch_order_rows(key_lens->data, key_lens->dtype == SVODK_I64, (int32_t)key_lens->shape[0],
+                                                (int32_t *)order->data, (hipStream_t)hip_stream);
+  if (e != hipSuccess) return fail(SVODK_ERR_LAUNCH, "%s: %s", op, hipGetErrorString(e));
+  return SVODK_KERNEL;
+}
+
 int64_t svodk_attention_workspace(const svodk_tensor *q, const svodk_tensor *k, const svodk_attn *opts) {
   if (!well_formed(q) || !well_formed(k) || opts == nullptr || q->rank != 4 || k->rank != 4) return 0;
   const int64_t batch = opts->batch_live > 0 ? opts->batch_live : q->shape[0];

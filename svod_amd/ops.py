@@ -47,6 +47,7 @@ class _Attn(ctypes.Structure):
         ("seg_start", ctypes.POINTER(_Tensor)), ("cache", ctypes.POINTER(_Cache)), ("bias", ctypes.POINTER(_Tensor)),
         ("splits", ctypes.c_int32), ("has_scale", ctypes.c_int32), ("scale", ctypes.c_float),
         ("batch_live", ctypes.c_int32), ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_int64),
+        ("row_order", ctypes.POINTER(_Tensor)),
     ]
 
 
@@ -95,6 +96,8 @@ def load_library() -> ctypes.CDLL:
         fn.argtypes = [tp] * n_tensors_before_eps + [ctypes.c_double, ctypes.c_int32] + [tp] * n_outputs + [ctypes.c_void_p]
     lib.svodk_plan_norm.restype = ctypes.c_int
     lib.svodk_plan_norm.argtypes = [ctypes.c_int32, i32p, ctypes.c_int32, i64p, ctypes.c_int32]
+    lib.svodk_order_rows.restype = ctypes.c_int
+    lib.svodk_order_rows.argtypes = [tp, tp, ctypes.c_void_p]
     lib.svodk_tune_streaming.restype = None
     lib.svodk_tune_streaming.argtypes = [ctypes.c_int32]
     lib.svodk_supported.restype = ctypes.c_int
@@ -222,6 +225,7 @@ class Attn:
     scale: Optional[float] = None
     bias: Optional[torch.Tensor] = None
     batch_live: Optional[int] = None
+    row_order: Optional[torch.Tensor] = None  # [B] int32 from ``order_rows``: not in the reference's Attn
 
 
 @dataclass
@@ -264,6 +268,7 @@ def _attn_options(opts: Attn, keep: list) -> _Attn:
     if opts.scale is not None:
         a.has_scale, a.scale = 1, float(opts.scale)
     a.batch_live = opts.batch_live or 0
+    a.row_order = _ref(keep, opts.row_order)
     return a
 
 
@@ -412,6 +417,18 @@ def plan_norm(has_target: bool, dtypes, x_dims) -> Optional[Fallback]:
     dt = (ctypes.c_int32 * len(dtypes))(*[_DTYPES[d] for d in dtypes])
     xd = None if x_dims is None else (ctypes.c_int64 * len(x_dims))(*x_dims)
     return _plan(lib.svodk_plan_norm(int(has_target), dt, len(dtypes), xd, 0 if x_dims is None else len(x_dims)))
+
+
+def order_rows(key_lens: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The batch rows in descending order of their key lengths (ties by row) as int32 ``[B]``, for
+    ``Attn.row_order``: a variable-length batch that runs its long rows first ends on its short tiles."""
+    lib = load_library()
+    if out is None:
+        out = torch.empty(key_lens.shape, dtype=torch.int32, device=key_lens.device)
+    keep: list = []
+    status = lib.svodk_order_rows(_ref(keep, key_lens), _ref(keep, out), ctypes.c_void_p(_stream(key_lens)))
+    _finish("order_rows", status)
+    return out
 
 
 def chosen() -> str:

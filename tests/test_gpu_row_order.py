@@ -1,0 +1,56 @@
+"""The batch row order of a launch (svodk_attn.row_order, svodk_order_rows): which row a workgroup takes
+is free, so any permutation gives the same bits; the one svodk_order_rows computes is the rows in
+descending order of their key lengths, ties by row."""
+import numpy as np
+import pytest
+import torch
+
+import svod_amd
+from svod_amd import Attn, KeyMask
+from util import Lcg, bf16_tensor, bits
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("n,dtype", [(1, torch.int32), (5, torch.int64), (64, torch.int32), (300, torch.int32),
+                                     (1500, torch.int64)])
+def test_order_rows_is_a_stable_descending_sort(device, n, dtype):
+    rng = np.random.default_rng(n)
+    lens = rng.integers(0, 40, size=n)  # many ties
+    got = svod_amd.order_rows(torch.from_numpy(lens).to(dtype).to(device)).cpu().numpy()
+    want = np.argsort(-lens, kind="stable")
+    assert np.array_equal(got, want)
+    assert svod_amd.chosen().startswith('Kernel { op: "order_rows"')
+
+
+# (b, t, tk, h, hkv, d, causal, splits)
+CASES = [(12, 300, 300, 4, 2, 64, False, None), (7, 200, 260, 4, 4, 128, True, None), (5, 130, 512, 2, 2, 64, False, 2)]
+
+
+@pytest.mark.parametrize("b,t,tk,h,hkv,d,causal,splits", CASES)
+def test_any_row_order_gives_the_same_bits(device, b, t, tk, h, hkv, d, causal, splits):
+    g = Lcg(21)
+    q, k, v = (bf16_tensor(x, device) for x in (g.bf16((b, t, h, d)), g.bf16((b, tk, hkv, d)), g.bf16((b, tk, hkv, d))))
+    lens = torch.tensor([(37 * i) % (tk + 1) for i in range(b)], dtype=torch.int32, device=device)
+    opts = dict(causal=causal, keys=KeyMask.lens(lens), splits=splits)
+    plain = bits(svod_amd.attention(q, k, v, Attn(**opts)))
+    longest_first = svod_amd.order_rows(lens)
+    assert np.array_equal(bits(svod_amd.attention(q, k, v, Attn(row_order=longest_first, **opts))), plain)
+    backwards = torch.arange(b - 1, -1, -1, dtype=torch.int32, device=device)
+    assert np.array_equal(bits(svod_amd.attention(q, k, v, Attn(row_order=backwards, **opts))), plain)
+
+
+def test_a_row_order_is_validated(device):
+    g = Lcg(2)
+    q, k = bf16_tensor(g.bf16((3, 64, 2, 64)), device), bf16_tensor(g.bf16((3, 64, 2, 64)), device)
+    with pytest.raises(svod_amd.OpError) as e:
+        svod_amd.attention(q, k, k, Attn(row_order=torch.zeros(4, dtype=torch.int32, device=device)))
+    assert e.value.kind == "Shape" and "row order" in str(e.value)
+    with pytest.raises(svod_amd.OpError) as e:
+        svod_amd.attention(q, k, k, Attn(row_order=torch.zeros(3, dtype=torch.int64, device=device)))
+    assert e.value.kind == "Dtype"
+    # Entries out of range are clamped, never followed out of the tensors.
+    wild = torch.tensor([-5, 1, 99], dtype=torch.int32, device=device)
+    out = svod_amd.attention(q, k, k, Attn(row_order=wild))
+    torch.cuda.synchronize()
+    assert out.shape == q.shape

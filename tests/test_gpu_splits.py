@@ -4,8 +4,8 @@
 Cases follow the reference's split tests in spirit (tk/src/test/unit/attention.rs:397-412,
 tk/src/test/unit/ops.rs:585-628): several split counts, more splits than a row has blocks, a
 lane with no keys, a negative scale's partial maxima, d 128.  The reference exercises splits
-through its cache mode, which this library has no kernel for; here the same split and merge run
-on plain calls."""
+through its cache mode (tests/test_gpu_cache.py holds those cases); here the same split and merge
+run on plain calls."""
 import numpy as np
 import pytest
 import torch

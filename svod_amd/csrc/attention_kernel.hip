@@ -667,7 +667,10 @@ struct Ranges {
   int32_t app_lens_i64;
 };
 
-template <int D, int NW, bool CAUSAL, bool SPLIT, bool RANGED, bool BIASED, bool CACHED, bool F16>
+// GROUPED: the query tile's rows are (head of the KV head's group, query) pairs instead of 128
+// queries of one head, for calls whose whole group fits a tile (a decoder step: heads / kv_heads
+// * T <= 128).  The group's heads then share one pass over their K and V instead of one each.
+template <int D, int NW, bool CAUSAL, bool SPLIT, bool RANGED, bool BIASED, bool CACHED, bool GROUPED, bool F16>
 __global__ __launch_bounds__(NW * 64, (D == 64 && !BIASED) ? 3 : 2) void flash_fwd_kernel(
     uint32_t unit_size, uint32_t unit_rcp, uint32_t nqt_u, uint32_t nqt_rcp, uint32_t kvh_u, uint32_t kvh_rcp,
     uint32_t units, uint32_t heads_group, const void *__restrict__ key_lens, const int32_t *__restrict__ row_order,
@@ -748,13 +751,23 @@ __global__ __launch_bounds__(NW * 64, (D == 64 && !BIASED) ? 3 : 2) void flash_f
   const int64_t q_row_stride = q_row_elems;
   const int64_t o_row_stride = (int64_t)heads * D;
   // ---- Q fragments: B operand of the score product, resident for the block.
-  const int row = q_off + w.wave * kWaveRows + ln;  // this lane's query
+  const int row = q_off + w.wave * kWaveRows + ln;  // this lane's row of the tile
+  static_assert(!GROUPED || (!CAUSAL && !RANGED), "grouped tiles take no per-row masks");
+  // This lane's query: row q_row of head q_head, when there is one.
+  int q_row = row, q_head = h;
+  bool q_ok = row < t;
+  if (GROUPED) {
+    const int in_group = row / t;
+    q_row = row - in_group * t;
+    q_ok = in_group < (int)geo.group;
+    q_head = kvh * (int)geo.group + min(in_group, (int)geo.group - 1);
+  }
   {
-    const uint16_t *q_ptr = q + ((int64_t)b * t + row) * q_row_stride + (int64_t)h * D + w.g * 8;
+    const uint16_t *q_ptr = q + ((int64_t)b * t + q_row) * q_row_stride + (int64_t)q_head * D + w.g * 8;
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
       u32x4 x = {0, 0, 0, 0};
-      if (row < t) x = *reinterpret_cast<const u32x4 *>(q_ptr + ks * 16);
+      if (q_ok) x = *reinterpret_cast<const u32x4 *>(q_ptr + ks * 16);
       w.qf[ks] = x;
     }
   }
@@ -819,10 +832,10 @@ __global__ __launch_bounds__(NW * 64, (D == 64 && !BIASED) ? 3 : 2) void flash_f
   w.mask_bytes = mask_bytes;
   w.wave_first_row = q_off + w.wave * kWaveRows - first_key;
   w.my_row = w.wave_first_row + ln;
-  w.my_row_ok = row < t;
+  w.my_row_ok = q_ok;
   if (BIASED) {
     // L566-571: the bias of this (batch or 0, head), this lane's row, from the tile's first key on.
-    const int64_t brow = ((int64_t)(rg.bias_per_batch ? b : 0) * heads + h) * t + min(row, t - 1);
+    const int64_t brow = ((int64_t)(rg.bias_per_batch ? b : 0) * heads + q_head) * t + min(q_row, t - 1);
     w.bias_row = rg.bias + brow * rg.bias_cols + first_key;
     w.bias_keys = rg.bias_cols - first_key;
   }
@@ -915,7 +928,7 @@ __global__ __launch_bounds__(NW * 64, (D == 64 && !BIASED) ? 3 : 2) void flash_f
   for (int i = 0; i < 32; i++) sv[i] = nv[i] = 0.0f;
   if (my_end > 0) {
     uint32_t bw[16];
-    if (BIASED) load_bias<D, NW>(w, 0, row < t, bw);
+    if (BIASED) load_bias<D, NW>(w, 0, q_ok, bw);
     scores<D, NW>(w, smem, 0, sv);
     if (!w.positive) {
 #pragma unroll
@@ -977,7 +990,7 @@ __global__ __launch_bounds__(NW * 64, (D == 64 && !BIASED) ? 3 : 2) void flash_f
         fill_tile<D, NW>(w, (const uint8_t *)(rg.v_app + at), bytes, 0, w.lds0 + 2 * TL::kBytes, v_src, app_row_bytes);
       }
       uint32_t bw[16];
-      if (BIASED) load_bias<D, NW>(w, tk - first_key, row < t, bw);  // their columns come last (L84-85)
+      if (BIASED) load_bias<D, NW>(w, tk - first_key, q_ok, bw);  // their columns come last (L84-85)
       __builtin_amdgcn_s_waitcnt(0x0f70);
       __syncthreads();
       scores<D, NW>(w, smem, 0, sv);
@@ -1007,8 +1020,8 @@ __global__ __launch_bounds__(NW * 64, (D == 64 && !BIASED) ? 3 : 2) void flash_f
   if (SPLIT) {
     // ---- the split's partial state (L899-921): the accumulator as it stands, the maximum in
     // the exponent's units (L848-853) and the sum.
-    if (row < t) {
-      const int64_t at = (((int64_t)split * sp.nbatch + b) * t + row) * heads + h;
+    if (q_ok) {
+      const int64_t at = (((int64_t)split * sp.nbatch + b) * t + q_row) * heads + q_head;
       if (w.g == 0) {
         sp.m_part[at] = w.positive ? w.m_run * w.c_exp : w.m_run;
         sp.l_part[at] = l_tot;
@@ -1027,8 +1040,8 @@ __global__ __launch_bounds__(NW * 64, (D == 64 && !BIASED) ? 3 : 2) void flash_f
   }
   // ---- out = o / (l == 0 ? 1 : l), bounded store (L892-898, L974-980).
   const float inv = 1.0f / (l_tot == 0.0f ? 1.0f : l_tot);
-  if (row < t) {
-    uint16_t *o_ptr = o + ((int64_t)b * t + row) * o_row_stride + (int64_t)h * D + 4 * w.g;
+  if (q_ok) {
+    uint16_t *o_ptr = o + ((int64_t)b * t + q_row) * o_row_stride + (int64_t)q_head * D + 4 * w.g;
 #pragma unroll
     for (int db = 0; db < DB; db++) {
 #pragma unroll
@@ -1384,12 +1397,13 @@ hipError_t launch_stream(const AttnArgs &a, hipStream_t stream, int64_t slots, c
   return hipGetLastError();
 }
 
-template <int D, int NW, bool CAUSAL, bool SPLIT, bool RANGED, bool BIASED, bool CACHED, bool F16>
+template <int D, int NW, bool CAUSAL, bool SPLIT, bool RANGED, bool BIASED, bool CACHED, bool GROUPED, bool F16>
 hipError_t launch(const AttnArgs &a, hipStream_t stream) {
   using TL = Tile<D>;
   constexpr int BQ = NW * kWaveRows;
   const int splits = SPLIT ? a.splits : 1;
-  const int nqt = (a.t + BQ - 1) / BQ * splits;  // grid x: query tile * splits + split (L512, L523)
+  // grid x: query tile * splits + split (L512, L523); a grouped call has one tile a KV head.
+  const int nqt = (GROUPED ? 1 : (a.t + BQ - 1) / BQ) * splits;
   const int64_t blocks = (int64_t)nqt * a.heads * a.batch;
   if (blocks == 0) return hipSuccess;
   if (blocks > 0x7ffffff0LL) return hipErrorInvalidConfiguration;
@@ -1398,7 +1412,7 @@ hipError_t launch(const AttnArgs &a, hipStream_t stream) {
   const int64_t kv_row = a.kv_row_elems > 0 ? a.kv_row_elems : (int64_t)a.kv_heads * a.d;
   // The fills address a (batch, kv head)'s rows with 32-bit byte offsets.
   if ((int64_t)a.tk * kv_row * 2 > 0x7fffffffLL || q_row > 0x7fffffffLL) return hipErrorInvalidValue;
-  auto kernel = flash_fwd_kernel<D, NW, CAUSAL, SPLIT, RANGED, BIASED, CACHED, F16>;
+  auto kernel = flash_fwd_kernel<D, NW, CAUSAL, SPLIT, RANGED, BIASED, CACHED, GROUPED, F16>;
   // The LDS ring is above the default limit of a launch: one attribute call per instantiation
   // and device, from whichever thread gets there first (a second call is harmless).
   static std::atomic<uint64_t> configured{0};  // a bit per device ordinal, devices past 63 always ask
@@ -1413,7 +1427,7 @@ hipError_t launch(const AttnArgs &a, hipStream_t stream) {
   }
   // Units of work (batch, KV head) are dealt over the XCDs in whole rounds; the workgroups of
   // a round's missing units exit at once.
-  const int64_t unit_size = (int64_t)(a.heads / a.kv_heads) * nqt;
+  const int64_t unit_size = (int64_t)(GROUPED ? 1 : a.heads / a.kv_heads) * nqt;
   const int64_t units = (int64_t)a.kv_heads * a.batch;
   const int64_t grid = (units + kXcds - 1) / kXcds * kXcds * unit_size;
   if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
@@ -1431,7 +1445,7 @@ hipError_t launch(const AttnArgs &a, hipStream_t stream) {
   // The streaming form, where asked for and where it has a kernel (head size 64, lengths or no
   // key mask, no window, no splits): `knob` workgroups per XCD, each walking its run of tiles.
   // It is never chosen unasked: measured, it has not beaten a workgroup per tile.
-  if constexpr (D == 64 && !SPLIT && !RANGED && !BIASED && !CACHED) {
+  if constexpr (D == 64 && !SPLIT && !RANGED && !BIASED && !CACHED && !GROUPED) {
     const int knob = g_stream_slots.load(std::memory_order_relaxed);
     if (knob > 0 && a.key_mask == nullptr && a.row_order == nullptr)
       return launch_stream<D, NW, CAUSAL, F16>(a, stream, knob, geo, q_row, kv_row);
@@ -1475,11 +1489,17 @@ hipError_t launch(const AttnArgs &a, hipStream_t stream) {
 
 template <int D, bool RANGED, bool BIASED, bool CACHED, bool F16>
 hipError_t launch_s(const AttnArgs &a, hipStream_t stream) {
+  if constexpr (!RANGED) {
+    if (attention_groups(a)) {
+      return a.splits > 1 ? launch<D, 4, false, true, false, BIASED, CACHED, true, F16>(a, stream)
+                          : launch<D, 4, false, false, false, BIASED, CACHED, true, F16>(a, stream);
+    }
+  }
   if (a.splits > 1)
-    return a.causal ? launch<D, 4, true, true, RANGED, BIASED, CACHED, F16>(a, stream)
-                    : launch<D, 4, false, true, RANGED, BIASED, CACHED, F16>(a, stream);
-  return a.causal ? launch<D, 4, true, false, RANGED, BIASED, CACHED, F16>(a, stream)
-                  : launch<D, 4, false, false, RANGED, BIASED, CACHED, F16>(a, stream);
+    return a.causal ? launch<D, 4, true, true, RANGED, BIASED, CACHED, false, F16>(a, stream)
+                    : launch<D, 4, false, true, RANGED, BIASED, CACHED, false, F16>(a, stream);
+  return a.causal ? launch<D, 4, true, false, RANGED, BIASED, CACHED, false, F16>(a, stream)
+                  : launch<D, 4, false, false, RANGED, BIASED, CACHED, false, F16>(a, stream);
 }
 
 template <int D, bool F16>
@@ -1531,6 +1551,12 @@ hipError_t launch_order_rows(const void *key_lens, int32_t lens_i64, int32_t n, 
 }
 
 bool attention_supports(int32_t d) { return d == 64 || d == 128; }
+
+bool attention_groups(const AttnArgs &a) {
+  const bool ranged = a.win_left >= 0 || a.chunk_size > 0 || a.seg_start != nullptr;
+  const int64_t group = a.kv_heads > 0 ? a.heads / a.kv_heads : 1;
+  return group > 1 && !a.causal && !ranged && group * a.t <= 128;
+}
 
 void attention_stream_slots(int32_t slots) { g_stream_slots.store(slots, std::memory_order_relaxed); }
 

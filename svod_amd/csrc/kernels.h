@@ -109,6 +109,9 @@ struct CombineArgs {
 };
 hipError_t launch_combine(const CombineArgs &a, hipStream_t stream);
 bool attention_supports(int32_t d);
+// Whether launch_attention runs `a` on grouped tiles: the heads of a KV head's group side by side
+// in one query tile (a decoder step under GQA: no causal or per-row mask, group * t <= 128).
+bool attention_groups(const AttnArgs &a);
 // order[p] = the batch row with the p-th most keys (ties by row), for AttnArgs::row_order.
 constexpr int32_t kMaxOrderedRows = 8192;
 hipError_t launch_order_rows(const void *key_lens, int32_t lens_i64, int32_t n, int32_t *order, hipStream_t stream);

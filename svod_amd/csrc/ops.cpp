@@ -262,13 +262,16 @@ int svodk_plan_heads(int32_t has_target, const int32_t *dtypes, int32_t n_dtypes
 // 151.5 -> 29.8 (16), 64 x 32 28.7 -> 16.8 (4), 64 x 64 82.7 -> 37.6 (8), 256 x 64 86.2 -> 67.4
 // (2), 320 x 24 32.7 -> 28.6 (2); from 640 workgroups on the rule answers one, which is fastest.
 // A window, a chunk mask or segment starts leave a tile few of the keys: the rule keeps those whole.
-static int split_count(const svodk_attn *opts, int64_t batch, int64_t t, int64_t heads, int64_t tk) {
+static int split_count(const svodk_attn *opts, int64_t batch, int64_t t, int64_t heads, int64_t kv_heads, int64_t tk) {
   const int32_t asked = opts->splits;
   const int64_t most = tk > 0 ? (tk + 63) / 64 : 1;
   if (asked == 1) return 1;
   if (asked > 1) return (int)(asked < most ? asked : most);
   if (opts->has_window || opts->has_chunk || opts->seg_start != nullptr) return 1;
-  const int64_t workgroups = (t + 127) / 128 * heads * batch;
+  // A decoder step under GQA runs a KV head's whole group in one tile (svodk::attention_groups).
+  const int64_t group = kv_heads > 0 ? heads / kv_heads : 1;
+  const bool grouped = group > 1 && !opts->causal && group * t <= 128;
+  const int64_t workgroups = grouped ? kv_heads * batch : (t + 127) / 128 * heads * batch;
   if (workgroups <= 0) return 1;
   const int64_t wanted = (512 + workgroups / 2) / workgroups;  // rounded
   const int64_t fits = most / 8;
@@ -541,7 +544,7 @@ static int attend(const svodk_tensor *q, const svodk_tensor *k, const svodk_tens
     }
   }
   // L280-302: key splits.  The partial tensors live in the caller's workspace.
-  a.splits = split_count(opts, a.batch, t, heads, tk);
+  a.splits = split_count(opts, a.batch, t, heads, kv_heads, tk);
   if (a.splits > 1) {
     const int64_t rows = (int64_t)a.batch * t * heads;
     int64_t need = (int64_t)a.splits * rows * (d + 2) * 4;
@@ -646,7 +649,8 @@ int svodk_order_rows(const svodk_tensor *key_lens, const svodk_tensor *order, vo
 int64_t svodk_attention_workspace(const svodk_tensor *q, const svodk_tensor *k, const svodk_attn *opts) {
   if (!well_formed(q) || !well_formed(k) || opts == nullptr || q->rank != 4 || k->rank != 4) return 0;
   const int64_t batch = opts->batch_live > 0 ? opts->batch_live : q->shape[0];
-  const int splits = split_count(opts, batch, q->shape[1], q->shape[2], k->shape[1]);
+  const int64_t kv_heads = opts->cache != nullptr ? opts->cache->kv_heads : k->shape[2];
+  const int splits = split_count(opts, batch, q->shape[1], q->shape[2], kv_heads, k->shape[1]);
   if (splits <= 1) return 0;
   return (int64_t)splits * batch * q->shape[1] * q->shape[2] * (q->shape[3] + 2) * 4;
 }

@@ -52,7 +52,8 @@ def test_grouped_tiles_match_repeated_kv_heads_bit_for_bit(device, name, b, t, t
     assert max_abs(to_np(grouped), want) < 2e-2
 
 
-def test_a_grouped_decoder_step_over_a_cache_with_appended_rows(device):
+@pytest.mark.parametrize("splits", [None, 2, 5])
+def test_a_grouped_decoder_step_over_a_cache_with_appended_rows(device, splits):
     b, rows, layers, t, d, h, hkv, tk, n = 4, 2, 2, 1, 64, 8, 2, 700, 1
     g = Lcg(9)
     q = g.bf16((b, t, h, d))
@@ -61,7 +62,7 @@ def test_a_grouped_decoder_step_over_a_cache_with_appended_rows(device):
     lens, row_map = np.array([700, 1, 333, 0]), np.array([1, 0, 0, 1])
     dev = lambda x: bf16_tensor(x, device)
     ints = lambda a: torch.tensor(a, dtype=torch.int32, device=device)
-    got = svod_amd.attention(dev(q), dev(k), dev(v), Attn(keys=KeyMask.lens(ints(lens)),
+    got = svod_amd.attention(dev(q), dev(k), dev(v), Attn(keys=KeyMask.lens(ints(lens)), splits=splits,
                              cache=Cache(hkv, hkv, ints(row_map), (dev(k_app), dev(v_app)))))
     torch.cuda.synchronize()
     p = oracle.AttnProblem(q, k, v, key_lens=lens, cache=oracle.Cache(hkv, hkv, row_map, (k_app, v_app)))

@@ -29,7 +29,8 @@ HBM_PEAK_GBS = 8000.0
 # this file, each scaled by what the counter reads for a 256 MiB device copy (x2.000 and x1.000);
 # the summaries are under profiles/.  Counters cannot be read from inside a timed run.
 HBM_TRAFFIC_BYTES = {"bge_m3": 110.31e6, "qwen3_attention": 176.79e6, "qwen3_prologue": 269.01e6,
-                     "qwen3_add_rms_norm": 268.56e6, "whisper": 245.96e6, "long": 127.65e6}
+                     "qwen3_add_rms_norm": 268.56e6, "whisper": 245.96e6, "whisper_decode": 127.19e6,
+                     "long": 127.65e6}
 
 
 def parse():
@@ -39,7 +40,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="bge_m3",
                     choices=["bge_m3", "bge_m3_bool", "qwen3_attention", "qwen3_prologue", "qwen3_add_rms_norm",
-                             "whisper", "long", "hbm_copy"],
+                             "whisper", "whisper_decode", "long", "hbm_copy"],
                     help="hbm_copy is a plain 256 MiB device copy: the known-size kernel the HBM counters "
                          "(FETCH_SIZE, WRITE_SIZE) are calibrated on")
     ap.add_argument("--layers", type=int, default=24, help="calls per step for the bge_m3 workloads")
@@ -122,6 +123,26 @@ def main():
         workload = "Qwen3-Embedding prologue bf16 qkv[8,2048,4096] -> q,k,v (RMSNorm eps 1e-6 + RoPE theta 1e6)"
         cpu_sample = ("heads", p)
         kernel_name, bound = "heads_kernel<128>", "hbm"
+    elif args.workload == "whisper_decode":
+        # One decoder step of Whisper-large-v3's cross-attention (model/src/whisper/decoder.rs:441-477): a query
+        # per lane against the 1500 encoder keys of its layer, read from a cache that holds every layer's heads.
+        from svod_amd import Cache
+        g = torch.Generator(device=dev).manual_seed(0x5EED0040)
+        b, tk, h, d, layers = 16, 1500, 20, 64, 32
+        k_cache = torch.randn((b, tk, layers * h, d), generator=g, device=dev).to(torch.bfloat16)
+        v_cache = torch.randn((b, tk, layers * h, d), generator=g, device=dev).to(torch.bfloat16)
+        qs = [torch.randn((b, 1, h, d), generator=g, device=dev).to(torch.bfloat16) for _ in range(layers)]
+        outs = [torch.empty_like(qs[0]) for _ in range(layers)]
+        lens = torch.full((b,), tk, dtype=torch.int32, device=dev)
+        ws = torch.empty(8 * b * h * (d + 2) * 4, dtype=torch.uint8, device=dev)
+        for layer in range(layers):
+            calls.append(lambda layer=layer: svod_amd.attention(
+                qs[layer], k_cache, v_cache, Attn(keys=KeyMask.lens(lens), cache=Cache(layer * h, h)), out=outs[layer],
+                workspace=ws))
+        bytes_min = 2 * b * tk * h * d * 2 + 2 * b * h * d * 2  # the layer's K and V heads read once, q and o
+        workload = ("Whisper-large-v3 decoder step, cross-attention bf16 B16 T1 H20 D64 over 1500 cached keys, "
+                    "32 layer calls/step on one cache [16,1500,640,64] (splits chosen by the library)")
+        kernel_name, bound = "flash_fwd_kernel<64, split, cached> + combine_kernel<64>", "hbm"
     elif args.workload == "qwen3_add_rms_norm":
         # The residual add + RMSNorm between Qwen3-Embedding's layers: hidden size 16 heads x 128 = 2048.
         g = torch.Generator(device=dev).manual_seed(0x5EED0030)
@@ -248,8 +269,9 @@ def main():
                 "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": HBM_TRAFFIC_BYTES.get(args.workload),
                 "traffic_unit": "bytes per launch", "kernel": kernel_name,
                 "kernel_us": round(kernel_us, 3), "bytes_per_launch": bytes_min}
-        metric = ("row norm GB/s on 1 MI355X" if args.workload == "qwen3_add_rms_norm" else
-                  "attention prologue GB/s on 1 MI355X")
+        metric = {"qwen3_add_rms_norm": "row norm GB/s on 1 MI355X",
+                  "whisper_decode": "decoder-step attention GB/s of K and V on 1 MI355X"}.get(
+                      args.workload, "attention prologue GB/s on 1 MI355X")
         unit = "GB/s"
 
     # ---- CPU baseline: the oracle's restatement of the reference graph path, bounded sample.

@@ -63,6 +63,7 @@ typedef __attribute__((ext_vector_type(4))) int i32x4;
 #define LDS_PTR(T) T __attribute__((address_space(3))) *
 
 constexpr int kBkv = 64;       // keys per ring slot
+constexpr int kScannedBlocks = 256;  // key blocks (16384 keys) of a key mask row scanned up front
 constexpr int kWaveRows = 32;  // query rows a wave owns: the N of the MFMA atom
 constexpr int kXcds = 8;       // accelerator dies of an MI355X, each with its own L2
 constexpr float kLog2e = 1.44269504088896340736f;
@@ -201,6 +202,11 @@ struct Wave {
   f32x16 acc[DB];
   float m_run, l_run;
   int mask_next;
+  // A key mask whose row was scanned at the start (rows of up to kScannedBlocks blocks): the
+  // blocks' 64-bit words, one copy a wave, in LDS after the ring.  Otherwise the words are read a
+  // lane a key, two blocks ahead of their use (mask_next).
+  bool scanned;
+  LDS_PTR(uint64_t) mask_words;
   // A streaming workgroup's next item (STREAM; nxt_end = 0: none): this item's
   // last steps request its first blocks.  The next item's blocks follow this item's at an even
   // position of the ring (end_even = end rounded up), so every item starts in slot 0.
@@ -288,7 +294,15 @@ template <int D, int NW, bool F16, unsigned FLAGS>
 __device__ __forceinline__ uint64_t uniform_bits(const Wave<D, NW, F16, FLAGS> &w, int blk, int word) {
   const int k0 = blk * kBkv;
   uint64_t kbits = ~0ull;
-  if (w.key_mask != nullptr) kbits = __builtin_amdgcn_ballot_w64(word != 0);
+  if (w.key_mask != nullptr) {
+    if (w.scanned) {
+      const uint64_t x = w.mask_words[blk];  // the same address in every lane
+      kbits = (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)x) |
+              (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(x >> 32)) << 32;
+    } else {
+      kbits = __builtin_amdgcn_ballot_w64(word != 0);
+    }
+  }
   if (k0 + kBkv > w.len) kbits &= (w.len > k0) ? (~0ull >> (64 - (w.len - k0))) : 0ull;
   return kbits;
 }
@@ -586,7 +600,7 @@ __device__ __forceinline__ void edge_step(Wave<D, NW, F16, FLAGS> &w, const uint
   uint32_t bw[16];
   if (w.biased && more) load_bias<D, NW>(w, (blk + 1) * kBkv, w.my_row_ok, bw);
   fill_v<D, NW>(w, blk + 1, par ^ 1);
-  if (blk + 2 < w.end) w.mask_next = mask_lane<D, NW>(w, blk + 2);
+  if (!w.scanned && blk + 2 < w.end) w.mask_next = mask_lane<D, NW>(w, blk + 2);
   fill_k<D, NW>(w, blk + 2, par);
   float corr;
   const float m_exp = adopt_maximum<D, NW>(w, bm, corr);
@@ -878,9 +892,37 @@ __global__ __launch_bounds__(NW * 64, (D == 64 && !BIASED) ? 3 : 2) void flash_f
   fill_k<D, NW>(w, 0, 0);
   fill_v<D, NW>(w, 0, 0);
   fill_k<D, NW>(w, 1, 1);
-  // Key-mask words are read two blocks ahead of their use.
-  const int word0 = mask_lane<D, NW>(w, 0);
-  w.mask_next = mask_lane<D, NW>(w, 1);
+  // A key mask row of up to kScannedBlocks blocks is scanned now, under the fills' flight: every
+  // wave ballots each block's 64 keys into a word of its own LDS copy.  The scan also says where
+  // the row's last visible key is (later blocks are skipped, like blocks past a length) and how
+  // many leading blocks hide nothing (those take the hot loop).  A longer row's words are read two
+  // blocks ahead of their use instead.
+  w.scanned = key_mask != nullptr && end <= kScannedBlocks;
+  w.mask_words = (LDS_PTR(uint64_t))(smem + TL::kLds) + w.wave * kScannedBlocks;
+  int word0 = 0, lead_open = 0, seen_end = 0;
+  w.mask_next = 0;
+  if (w.scanned) {
+    bool open = true;
+    for (int base = 0; base < end; base += 8) {
+      int words[8];
+#pragma unroll
+      for (int i = 0; i < 8; i++) words[i] = base + i < end ? mask_lane<D, NW>(w, base + i) : 0;
+#pragma unroll
+      for (int i = 0; i < 8; i++) {
+        if (base + i >= end) break;
+        const uint64_t bits = __builtin_amdgcn_ballot_w64(words[i] != 0);
+        if (w.lane == 0) w.mask_words[base + i] = bits;
+        if (bits != 0) seen_end = base + i + 1;
+        open = open && bits == ~0ull;
+        lead_open += open ? 1 : 0;
+      }
+    }
+    end = min(end, seen_end);
+    w.end = end;
+  } else if (key_mask != nullptr) {
+    word0 = mask_lane<D, NW>(w, 0);
+    w.mask_next = mask_lane<D, NW>(w, 1);
+  }
 
   // ---- per-lane LDS offsets of the operand reads.
   // K fragment (kb, ks): row 32kb + ln, logical chunk 2ks + g.
@@ -946,8 +988,9 @@ __global__ __launch_bounds__(NW * 64, (D == 64 && !BIASED) ? 3 : 2) void flash_f
   // for a causal wave, below its first row's diagonal.  A key mask puts every block on the
   // edge path.  Step j is hot when block j+1 is such a block.
   int full = 0;
-  if (w.positive && key_mask == nullptr) {
+  if (w.positive && (key_mask == nullptr || w.scanned)) {
     full = min(my_end, len / kBkv);
+    if (w.scanned) full = min(full, lead_open);
     if (RANGED)
       full = min(full, w.hi_first < 0 ? 0 : (w.hi_first + 1) / kBkv);
     else if (CAUSAL)
@@ -1166,6 +1209,7 @@ __global__ __launch_bounds__(NW * 64, 3) void flash_stream_kernel(
   const int64_t o_row_stride = (int64_t)heads * D;
   w.tk = tk;
   w.key_mask = nullptr;
+  w.scanned = false;
   w.mask_row = 0;
   w.mask_bytes = 0;
   w.mask_next = 0;
@@ -1407,7 +1451,9 @@ hipError_t launch(const AttnArgs &a, hipStream_t stream) {
   const int64_t blocks = (int64_t)nqt * a.heads * a.batch;
   if (blocks == 0) return hipSuccess;
   if (blocks > 0x7ffffff0LL) return hipErrorInvalidConfiguration;
-  constexpr int smem = TL::kLds;
+  // The ring, and behind it the words of a scanned key mask row (a copy a wave).
+  constexpr int kMaskLds = NW * kScannedBlocks * 8;
+  const int smem = TL::kLds + (a.key_mask != nullptr ? kMaskLds : 0);
   const int64_t q_row = a.q_row_elems > 0 ? a.q_row_elems : (int64_t)a.heads * a.d;
   const int64_t kv_row = a.kv_row_elems > 0 ? a.kv_row_elems : (int64_t)a.kv_heads * a.d;
   // The fills address a (batch, kv head)'s rows with 32-bit byte offsets.
@@ -1421,7 +1467,8 @@ hipError_t launch(const AttnArgs &a, hipStream_t stream) {
   if (e != hipSuccess) return e;
   const uint64_t bit = device < 64 ? 1ull << device : 0;
   if ((configured.load(std::memory_order_acquire) & bit) == 0) {
-    e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            TL::kLds + kMaskLds);
     if (e != hipSuccess) return e;
     configured.fetch_or(bit, std::memory_order_release);
   }

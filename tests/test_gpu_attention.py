@@ -177,3 +177,49 @@ def test_visibility_is_bit_exact(device):
         vis = oracle.visible(b, t, tk, causal=causal, key_mask=mask).astype(bool)
         # Scores are O(1) here, so every visible key keeps a weight far above bf16's floor.
         assert np.array_equal(got != 0.0, vis)
+
+
+MASK_PATTERNS = {
+    "a hidden block in the middle, hidden blocks at the end": lambda b, tk: np.stack(
+        [(np.arange(tk) < 300) & ~((np.arange(tk) >= 128) & (np.arange(tk) < 192)) for _ in range(b)]),
+    "the first two blocks hidden": lambda b, tk: np.stack([np.arange(tk) >= 128 + 7 * i for i in range(b)]),
+    "one visible key in the last block": lambda b, tk: np.stack([np.arange(tk) == tk - 1 - i for i in range(b)]),
+    "every other block hidden": lambda b, tk: np.stack([(np.arange(tk) // 64 + i) % 2 == 0 for i in range(b)]),
+    "a row of nothing": lambda b, tk: np.stack([np.zeros(tk, dtype=bool) if i == 1 else np.arange(tk) % 3 != 0 for i in range(b)]),
+}
+
+
+@pytest.mark.parametrize("pattern", list(MASK_PATTERNS), ids=list(MASK_PATTERNS))
+@pytest.mark.parametrize("causal", [False, True])
+def test_key_masks_with_whole_hidden_blocks(device, pattern, causal):
+    """A key mask row is scanned at the start of a tile: blocks past its last visible key are skipped and
+    leading blocks that hide nothing take the hot loop.  Whatever the pattern, the result is the direct softmax's,
+    and the same as with the mask folded into an additive bias of -inf (which takes neither shortcut)."""
+    b, t, tk, h, d = 3, 200, 500, 2, 64
+    q, k, v = graph_case(b, t, tk, h, h, d)
+    mask = MASK_PATTERNS[pattern](b, tk)
+    got = to_np(run(device, q, k, v, causal, mask=mask))
+    want = oracle.attention_direct(oracle.AttnProblem(q, k, v, causal=causal, key_mask=mask))
+    assert max_abs(got, want) < 2e-2
+    rows_without_keys = ~oracle.visible(b, t, tk, causal=causal, key_mask=mask).astype(bool).any(-1)  # [b, t]
+    assert not got[rows_without_keys].any()
+    walls = np.where(mask[:, None, None, :], 0.0, -np.inf).astype(np.float32) * np.ones((b, h, t, tk), dtype=np.float32)
+    biased = svod_amd.attention(bf16_tensor(q, device), bf16_tensor(k, device), bf16_tensor(v, device),
+                                Attn(causal=causal, bias=bf16_tensor(np.nan_to_num(walls, nan=0.0, neginf=-np.inf), device)))
+    assert max_abs(to_np(biased), want) < 2e-2
+
+
+def test_a_key_mask_row_too_long_to_scan(device):
+    """Past 256 blocks (16384 keys) the mask words are read two blocks ahead of their use instead."""
+    b, t, tk, h, d = 1, 40, 16500, 1, 64
+    q, k, v = graph_case(b, t, tk, h, h, d)
+    mask = (np.arange(tk)[None, :] % 7 != 3) & (np.arange(tk)[None, :] < 16450)
+    keys = KeyMask.bool(torch.from_numpy(mask).to(device))
+    want = oracle.attention_direct(oracle.AttnProblem(q, k, v, key_mask=mask))
+    dq, dk, dv = (bf16_tensor(x, device) for x in (q, k, v))
+    whole = svod_amd.attention(dq, dk, dv, Attn(keys=keys, splits=1))  # one pass over 258 blocks: too long to scan
+    assert "flash_attention" in svod_amd.chosen()
+    assert max_abs(to_np(whole), want) < 2e-2
+    split = svod_amd.attention(dq, dk, dv, Attn(keys=keys))  # split unasked: every split scans its share
+    assert "combine_splits" in svod_amd.chosen()
+    assert max_abs(to_np(split), want) < 2e-2

@@ -49,7 +49,7 @@ def parse():
                          "none is served from the Infinity Cache")
     ap.add_argument("--no-graph", action="store_true", help="enqueue eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-row-order", action="store_true",
-                    help="bge_m3: take the batch rows as they come instead of ordering them by length once per step")
+                    help="bge_m3, bge_m3_bool: take the batch rows as they come instead of ordering them by length once per step")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="rough budget of the CPU baseline sample")
     return ap.parse_args()
@@ -88,9 +88,10 @@ def main():
         # the step orders the batch rows by length once (one small launch, inside the timed region) and
         # hands the order to its 24 layer calls.  --no-row-order runs the rows as they come.
         order = None
-        if args.workload == "bge_m3" and not args.no_row_order:
+        if not args.no_row_order:
             order = torch.empty(sets[0].key_lens.shape, dtype=torch.int32, device=dev)
-            extra_calls.append(lambda: svod_amd.order_rows(sets[0].key_lens, out=order))
+            keys0 = sets[0].key_lens if args.workload == "bge_m3" else sets[0].key_mask()
+            extra_calls.append(lambda: svod_amd.order_rows(keys0, out=order))
         for w in sets:
             keys = KeyMask.lens(w.key_lens) if args.workload == "bge_m3" else KeyMask.bool(w.key_mask())
             out = torch.empty_like(w.q)

@@ -169,15 +169,16 @@ int svodk_attention_packed(const svodk_tensor *qkv, int32_t heads, int32_t kv_he
                            const svodk_tensor *out, void *hip_stream);
 
 /*
- * The batch rows in descending order of their key lengths, ties by row: order[p] = the row with
- * the p-th most keys, for svodk_attn.row_order.  No counterpart in the reference, whose grid takes
- * the rows as they come: workgroups are dispatched in launch order, so a variable-length batch
- * whose rows run grouped by length keeps a CU's workgroups in step and ends on its short tiles
- * (BGE-M3-shaped batches: 3 % less kernel time with operands cold in HBM, 8-12 % with operands
- * still in the Infinity Cache).  key_lens [B] I32 or I64, order [B] I32, B <= 8192.  One small
- * launch on the stream.
+ * The batch rows in descending order of their key counts, ties by row: order[p] = the row with
+ * the p-th most keys, for svodk_attn.row_order.  `keys` is what the call's key mask is: [B] lengths
+ * (I32 or I64) or a [B, Tk] mask (BOOL or I32), a row of which counts up to its last visible key.
+ * No counterpart in the reference, whose grid takes the rows as they come: workgroups are
+ * dispatched in launch order, so a variable-length batch whose rows run grouped by length keeps a
+ * CU's workgroups in step and ends on its short tiles (BGE-M3-shaped batches: 3 % less kernel time
+ * with operands cold in HBM, 8-12 % with operands still in the Infinity Cache).  order [B] I32,
+ * B <= 8192.  One small launch on the stream.
  */
-int svodk_order_rows(const svodk_tensor *key_lens, const svodk_tensor *order, void *hip_stream);
+int svodk_order_rows(const svodk_tensor *keys, const svodk_tensor *order, void *hip_stream);
 
 /*
  * Bytes of `workspace` svodk_attention needs for these operands and options:

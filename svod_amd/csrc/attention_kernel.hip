@@ -1567,14 +1567,32 @@ hipError_t launch_d(const AttnArgs &a, hipStream_t stream) {
   return a.f16 ? launch_t<D, true>(a, stream) : launch_t<D, false>(a, stream);
 }
 
-// The batch rows in descending order of their key lengths, ties by row: order[p] = the row with
-// the p-th most keys.  One workgroup; a thread ranks its rows against all of them in LDS.
-__global__ __launch_bounds__(256) void order_rows_kernel(const void *__restrict__ key_lens, int32_t lens_i64, int32_t n,
-                                                         int32_t *__restrict__ order) {
+// The batch rows in descending order of their key counts, ties by row: order[p] = the row with
+// the p-th most keys.  A row's count is its length, or with a [n, tk] key mask the place after its
+// last visible key (what a tile's key blocks run to).  One workgroup; a thread ranks its rows
+// against all of them in LDS.
+__global__ __launch_bounds__(256) void order_rows_kernel(const void *__restrict__ keys, int32_t elem_bytes, int32_t n,
+                                                         int32_t tk, int32_t *__restrict__ order) {
   extern __shared__ int32_t lens_sh[];
-  for (int i = threadIdx.x; i < n; i += 256) {
-    const long long x = lens_i64 ? ((const long long *)key_lens)[i] : (long long)((const int *)key_lens)[i];
-    lens_sh[i] = (int32_t)(x < 0 ? 0 : (x > 0x7fffffffLL ? 0x7fffffffLL : x));
+  if (tk < 0) {
+    for (int i = threadIdx.x; i < n; i += 256) {
+      const long long x = elem_bytes == 8 ? ((const long long *)keys)[i] : (long long)((const int *)keys)[i];
+      lens_sh[i] = (int32_t)(x < 0 ? 0 : (x > 0x7fffffffLL ? 0x7fffffffLL : x));
+    }
+  } else {
+    // A wave a row at a time: the highest key any lane finds visible.
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int i = wave; i < n; i += 4) {
+      int last = 0;
+      for (int j = lane; j < tk; j += 64) {
+        const int64_t at = (int64_t)i * tk + j;
+        const int x = elem_bytes == 1 ? (int)((const uint8_t *)keys)[at] : ((const int *)keys)[at];
+        if (x != 0) last = j + 1;
+      }
+#pragma unroll
+      for (int m = 32; m >= 1; m >>= 1) last = max(last, __shfl_xor(last, m, 64));
+      if (lane == 0) lens_sh[i] = last;
+    }
   }
   __syncthreads();
   for (int i = threadIdx.x; i < n; i += 256) {
@@ -1590,10 +1608,11 @@ __global__ __launch_bounds__(256) void order_rows_kernel(const void *__restrict_
 
 }  // namespace
 
-hipError_t launch_order_rows(const void *key_lens, int32_t lens_i64, int32_t n, int32_t *order, hipStream_t stream) {
+hipError_t launch_order_rows(const void *keys, int32_t elem_bytes, int32_t n, int32_t tk, int32_t *order,
+                             hipStream_t stream) {
   if (n <= 0) return hipSuccess;
   if (n > kMaxOrderedRows) return hipErrorInvalidValue;
-  hipLaunchKernelGGL(order_rows_kernel, dim3(1), dim3(256), (size_t)n * 4, stream, key_lens, lens_i64, n, order);
+  hipLaunchKernelGGL(order_rows_kernel, dim3(1), dim3(256), (size_t)n * 4, stream, keys, elem_bytes, n, tk, order);
   return hipGetLastError();
 }
 

@@ -112,9 +112,11 @@ bool attention_supports(int32_t d);
 // Whether launch_attention runs `a` on grouped tiles: the heads of a KV head's group side by side
 // in one query tile (a decoder step under GQA: no causal or per-row mask, group * t <= 128).
 bool attention_groups(const AttnArgs &a);
-// order[p] = the batch row with the p-th most keys (ties by row), for AttnArgs::row_order.
+// order[p] = the batch row with the p-th most keys (ties by row), for AttnArgs::row_order.  `keys` is
+// [n] lengths (tk < 0; elements of 4 or 8 bytes) or an [n, tk] key mask (elements of 1 or 4 bytes).
 constexpr int32_t kMaxOrderedRows = 8192;
-hipError_t launch_order_rows(const void *key_lens, int32_t lens_i64, int32_t n, int32_t *order, hipStream_t stream);
+hipError_t launch_order_rows(const void *keys, int32_t elem_bytes, int32_t n, int32_t tk, int32_t *order,
+                             hipStream_t stream);
 // Tuning of the streaming form (workgroups that walk runs of query tiles): see svodk_tune_streaming.
 void attention_stream_slots(int32_t slots);
 // Text of the tile configuration launch_attention picks for `a` (for chosen()).

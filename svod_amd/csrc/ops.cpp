@@ -621,27 +621,30 @@ int svodk_attention_packed(const svodk_tensor *qkv, int32_t heads, int32_t kv_he
 void svodk_tune_streaming(int32_t workgroups_per_xcd) { svodk::attention_stream_slots(workgroups_per_xcd); }
 
 // The workspace of a split call (tk/src/ops/attention.rs:285-293).
-int svodk_order_rows(const svodk_tensor *key_lens, const svodk_tensor *order, void *hip_stream) {
+int svodk_order_rows(const svodk_tensor *keys, const svodk_tensor *order, void *hip_stream) {
   const char *op = "order_rows";
-  if (!well_formed(key_lens) || !well_formed(order))
+  if (!well_formed(keys) || !well_formed(order))
     return fail(SVODK_ERR_ARGUMENT, "%s: a null or malformed tensor descriptor", op);
-  if (!(key_lens->rank == 1 && order->rank == 1 && order->shape[0] == key_lens->shape[0]))
-    return fail(SVODK_ERR_SHAPE, "%s: key lens %s and order %s, expected [B] and [B]", op, fmt_shape(key_lens).c_str(),
-                fmt_shape(order).c_str());
-  if (!is_int(key_lens->dtype))
-    return fail(SVODK_ERR_DTYPE, "%s: key lens is %s, the input is an integer type", op, dtype_name(key_lens->dtype));
+  const bool mask = keys->rank == 2;
+  if (!((keys->rank == 1 || mask) && order->rank == 1 && order->shape[0] == keys->shape[0]))
+    return fail(SVODK_ERR_SHAPE, "%s: keys %s and order %s, expected [B] or [B, Tk] and [B]", op,
+                fmt_shape(keys).c_str(), fmt_shape(order).c_str());
+  if (mask ? !(keys->dtype == SVODK_BOOL || keys->dtype == SVODK_I32) : !is_int(keys->dtype))
+    return fail(SVODK_ERR_DTYPE, "%s: keys are %s, the input is %s", op, dtype_name(keys->dtype),
+                mask ? "Bool or Int32" : "an integer type");
   if (order->dtype != SVODK_I32)
     return fail(SVODK_ERR_DTYPE, "%s: order is %s, the output is Int32", op, dtype_name(order->dtype));
-  if (key_lens->shape[0] > svodk::kMaxOrderedRows)
-    return fail(SVODK_ERR_SHAPE, "%s: %lld rows, at most %d", op, (long long)key_lens->shape[0], svodk::kMaxOrderedRows);
+  if (keys->shape[0] > svodk::kMaxOrderedRows || (mask && keys->shape[1] > 0x7fffffff))
+    return fail(SVODK_ERR_SHAPE, "%s: %lld rows, at most %d", op, (long long)keys->shape[0], svodk::kMaxOrderedRows);
   if (!current_device_has_kernels()) return ran_graph(op, SVODK_GRAPH_TARGET);
-  if (key_lens->data == nullptr || order->data == nullptr) return fail(SVODK_ERR_ARGUMENT, "%s: a null device pointer", op);
-  Span spans[2] = {{"key_lens", key_lens->data, (size_t)numel(key_lens) * dtype_bytes(key_lens->dtype), false},
+  if (keys->data == nullptr || order->data == nullptr) return fail(SVODK_ERR_ARGUMENT, "%s: a null device pointer", op);
+  Span spans[2] = {{"keys", keys->data, (size_t)numel(keys) * dtype_bytes(keys->dtype), false},
                    {"order", order->data, (size_t)numel(order) * 4, true}};
   if (int rc = check_aliasing(op, spans, 2)) return rc;
   ran(op, "order_rows", "one workgroup");
-  const hipError_t e = svodk::launch_order_rows(key_lens->data, key_lens->dtype == SVODK_I64, (int32_t)key_lens->shape[0],
-                                                (int32_t *)order->data, (hipStream_t)hip_stream);
+  const hipError_t e = svodk::launch_order_rows(keys->data, (int32_t)dtype_bytes(keys->dtype), (int32_t)keys->shape[0],
+                                                mask ? (int32_t)keys->shape[1] : -1, (int32_t *)order->data,
+                                                (hipStream_t)hip_stream);
   if (e != hipSuccess) return fail(SVODK_ERR_LAUNCH, "%s: %s", op, hipGetErrorString(e));
   return SVODK_KERNEL;
 }

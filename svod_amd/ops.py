@@ -419,14 +419,15 @@ def plan_norm(has_target: bool, dtypes, x_dims) -> Optional[Fallback]:
     return _plan(lib.svodk_plan_norm(int(has_target), dt, len(dtypes), xd, 0 if x_dims is None else len(x_dims)))
 
 
-def order_rows(key_lens: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """The batch rows in descending order of their key lengths (ties by row) as int32 ``[B]``, for
-    ``Attn.row_order``: a variable-length batch that runs its long rows first ends on its short tiles."""
+def order_rows(keys: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The batch rows in descending order of their key counts (ties by row) as int32 ``[B]``, for
+    ``Attn.row_order``; ``keys`` is ``[B]`` lengths or a ``[B, Tk]`` key mask.  A variable-length batch whose
+    rows run grouped by length ends on its short tiles."""
     lib = load_library()
     if out is None:
-        out = torch.empty(key_lens.shape, dtype=torch.int32, device=key_lens.device)
+        out = torch.empty(keys.shape[:1], dtype=torch.int32, device=keys.device)
     keep: list = []
-    status = lib.svodk_order_rows(_ref(keep, key_lens), _ref(keep, out), ctypes.c_void_p(_stream(key_lens)))
+    status = lib.svodk_order_rows(_ref(keep, keys), _ref(keep, out), ctypes.c_void_p(_stream(keys)))
     _finish("order_rows", status)
     return out
 

@@ -23,6 +23,19 @@ def test_order_rows_is_a_stable_descending_sort(device, n, dtype):
     assert svod_amd.chosen().startswith('Kernel { op: "order_rows"')
 
 
+@pytest.mark.parametrize("dtype", [torch.bool, torch.int32])
+def test_order_rows_of_a_key_mask_counts_up_to_the_last_visible_key(device, dtype):
+    rng = np.random.default_rng(4)
+    n, tk = 37, 300
+    mask = rng.random((n, tk)) < 0.02
+    mask[5] = False                      # a row of nothing sorts last
+    mask[9, tk - 1] = True               # a full-length row sorts first
+    reach = np.where(mask.any(1), tk - np.argmax(mask[:, ::-1], axis=1), 0)
+    got = svod_amd.order_rows(torch.from_numpy(mask).to(dtype).to(device)).cpu().numpy()
+    assert np.array_equal(got, np.argsort(-reach, kind="stable"))
+    assert got[0] == 9 and got[-1] == 5
+
+
 # (b, t, tk, h, hkv, d, causal, splits)
 CASES = [(12, 300, 300, 4, 2, 64, False, None), (7, 200, 260, 4, 4, 128, True, None), (5, 130, 512, 2, 2, 64, False, 2)]
 

@@ -433,8 +433,16 @@ static int attend(const svodk_tensor *q, const svodk_tensor *k, const svodk_tens
     return fail(SVODK_ERR_DTYPE, "%s: seg start is %s, the input is Int32 or Int64", op,
                 dtype_name(opts->seg_start->dtype));
   const int64_t t = q->shape[1], tk = k->shape[1], d = q->shape[3];
-  if (t > 0x7fffffff || tk > 0x7fffffff || heads > 0x7fffffff || cap > 0x7fffffff)
+  if (t > 0x7fffffff || tk > 0x7fffffff || heads > 0xffff || cap > 0x7fffffff)
     return ran_graph(op, SVODK_GRAPH_SHAPE);
+  {
+    // The kernel addresses a (batch, KV head)'s rows with 32-bit byte offsets and counts its
+    // workgroups in 31 bits: shapes past either keep the graph.
+    const int64_t row_elems = packed ? (heads + 2 * kv_heads) * d : k->shape[2] * d;
+    const int64_t tiles = (t + 127) / 128 * heads * cap;
+    if (tk * row_elems * 2 > 0x7fffffffLL || row_elems > 0x3fffffff || tiles * 64 > 0x7ffffff0LL)
+      return ran_graph(op, SVODK_GRAPH_SHAPE);
+  }
 
   // A packed operand is one parameter (L268): its views overlap one another by construction.
   const size_t packed_bytes = packed ? (size_t)numel(packed) * 2 : 0;

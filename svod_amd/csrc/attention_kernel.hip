@@ -94,9 +94,14 @@ struct Tile {
   static constexpr int kBytes = kBkv * kRowBytes;
   static constexpr int kLds = 4 * kBytes;
   static constexpr int kInstrs = kBytes / 1024;  // wave-wide 1 KiB fills per tile
-  __device__ static constexpr int swz_k(int row) { return D == 64 ? ((row >> 1) & 7) : (row & 15); }
+  // D = 32: rows are 64 bytes, four to the bank period, so 16 rows at one logical chunk spread over
+  // the period's 16 chunk places when the chunk is xor-ed with row / 4; a V row is one 64-byte
+  // group and four consecutive rows are the whole period as they lie.
+  __device__ static constexpr int swz_k(int row) {
+    return D == 32 ? ((row >> 2) & 3) : D == 64 ? ((row >> 1) & 7) : (row & 15);
+  }
   // In units of 64-byte groups (4 chunks).
-  __device__ static constexpr int swz_v(int row) { return D == 64 ? ((row >> 1) & 1) : (row & 3); }
+  __device__ static constexpr int swz_v(int row) { return D == 32 ? 0 : D == 64 ? ((row >> 1) & 1) : (row & 3); }
 };
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
@@ -685,7 +690,7 @@ struct Ranges {
 // queries of one head, for calls whose whole group fits a tile (a decoder step: heads / kv_heads
 // * T <= 128).  The group's heads then share one pass over their K and V instead of one each.
 template <int D, int NW, bool CAUSAL, bool SPLIT, bool RANGED, bool BIASED, bool CACHED, bool GROUPED, bool F16>
-__global__ __launch_bounds__(NW * 64, (D == 64 && !BIASED) ? 3 : 2) void flash_fwd_kernel(
+__global__ __launch_bounds__(NW * 64, (D <= 64 && !BIASED) ? 3 : 2) void flash_fwd_kernel(
     uint32_t unit_size, uint32_t unit_rcp, uint32_t nqt_u, uint32_t nqt_rcp, uint32_t kvh_u, uint32_t kvh_rcp,
     uint32_t units, uint32_t heads_group, const void *__restrict__ key_lens, const int32_t *__restrict__ row_order,
     int32_t t, uint32_t tk_lens64, const uint16_t *__restrict__ q, const uint16_t *__restrict__ k,
@@ -1616,7 +1621,7 @@ hipError_t launch_order_rows(const void *keys, int32_t elem_bytes, int32_t n, in
   return hipGetLastError();
 }
 
-bool attention_supports(int32_t d) { return d == 64 || d == 128; }
+bool attention_supports(int32_t d) { return d == 32 || d == 64 || d == 128; }
 
 bool attention_groups(const AttnArgs &a) {
   const bool ranged = a.win_left >= 0 || a.chunk_size > 0 || a.seg_start != nullptr;
@@ -1641,6 +1646,7 @@ const char *attention_config(const AttnArgs &a) {
 
 hipError_t launch_attention(const AttnArgs &a, hipStream_t stream) {
   switch (a.d) {
+    case 32: return launch_d<32>(a, stream);
     case 64: return launch_d<64>(a, stream);
     case 128: return launch_d<128>(a, stream);
     default: return hipErrorInvalidValue;

@@ -1160,7 +1160,7 @@ __global__ __launch_bounds__(NW * 64, 3) void flash_stream_kernel(
     uint32_t units, uint32_t heads_group, const void *__restrict__ key_lens, const uint16_t *__restrict__ q, int32_t t,
     uint32_t tk_lens64, const uint16_t *__restrict__ k, const uint16_t *__restrict__ v,
     uint16_t *__restrict__ o, float scale, int32_t q_row_elems, int32_t kv_row_elems, uint32_t slots,
-    uint32_t queue_set) {
+    uint32_t queue_set, const int32_t *__restrict__ row_order) {
 #if defined(__HIP_DEVICE_COMPILE__)
   const Geometry geo = {unit_size, unit_rcp, nqt_u, nqt_rcp, kvh_u, kvh_rcp, heads_group >> 16, units};
   const int heads = (int)(heads_group & 0xffffu);
@@ -1252,9 +1252,17 @@ __global__ __launch_bounds__(NW * 64, 3) void flash_stream_kernel(
     const uint32_t within = s - round * geo.unit_size;
     const uint32_t head_in_group = div_by(within, geo.nqt, geo.nqt_rcp);
     const int order = (int)(within - head_in_group * geo.nqt);
-    it.b = (int)div_by(unit, geo.kv_heads, geo.kvh_rcp);
-    const int kvh = (int)(unit - (uint32_t)it.b * geo.kv_heads);
+    const int b_place = (int)div_by(unit, geo.kv_heads, geo.kvh_rcp);
+    const int kvh = (int)(unit - (uint32_t)b_place * geo.kv_heads);
     it.h = kvh * (int)geo.group + (int)head_in_group;
+    // The batch row of this place of the launch (AttnArgs::row_order), by scalar load like the length.
+    it.b = b_place;
+    if (row_order != nullptr) {
+      int x;
+      asm volatile("s_load_dword %0, %1, %2\n\ts_waitcnt lgkmcnt(0)" : "=s"(x) : "s"(row_order), "s"(b_place * 4) : "memory");
+      const int nbatch = (int)div_by(geo.units, geo.kv_heads, geo.kvh_rcp);
+      it.b = min(max(x, 0), nbatch - 1);
+    }
     const int qt = CAUSAL ? (int)geo.nqt - 1 - order : order;  // L524-528: longest first under a causal mask
     it.q_off = qt * BQ;
     it.len = len_of_uniform(key_lens, lens_i64, tk, it.b);
@@ -1442,7 +1450,7 @@ hipError_t launch_stream(const AttnArgs &a, hipStream_t stream, int64_t slots, c
                      geo.nqt, geo.nqt_rcp, geo.kv_heads, geo.kvh_rcp, geo.units, heads_group, a.key_lens,
                      (const uint16_t *)a.q, a.t, tk_lens64, (const uint16_t *)a.k, (const uint16_t *)a.v,
                      (uint16_t *)a.o, a.scale, (int32_t)q_row, (int32_t)kv_row, (uint32_t)slots,
-                     g_queue_turn.fetch_add(1u, std::memory_order_relaxed) % kQueueSets);
+                     g_queue_turn.fetch_add(1u, std::memory_order_relaxed) % kQueueSets, (const int32_t *)a.row_order);
   return hipGetLastError();
 }
 
@@ -1499,7 +1507,7 @@ hipError_t launch(const AttnArgs &a, hipStream_t stream) {
   // It is never chosen unasked: measured, it has not beaten a workgroup per tile.
   if constexpr (D == 64 && !SPLIT && !RANGED && !BIASED && !CACHED && !GROUPED) {
     const int knob = g_stream_slots.load(std::memory_order_relaxed);
-    if (knob > 0 && a.key_mask == nullptr && a.row_order == nullptr)
+    if (knob > 0 && a.key_mask == nullptr)
       return launch_stream<D, NW, CAUSAL, F16>(a, stream, knob, geo, q_row, kv_row);
   }
   const uint32_t heads_group = (uint32_t)a.heads | geo.group << 16;

@@ -114,3 +114,16 @@ def test_two_streams_at_once_do_not_share_counters(device):
     torch.cuda.synchronize()
     assert np.array_equal(bits(o1), want1)
     assert np.array_equal(bits(o2), want2)
+
+
+def test_streaming_follows_a_row_order(device):
+    b, t, tk, h, hkv = 9, 300, 300, 4, 2
+    q, k, v = (bf16_tensor(x, device) for x in case(b, t, tk, h, hkv, seed=41))
+    lens = torch.tensor([300, 7, 64, 129, 0, 255, 300, 65, 1], dtype=torch.int32, device=device)
+    order = svod_amd.order_rows(lens)
+    svod_amd.tune_streaming(-1)
+    plain = bits(svod_amd.attention(q, k, v, Attn(keys=KeyMask.lens(lens))))
+    svod_amd.tune_streaming(3)
+    streamed = svod_amd.attention(q, k, v, Attn(keys=KeyMask.lens(lens), row_order=order))
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(streamed), plain)

@@ -689,20 +689,20 @@ struct Ranges {
 // GROUPED: the query tile's rows are (head of the KV head's group, query) pairs instead of 128
 // queries of one head, for calls whose whole group fits a tile (a decoder step: heads / kv_heads
 // * T <= 128).  The group's heads then share one pass over their K and V instead of one each.
-template <int D, int NW, bool CAUSAL, bool SPLIT, bool RANGED, bool BIASED, bool CACHED, bool GROUPED, bool F16>
-__global__ __launch_bounds__(NW * 64, (D <= 64 && !BIASED) ? 3 : 2) void flash_fwd_kernel(
-    uint32_t unit_size, uint32_t unit_rcp, uint32_t nqt_u, uint32_t nqt_rcp, uint32_t kvh_u, uint32_t kvh_rcp,
-    uint32_t units, uint32_t heads_group, const void *__restrict__ key_lens, const int32_t *__restrict__ row_order,
-    int32_t t, uint32_t tk_lens64, const uint16_t *__restrict__ q, const uint16_t *__restrict__ k,
-    const uint16_t *__restrict__ v, uint16_t *__restrict__ o, const void *__restrict__ key_mask, int32_t mask_bytes,
-    float scale, Splits sp, int32_t q_row_elems, int32_t kv_row_elems, Ranges rg) {
-  // The body is device code only: the host pass needs the kernel's handle, not its
-  // instructions (and drops the whole instantiation over the LDS-fill instructions).
+// The workgroup's whole program, for the kernels below to inline: `smem` is the workgroup's LDS (the
+// ring, and behind it the scanned key mask words of a launch with a key mask).  Device code only:
+// the host pass needs a kernel's handle, not its instructions (and would drop the whole
+// instantiation over the LDS-fill instructions).
 #if defined(__HIP_DEVICE_COMPILE__)
-  // The first 14 dwords of the arguments (up to tk_lens64) arrive in registers with the wave
-  // (kernarg preload, scalars and pointers only): they are what the workgroup's coordinates,
-  // its batch row and its length need, so none of those waits for an argument load.  Two of them
-  // are packed to fit: heads | group << 16, and tk | (key_lens is 64-bit) << 31.
+template <int D, int NW, bool CAUSAL, bool SPLIT, bool RANGED, bool BIASED, bool CACHED, bool GROUPED, bool F16>
+__device__ __forceinline__ void flash_fwd_body(
+    uint8_t *smem, uint32_t unit_size, uint32_t unit_rcp, uint32_t nqt_u, uint32_t nqt_rcp, uint32_t kvh_u,
+    uint32_t kvh_rcp, uint32_t units, uint32_t heads_group, const void *__restrict__ key_lens,
+    const int32_t *__restrict__ row_order, int32_t t, uint32_t tk_lens64, const uint16_t *__restrict__ q,
+    const uint16_t *__restrict__ k, const uint16_t *__restrict__ v, uint16_t *__restrict__ o,
+    const void *__restrict__ key_mask, int32_t mask_bytes, float scale, const Splits &sp, int32_t q_row_elems,
+    int32_t kv_row_elems, const Ranges &rg) {
+  // Two of the arguments are packed: heads | group << 16, and tk | (key_lens is 64-bit) << 31.
   const Geometry geo = {unit_size, unit_rcp, nqt_u, nqt_rcp, kvh_u, kvh_rcp, heads_group >> 16, units};
   const int heads = (int)(heads_group & 0xffffu);
   const int tk = (int)(tk_lens64 & 0x7fffffffu);
@@ -712,8 +712,6 @@ __global__ __launch_bounds__(NW * 64, (D <= 64 && !BIASED) ? 3 : 2) void flash_f
   constexpr int BQ = NW * kWaveRows;
   constexpr int KS = W::KS, DB = W::DB;
   static_assert(TL::kInstrs % NW == 0, "the tile fills in whole wave instructions per wave");
-
-  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
 
   // A unit of work is one (batch, KV head): the query tiles of the heads that share its K and
   // V.  Workgroups are dealt to the 8 XCDs round-robin, each XCD with its own L2, so the units
@@ -1101,7 +1099,25 @@ __global__ __launch_bounds__(NW * 64, (D <= 64 && !BIASED) ? 3 : 2) void flash_f
       }
     }
   }
+}
 #endif  // __HIP_DEVICE_COMPILE__
+
+template <int D, int NW, bool CAUSAL, bool SPLIT, bool RANGED, bool BIASED, bool CACHED, bool GROUPED, bool F16>
+__global__ __launch_bounds__(NW * 64, (D <= 64 && !BIASED) ? 3 : 2) void flash_fwd_kernel(
+    uint32_t unit_size, uint32_t unit_rcp, uint32_t nqt_u, uint32_t nqt_rcp, uint32_t kvh_u, uint32_t kvh_rcp,
+    uint32_t units, uint32_t heads_group, const void *__restrict__ key_lens, const int32_t *__restrict__ row_order,
+    int32_t t, uint32_t tk_lens64, const uint16_t *__restrict__ q, const uint16_t *__restrict__ k,
+    const uint16_t *__restrict__ v, uint16_t *__restrict__ o, const void *__restrict__ key_mask, int32_t mask_bytes,
+    float scale, Splits sp, int32_t q_row_elems, int32_t kv_row_elems, Ranges rg) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  // The first 14 dwords of the arguments (up to tk_lens64) arrive in registers with the wave
+  // (kernarg preload, scalars and pointers only): they are what the workgroup's coordinates,
+  // its batch row and its length need, so none of those waits for an argument load.
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+  flash_fwd_body<D, NW, CAUSAL, SPLIT, RANGED, BIASED, CACHED, GROUPED, F16>(
+      smem, unit_size, unit_rcp, nqt_u, nqt_rcp, kvh_u, kvh_rcp, units, heads_group, key_lens, row_order, t, tk_lens64,
+      q, k, v, o, key_mask, mask_bytes, scale, sp, q_row_elems, kv_row_elems, rg);
+#endif
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -1,6 +1,7 @@
 """Builds ``libsvodk_gfx950.so`` in-tree with hipcc, for gfx950 only.
 
-``python -m svod_amd.build`` compiles every source under ``csrc/``.  The
+``python -m svod_amd.build`` compiles every source under ``csrc/`` into the library and
+then into the code objects under ``co/`` (``--code-objects``: only those).  The
 library is never built implicitly at import: loading fails loudly when it is
 missing, so a stale or absent build cannot hide behind another code path.
 """
@@ -55,6 +56,47 @@ def build(verbose: bool = False) -> str:
     return LIB
 
 
+def build_code_objects(verbose: bool = False) -> str:
+    """Writes ``co/*.co`` — the kernels as stand-alone AMDGPU code objects with flat argument
+    records (``code_object.py`` says for whom) — and ``co/manifest.json``, after checking each
+    kernel against the loader's conditions."""
+    import json
+
+    from . import code_object as co
+
+    cc = hipcc()
+    os.makedirs(co.CO_DIR, exist_ok=True)
+    table = co.entries()
+    built = {}
+    for name, e in table.items():
+        if e["file"] in built:
+            continue
+        path = os.path.join(co.CO_DIR, e["file"])
+        # No argument preload here: a loader that writes its own user registers passes the record's address only.
+        extra = [f for f in EXTRA_FLAGS.get(e["source"], []) if "kernarg-preload" not in f]
+        extra = [f for i, f in enumerate(extra) if not (f == "-mllvm" and (i + 1 == len(extra) or extra[i + 1] == "-mllvm"))]
+        cmd = [cc, "-x", "hip", *DEVICE_FLAGS, "--offload-device-only", "--no-gpu-bundle-output", "-DSVODK_CODE_OBJECT",
+               "-O3", "-std=c++17", "-Wall", "-Wno-unused-command-line-argument", *extra,
+               os.path.join(CSRC, e["source"]), "-o", path]
+        _run(cmd, verbose)
+        with open(path, "rb") as f:
+            built[e["file"]] = f.read()
+    manifest = {"arch": "gfx950", "record": "buffers are 8-byte addresses, scalars 4-byte integers, in this order at "
+                                            "natural alignment; *_bits scalars are an f32's bit pattern",
+                "kernels": {}}
+    for name, e in table.items():
+        kd = co.check(built[e["file"]], name, e["params"])
+        manifest["kernels"][name] = {**{k: v for k, v in e.items() if k != "source"},
+                                     "kernarg_size": kd.kernarg_size, "lds_bytes": kd.group_segment_fixed_size}
+    for f in built:
+        unlisted = set(co.CodeObject.parse(built[f]).kernels()) - set(table)
+        if unlisted:
+            raise RuntimeError(f"{f}: kernels without a manifest entry: {sorted(unlisted)}")
+    with open(os.path.join(co.CO_DIR, "manifest.json"), "w") as f:
+        json.dump(manifest, f, indent=1)
+    return str(co.CO_DIR)
+
+
 def _run(cmd, verbose):
     if verbose:
         print(" ".join(cmd), flush=True)
@@ -68,4 +110,8 @@ def _run(cmd, verbose):
 
 
 if __name__ == "__main__":
-    print(build(verbose=True))
+    if "--code-objects" in sys.argv[1:]:
+        print(build_code_objects(verbose=True))
+    else:
+        print(build(verbose=True))
+        print(build_code_objects(verbose=True))

@@ -69,10 +69,12 @@ constexpr int kXcds = 8;       // accelerator dies of an MI355X, each with its o
 constexpr float kLog2e = 1.44269504088896340736f;
 constexpr float kRescaleAbove = 8.0f;  // tk/src/kernels/attention.rs:379
 
+#if !defined(SVODK_CODE_OBJECT)
 // Workgroups per XCD of the streaming form; <= 0 = a workgroup per query tile instead.
 std::atomic<int> g_stream_slots{0};
 // Streaming launches so far: each takes the next set of shared counters.
 std::atomic<uint32_t> g_queue_turn{0};
+#endif
 
 // A ring slot holds a [64 keys, D] tile, rows unpadded (D*2 bytes), filled by
 // buffer_load_dwordx4 ... lds: a wave instruction lands 64 consecutive 16-byte
@@ -1120,6 +1122,7 @@ __global__ __launch_bounds__(NW * 64, (D <= 64 && !BIASED) ? 3 : 2) void flash_f
 #endif
 }
 
+#if !defined(SVODK_CODE_OBJECT)  // the library's kernels and their launches: not part of a code object build
 // ---------------------------------------------------------------------------------------------
 // The streaming form: a workgroup walks query tiles (items) one after another as a single stream
 // of key blocks.  The last steps of an item fill the ring with the next item's first blocks, and
@@ -1678,3 +1681,76 @@ hipError_t launch_attention(const AttnArgs &a, hipStream_t stream) {
 }
 
 }  // namespace svodk
+
+#else  // SVODK_CODE_OBJECT
+// ---------------------------------------------------------------------------------------------
+// The same program as kernels a loader outside the HIP runtime can run: the reference's device
+// layer loads an AMDGPU code object, finds `<name>.kd`, and launches it with a flat argument
+// record (device/src/amd/program.rs:77-266, 403-414, 655-675; device/src/hcq.rs:1262-1285):
+//   * buffers are 8-byte addresses, every scalar a 4-byte integer, in parameter order at their
+//     natural alignment; nothing hidden follows them (the record is kernarg_size bytes, zeroed);
+//   * LDS is what the kernel descriptor says (group_segment_fixed_size): static, no launch-time size;
+//   * no dispatch packet pointer: the kernel may know its workgroup and lane, not the grid's or
+//     the workgroup's size (ENABLE_SGPR_DISPATCH_PTR must be clear);
+//   * the launch names workgroup COUNTS and the workgroup's threads.
+// So these take plain dimensions and work the launch geometry out themselves (three unsigned
+// divisions a workgroup), the scale travels as its bit pattern, and arguments are not preloaded
+// into registers (a loader that writes its own user registers hands over the record's address only).
+//
+// Parameters follow the reference kernel's order (tk/src/kernels/attention.rs:308-327, 452-459):
+// q, k, v, o, then key_lens ([batch] i32, or address 0 for none), then the scalars
+// batch, t, tk, heads, kv_heads, scale_bits.  Launch: workgroups
+// [ceil(batch * kv_heads, 8) * (heads / kv_heads) * ceil(t / 128), 1, 1] of [256, 1, 1] threads.
+// The host side's checks are the caller's: heads a multiple of kv_heads, heads < 65536, dimensions
+// positive, tk * kv_heads * D * 2 < 2^31.
+// ---------------------------------------------------------------------------------------------
+#if defined(__HIP_DEVICE_COMPILE__)
+// floor(2^32 / d) for div_by, or one less where d divides 2^32 (the estimate stays within one).
+__device__ __forceinline__ uint32_t rcp_for(uint32_t d) { return d <= 1 ? 0xffffffffu : 0xffffffffu / d; }
+
+template <int D, bool CAUSAL, bool F16>
+__device__ __forceinline__ void attention_entry(uint8_t *smem, const uint16_t *q, const uint16_t *k, const uint16_t *v,
+                                                uint16_t *o, const void *key_lens, int32_t batch, int32_t t,
+                                                int32_t tk, int32_t heads, int32_t kv_heads, int32_t scale_bits) {
+  constexpr int NW = 4;
+  if (batch <= 0 || t <= 0 || tk < 0 || kv_heads <= 0 || heads < kv_heads) return;
+  const uint32_t group = (uint32_t)heads / (uint32_t)kv_heads;
+  const uint32_t nqt = ((uint32_t)t + NW * kWaveRows - 1) / (NW * kWaveRows);
+  const uint32_t unit_size = group * nqt;
+  const Splits sp = {1u, 0xffffffffu, nullptr, nullptr, nullptr, (uint32_t)batch};
+  Ranges rg = {};
+  rg.win_left = -1;
+  rg.chunk_left = -1;
+  flash_fwd_body<D, NW, CAUSAL, false, false, false, false, false, F16>(
+      smem, unit_size, rcp_for(unit_size), nqt, rcp_for(nqt), (uint32_t)kv_heads, rcp_for((uint32_t)kv_heads),
+      (uint32_t)kv_heads * (uint32_t)batch, (uint32_t)heads | group << 16, key_lens, nullptr, t, (uint32_t)tk, q, k, v, o,
+      nullptr, 0, __builtin_bit_cast(float, scale_bits), sp, heads * D, kv_heads * D, rg);
+}
+#endif
+
+#define SVODK_ATTENTION_ENTRY(NAME, D, CAUSAL, F16)                                                                  \
+  extern "C" __global__ __launch_bounds__(256, (D) <= 64 ? 3 : 2) void NAME(                                          \
+      const uint16_t *__restrict__ q, const uint16_t *__restrict__ k, const uint16_t *__restrict__ v,                 \
+      uint16_t *__restrict__ o, const void *__restrict__ key_lens, int32_t batch, int32_t t, int32_t tk, int32_t heads, \
+      int32_t kv_heads, int32_t scale_bits) {                                                                         \
+    __shared__ __attribute__((aligned(1024))) uint8_t smem[Tile<D>::kLds];                                            \
+    attention_entry<D, CAUSAL, F16>(smem, q, k, v, o, key_lens, batch, t, tk, heads, kv_heads, scale_bits);           \
+  }
+
+SVODK_ATTENTION_ENTRY(svodk_attention_d32_bf16, 32, false, false)
+SVODK_ATTENTION_ENTRY(svodk_attention_d32_bf16_causal, 32, true, false)
+SVODK_ATTENTION_ENTRY(svodk_attention_d64_bf16, 64, false, false)
+SVODK_ATTENTION_ENTRY(svodk_attention_d64_bf16_causal, 64, true, false)
+SVODK_ATTENTION_ENTRY(svodk_attention_d128_bf16, 128, false, false)
+SVODK_ATTENTION_ENTRY(svodk_attention_d128_bf16_causal, 128, true, false)
+SVODK_ATTENTION_ENTRY(svodk_attention_d32_f16, 32, false, true)
+SVODK_ATTENTION_ENTRY(svodk_attention_d32_f16_causal, 32, true, true)
+SVODK_ATTENTION_ENTRY(svodk_attention_d64_f16, 64, false, true)
+SVODK_ATTENTION_ENTRY(svodk_attention_d64_f16_causal, 64, true, true)
+SVODK_ATTENTION_ENTRY(svodk_attention_d128_f16, 128, false, true)
+SVODK_ATTENTION_ENTRY(svodk_attention_d128_f16_causal, 128, true, true)
+#undef SVODK_ATTENTION_ENTRY
+
+}  // namespace
+}  // namespace svodk
+#endif  // SVODK_CODE_OBJECT

@@ -49,15 +49,14 @@ struct Div64 {
 // and every byte is touched once, so loads and stores are marked non-temporal.
 constexpr int kItems = 1;
 
+// The workgroup's program, for the kernels below to inline.
 template <int D, typename Div, bool F16>
-__global__ __launch_bounds__(kThreads) void heads_kernel(const uint16_t *__restrict__ qkv,
-                                                         const uint16_t *__restrict__ q_w,
-                                                         const uint16_t *__restrict__ k_w,
-                                                         const uint16_t *__restrict__ cos_t,
-                                                         const uint16_t *__restrict__ sin_t, uint16_t *__restrict__ q,
-                                                         uint16_t *__restrict__ k, uint16_t *__restrict__ v,
-                                                         int64_t items, Div by_slots, Div by_t, int32_t heads,
-                                                         int32_t kv_heads, float eps, int32_t rope) {
+__device__ __forceinline__ void heads_body(const uint16_t *__restrict__ qkv, const uint16_t *__restrict__ q_w,
+                                           const uint16_t *__restrict__ k_w, const uint16_t *__restrict__ cos_t,
+                                           const uint16_t *__restrict__ sin_t, uint16_t *__restrict__ q,
+                                           uint16_t *__restrict__ k, uint16_t *__restrict__ v, int64_t items,
+                                           const Div &by_slots, const Div &by_t, int32_t heads, int32_t kv_heads,
+                                           float eps, int32_t rope) {
 #pragma clang fp contract(off)
   typedef typename Div::index Index;
   constexpr int kHalf = D / 2;
@@ -158,6 +157,19 @@ __global__ __launch_bounds__(kThreads) void heads_kernel(const uint16_t *__restr
   }
 }
 
+#if !defined(SVODK_CODE_OBJECT)  // the library's kernel and its launch: not part of a code object build
+template <int D, typename Div, bool F16>
+__global__ __launch_bounds__(kThreads) void heads_kernel(const uint16_t *__restrict__ qkv,
+                                                         const uint16_t *__restrict__ q_w,
+                                                         const uint16_t *__restrict__ k_w,
+                                                         const uint16_t *__restrict__ cos_t,
+                                                         const uint16_t *__restrict__ sin_t, uint16_t *__restrict__ q,
+                                                         uint16_t *__restrict__ k, uint16_t *__restrict__ v,
+                                                         int64_t items, Div by_slots, Div by_t, int32_t heads,
+                                                         int32_t kv_heads, float eps, int32_t rope) {
+  heads_body<D, Div, F16>(qkv, q_w, k_w, cos_t, sin_t, q, k, v, items, by_slots, by_t, heads, kv_heads, eps, rope);
+}
+
 template <int D, bool F16>
 hipError_t launch(const HeadsArgs &a, hipStream_t stream) {
   constexpr int kLanes = D / 16;
@@ -207,3 +219,43 @@ hipError_t launch_heads(const HeadsArgs &a, hipStream_t stream) {
 }
 
 }  // namespace svodk
+
+#else  // SVODK_CODE_OBJECT
+// The prologue as kernels for a loader that takes a code object and a flat argument record
+// (device/src/amd/program.rs:403-414, 655-675; device/src/hcq.rs:1262-1285): buffers first, then
+// 4-byte scalars, nothing hidden, no launch geometry from the dispatch packet.
+// Parameters: qkv, q_w, k_w (address 0: that norm is off), cos, sin (unread when rope is 0), q, k, v,
+// then rows (batch * t), t, heads, kv_heads, eps_bits, rope (0 none, 1 a [t, D/2] table shared by
+// the batch, 2 a [rows, D/2] table).  Launch: ceil(rows * (heads + 2 kv_heads) * (D / 16) / 256)
+// workgroups of 256 threads; rows * (heads + 2 kv_heads) * (D / 16) < 2^32 - 256 is the caller's check.
+template <int D, bool F16>
+__device__ __forceinline__ void heads_entry(const uint16_t *qkv, const uint16_t *q_w, const uint16_t *k_w,
+                                            const uint16_t *cos_t, const uint16_t *sin_t, uint16_t *q, uint16_t *k,
+                                            uint16_t *v, int32_t rows, int32_t t, int32_t heads, int32_t kv_heads,
+                                            int32_t eps_bits, int32_t rope) {
+  if (rows <= 0 || heads < 0 || kv_heads < 0 || heads + 2 * kv_heads <= 0) return;
+  auto rcp = [](uint32_t d) { return d <= 1 ? 0xffffffffu : 0xffffffffu / d; };  // within one of floor(2^32 / d)
+  const uint32_t slots = (uint32_t)(heads + 2 * kv_heads), tt = (uint32_t)(t > 0 ? t : 1);
+  const Div32 by_slots = {slots, rcp(slots)}, by_t = {tt, rcp(tt)};
+  heads_body<D, Div32, F16>(qkv, q_w, k_w, cos_t, sin_t, q, k, v, (int64_t)rows * slots, by_slots, by_t, heads, kv_heads,
+                            __builtin_bit_cast(float, eps_bits), rope);
+}
+
+#define SVODK_HEADS_ENTRY(NAME, D, F16)                                                                              \
+  extern "C" __global__ __launch_bounds__(kThreads) void NAME(                                                        \
+      const uint16_t *__restrict__ qkv, const uint16_t *__restrict__ q_w, const uint16_t *__restrict__ k_w,           \
+      const uint16_t *__restrict__ cos_t, const uint16_t *__restrict__ sin_t, uint16_t *__restrict__ q,               \
+      uint16_t *__restrict__ k, uint16_t *__restrict__ v, int32_t rows, int32_t t, int32_t heads, int32_t kv_heads,   \
+      int32_t eps_bits, int32_t rope) {                                                                               \
+    heads_entry<D, F16>(qkv, q_w, k_w, cos_t, sin_t, q, k, v, rows, t, heads, kv_heads, eps_bits, rope);              \
+  }
+
+SVODK_HEADS_ENTRY(svodk_heads_d64_bf16, 64, false)
+SVODK_HEADS_ENTRY(svodk_heads_d128_bf16, 128, false)
+SVODK_HEADS_ENTRY(svodk_heads_d64_f16, 64, true)
+SVODK_HEADS_ENTRY(svodk_heads_d128_f16, 128, true)
+#undef SVODK_HEADS_ENTRY
+
+}  // namespace
+}  // namespace svodk
+#endif  // SVODK_CODE_OBJECT

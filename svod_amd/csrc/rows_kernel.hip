@@ -33,13 +33,12 @@ __device__ __forceinline__ u32x4 load_once(const u32x4 *p) { return __builtin_no
 __device__ __forceinline__ void store_once(u32x4 *p, const u32x4 &v) { __builtin_nontemporal_store(v, p); }
 
 // SPANS = ceil(d / 512): the 128-bit accesses a lane makes per row and tensor.
+// The workgroup's program, for the kernels below to inline.
 template <int SPANS, bool LAYER, bool RESIDUAL, bool BIAS, bool F16>
-__global__ __launch_bounds__(kRowsPerBlock * 64) void rows_kernel(const uint16_t *__restrict__ x,
-                                                                   const uint16_t *__restrict__ residual,
-                                                                   const uint16_t *__restrict__ w,
-                                                                   const uint16_t *__restrict__ b,
-                                                                   uint16_t *__restrict__ out, uint16_t *__restrict__ sum,
-                                                                   int64_t rows, int32_t d, float inv_d, float eps) {
+__device__ __forceinline__ void rows_body(const uint16_t *__restrict__ x, const uint16_t *__restrict__ residual,
+                                          const uint16_t *__restrict__ w, const uint16_t *__restrict__ b,
+                                          uint16_t *__restrict__ out, uint16_t *__restrict__ sum, int64_t rows, int32_t d,
+                                          float inv_d, float eps) {
   const int lane = threadIdx.x & 63;
   const int64_t row = (int64_t)blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
   if (row >= rows) return;
@@ -110,6 +109,17 @@ __global__ __launch_bounds__(kRowsPerBlock * 64) void rows_kernel(const uint16_t
   }
 }
 
+#if !defined(SVODK_CODE_OBJECT)  // the library's kernel and its launch: not part of a code object build
+template <int SPANS, bool LAYER, bool RESIDUAL, bool BIAS, bool F16>
+__global__ __launch_bounds__(kRowsPerBlock * 64) void rows_kernel(const uint16_t *__restrict__ x,
+                                                                   const uint16_t *__restrict__ residual,
+                                                                   const uint16_t *__restrict__ w,
+                                                                   const uint16_t *__restrict__ b,
+                                                                   uint16_t *__restrict__ out, uint16_t *__restrict__ sum,
+                                                                   int64_t rows, int32_t d, float inv_d, float eps) {
+  rows_body<SPANS, LAYER, RESIDUAL, BIAS, F16>(x, residual, w, b, out, sum, rows, d, inv_d, eps);
+}
+
 template <int SPANS, bool LAYER, bool RESIDUAL, bool BIAS, bool F16>
 hipError_t launch_rows(const NormArgs &a, hipStream_t stream) {
   const int64_t blocks = (a.rows + kRowsPerBlock - 1) / kRowsPerBlock;
@@ -157,3 +167,56 @@ hipError_t launch_norm(const NormArgs &a, hipStream_t stream) {
 }
 
 }  // namespace svodk
+
+#else  // SVODK_CODE_OBJECT
+// The row norms as kernels for a loader that takes a code object and a flat argument record
+// (device/src/amd/program.rs:403-414, 655-675; device/src/hcq.rs:1262-1285): buffers first, then
+// 4-byte scalars, nothing hidden.  A kernel covers the row lengths up to the one in its name
+// (d a multiple of 256).  Parameters, in the reference kernels' order (tk/src/kernels/rows.rs:41-50):
+//   rms_norm        x, w, out                    rows, d, eps_bits
+//   add_rms_norm    x, residual, w, out, sum     rows, d, eps_bits
+//   layer_norm      x, w, b, out                 rows, d, eps_bits
+//   add_layer_norm  x, residual, w, b, out, sum  rows, d, eps_bits
+// Launch: ceil(rows / 4) workgroups of 256 threads.
+#define SVODK_ROWS_ENTRIES(DMAX, TYPE, F16)                                                                           \
+  extern "C" __global__ __launch_bounds__(kRowsPerBlock * 64) void svodk_rms_norm_d##DMAX##_##TYPE(                    \
+      const uint16_t *__restrict__ x, const uint16_t *__restrict__ w, uint16_t *__restrict__ out, int32_t rows,         \
+      int32_t d, int32_t eps_bits) {                                                                                   \
+    if (d <= 0 || d > DMAX) return;                                                                                    \
+    rows_body<DMAX / kSpan, false, false, false, F16>(x, nullptr, w, nullptr, out, nullptr, rows, d, 1.0f / (float)d,  \
+                                                      __builtin_bit_cast(float, eps_bits));                            \
+  }                                                                                                                    \
+  extern "C" __global__ __launch_bounds__(kRowsPerBlock * 64) void svodk_add_rms_norm_d##DMAX##_##TYPE(                \
+      const uint16_t *__restrict__ x, const uint16_t *__restrict__ residual, const uint16_t *__restrict__ w,           \
+      uint16_t *__restrict__ out, uint16_t *__restrict__ sum, int32_t rows, int32_t d, int32_t eps_bits) {             \
+    if (d <= 0 || d > DMAX) return;                                                                                    \
+    rows_body<DMAX / kSpan, false, true, false, F16>(x, residual, w, nullptr, out, sum, rows, d, 1.0f / (float)d,      \
+                                                     __builtin_bit_cast(float, eps_bits));                             \
+  }                                                                                                                    \
+  extern "C" __global__ __launch_bounds__(kRowsPerBlock * 64) void svodk_layer_norm_d##DMAX##_##TYPE(                  \
+      const uint16_t *__restrict__ x, const uint16_t *__restrict__ w, const uint16_t *__restrict__ b,                  \
+      uint16_t *__restrict__ out, int32_t rows, int32_t d, int32_t eps_bits) {                                         \
+    if (d <= 0 || d > DMAX) return;                                                                                    \
+    rows_body<DMAX / kSpan, true, false, true, F16>(x, nullptr, w, b, out, nullptr, rows, d, 1.0f / (float)d,          \
+                                                    __builtin_bit_cast(float, eps_bits));                              \
+  }                                                                                                                    \
+  extern "C" __global__ __launch_bounds__(kRowsPerBlock * 64) void svodk_add_layer_norm_d##DMAX##_##TYPE(              \
+      const uint16_t *__restrict__ x, const uint16_t *__restrict__ residual, const uint16_t *__restrict__ w,           \
+      const uint16_t *__restrict__ b, uint16_t *__restrict__ out, uint16_t *__restrict__ sum, int32_t rows, int32_t d, \
+      int32_t eps_bits) {                                                                                              \
+    if (d <= 0 || d > DMAX) return;                                                                                    \
+    rows_body<DMAX / kSpan, true, true, true, F16>(x, residual, w, b, out, sum, rows, d, 1.0f / (float)d,              \
+                                                   __builtin_bit_cast(float, eps_bits));                               \
+  }
+
+SVODK_ROWS_ENTRIES(1024, bf16, false)
+SVODK_ROWS_ENTRIES(2048, bf16, false)
+SVODK_ROWS_ENTRIES(4096, bf16, false)
+SVODK_ROWS_ENTRIES(1024, f16, true)
+SVODK_ROWS_ENTRIES(2048, f16, true)
+SVODK_ROWS_ENTRIES(4096, f16, true)
+#undef SVODK_ROWS_ENTRIES
+
+}  // namespace
+}  // namespace svodk
+#endif  // SVODK_CODE_OBJECT

@@ -197,7 +197,7 @@ class CodeObject:
 
 def packed_size(params: Sequence[Tuple[str, str]]) -> int:
     """Bytes of the argument record: an address is 8 bytes, a scalar 4, each at its natural
-    alignment, in parameter order (device/src/hcq.rs:1275-1283)."""
+    alignment, in parameter order (device/src/hcq.rs:1278-1285)."""
     cursor = 0
     for _name, kind in params:
         width = 8 if kind == "buffer" else 4
@@ -207,7 +207,7 @@ def packed_size(params: Sequence[Tuple[str, str]]) -> int:
 
 def pack(params: Sequence[Tuple[str, str]], values: Dict[str, int], size: int) -> bytes:
     """The argument record for `values` (addresses and 32-bit scalars by parameter name), zero
-    filled to `size` bytes as the loader does (device/src/amd/program.rs:679-681)."""
+    filled to `size` bytes as the loader does (device/src/amd/program.rs:680)."""
     record = bytearray(size)
     cursor = 0
     for name, kind in params:
@@ -258,7 +258,7 @@ def check(data: bytes, kernel: str, params: Sequence[Tuple[str, str]]) -> Descri
         raise CodeObjectError(f"{kernel}: {kd.group_segment_fixed_size} bytes of LDS")
     if kd.private_segment_fixed_size:
         raise CodeObjectError(f"{kernel}: {kd.private_segment_fixed_size} bytes of scratch a lane (spills)")
-    # The entry is the descriptor's address plus this offset (program.rs:384), 256-byte aligned.
+    # The entry is the descriptor's address plus this offset (program.rs:387), 256-byte aligned.
     entry = co.symbols[kernel + ".kd"][0] + kd.kernel_code_entry_byte_offset
     if co.e_type == 3 and (kd.kernel_code_entry_byte_offset == 0 or entry % 256):
         raise CodeObjectError(f"{kernel}: entry at {entry:#x}")

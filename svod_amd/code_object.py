@@ -42,6 +42,7 @@ CO_DIR = Path(__file__).resolve().parent / "co"
 B, S = "buffer", "scalar"
 _ATTENTION = [("q", B), ("k", B), ("v", B), ("o", B), ("key_lens", B),
               ("batch", S), ("t", S), ("tk", S), ("heads", S), ("kv_heads", S), ("scale_bits", S)]
+_ATTENTION_MASK = [p if p[0] != "key_lens" else ("key_mask", B) for p in _ATTENTION]
 _HEADS = [("qkv", B), ("q_w", B), ("k_w", B), ("cos", B), ("sin", B), ("q", B), ("k", B), ("v", B),
           ("rows", S), ("t", S), ("heads", S), ("kv_heads", S), ("eps_bits", S), ("rope", S)]
 _TAIL = [("rows", S), ("d", S), ("eps_bits", S)]
@@ -66,11 +67,15 @@ def entries() -> Dict[str, dict]:
                     "op": "attention", "dtype": dtype, "head_dim": d, "causal": causal,
                     "cfg": f"FaCfg {{ bq: 128, bkv: 64, stages: 2, splits: 1, forms: {{ raw_max, skip_rescale }}, "
                            f"warp_rows: 32, core: mfma_f32_32x32x16_{dtype} }}"}
+                if d != 32:  # with a [batch, tk] byte mask in place of the lengths
+                    plain = out[f"svodk_attention_d{d}_{dtype}" + ("_causal" if causal else "")]
+                    out[f"svodk_attention_d{d}_{dtype}" + ("_causal" if causal else "") + "_mask"] = {
+                        **plain, "params": _ATTENTION_MASK, "key_mask": True}
         for d in (64, 128):
             out[f"svodk_heads_d{d}_{dtype}"] = {
                 "file": "svodk_heads.co", "source": "heads_kernel.hip", "params": _HEADS, "local": [256, 1, 1],
                 "workgroups": f"(rows * (heads + 2 * kv_heads) * {d // 16} + 255) // 256",
-                "op": "heads", "dtype": dtype, "head_dim": d, "cfg": "HeadsCfg { br: 1 }"}
+                "op": "heads", "dtype": dtype, "head_dim": d, "cfg": "NormCfg { lanes_per_head: d/16, block: 256 }"}
         for kind, params in _ROWS.items():
             for dmax in (1024, 2048, 4096):
                 out[f"svodk_{kind}_d{dmax}_{dtype}"] = {

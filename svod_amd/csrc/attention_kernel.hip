@@ -682,6 +682,7 @@ struct Ranges {
   int32_t kv_head_start;        // the first of the launch's kv heads in a cache row
   const void *row_map;          // [B] cache row per batch lane, or null: row b
   int32_t row_map_i64;
+  int32_t cache_rows;           // rows of the cache: a mapped row is held inside them
   const uint16_t *k_app, *v_app;  // [B, app_rows, kv_heads, D] scored after the cached keys, or null
   int32_t app_rows;             // at most a key block
   const void *app_lens;         // [B] visible appended rows, or null: all
@@ -871,8 +872,12 @@ __device__ __forceinline__ void flash_fwd_body(
   int64_t kv_row = b;
   int kv_col = kvh;
   if (CACHED) {
-    if (rg.row_map != nullptr)
-      kv_row = rg.row_map_i64 ? ((const long long *)rg.row_map)[b] : (long long)((const int *)rg.row_map)[b];
+    if (rg.row_map != nullptr) {
+      // The map is device data nobody has checked: a row outside the cache reads its nearest row
+      // instead of memory that is not there.
+      const long long x = rg.row_map_i64 ? ((const long long *)rg.row_map)[b] : (long long)((const int *)rg.row_map)[b];
+      kv_row = x < 0 ? 0 : (x < rg.cache_rows ? x : rg.cache_rows - 1);
+    }
     kv_col += rg.kv_head_start;
   }
   w.k_base = (const uint8_t *)(k + (kv_row * tk + first_key) * kv_row_elems + (int64_t)kv_col * D);
@@ -1553,6 +1558,7 @@ hipError_t launch(const AttnArgs &a, hipStream_t stream) {
   rg.kv_head_start = a.kv_head_start;
   rg.row_map = a.row_map;
   rg.row_map_i64 = a.row_map_i64;
+  rg.cache_rows = a.cache_rows;
   rg.k_app = (const uint16_t *)a.k_app;
   rg.v_app = (const uint16_t *)a.v_app;
   rg.app_rows = a.app_rows;
@@ -1698,8 +1704,9 @@ hipError_t launch_attention(const AttnArgs &a, hipStream_t stream) {
 // into registers (a loader that writes its own user registers hands over the record's address only).
 //
 // Parameters follow the reference kernel's order (tk/src/kernels/attention.rs:308-327, 452-459):
-// q, k, v, o, then key_lens ([batch] i32, or address 0 for none), then the scalars
-// batch, t, tk, heads, kv_heads, scale_bits.  Launch: workgroups
+// q, k, v, o, then key_lens ([batch] i32, or address 0 for none) or, for the `_mask` kernels,
+// key_mask ([batch, tk] bytes, a key visible where its byte is not 0: a Bool tensor as it lies in
+// memory), then the scalars batch, t, tk, heads, kv_heads, scale_bits.  Launch: workgroups
 // [ceil(batch * kv_heads, 8) * (heads / kv_heads) * ceil(t / 128), 1, 1] of [256, 1, 1] threads.
 // The host side's checks are the caller's: heads a multiple of kv_heads, heads < 65536, dimensions
 // positive, tk * kv_heads * D * 2 < 2^31.
@@ -1710,8 +1717,9 @@ __device__ __forceinline__ uint32_t rcp_for(uint32_t d) { return d <= 1 ? 0xffff
 
 template <int D, bool CAUSAL, bool F16>
 __device__ __forceinline__ void attention_entry(uint8_t *smem, const uint16_t *q, const uint16_t *k, const uint16_t *v,
-                                                uint16_t *o, const void *key_lens, int32_t batch, int32_t t,
-                                                int32_t tk, int32_t heads, int32_t kv_heads, int32_t scale_bits) {
+                                                uint16_t *o, const void *key_lens, const void *key_mask, int32_t batch,
+                                                int32_t t, int32_t tk, int32_t heads, int32_t kv_heads,
+                                                int32_t scale_bits) {
   constexpr int NW = 4;
   if (batch <= 0 || t <= 0 || tk < 0 || kv_heads <= 0 || heads < kv_heads) return;
   const uint32_t group = (uint32_t)heads / (uint32_t)kv_heads;
@@ -1724,7 +1732,7 @@ __device__ __forceinline__ void attention_entry(uint8_t *smem, const uint16_t *q
   flash_fwd_body<D, NW, CAUSAL, false, false, false, false, false, F16>(
       smem, unit_size, rcp_for(unit_size), nqt, rcp_for(nqt), (uint32_t)kv_heads, rcp_for((uint32_t)kv_heads),
       (uint32_t)kv_heads * (uint32_t)batch, (uint32_t)heads | group << 16, key_lens, nullptr, t, (uint32_t)tk, q, k, v, o,
-      nullptr, 0, __builtin_bit_cast(float, scale_bits), sp, heads * D, kv_heads * D, rg);
+      key_mask, 1, __builtin_bit_cast(float, scale_bits), sp, heads * D, kv_heads * D, rg);
 }
 #endif
 
@@ -1734,7 +1742,17 @@ __device__ __forceinline__ void attention_entry(uint8_t *smem, const uint16_t *q
       uint16_t *__restrict__ o, const void *__restrict__ key_lens, int32_t batch, int32_t t, int32_t tk, int32_t heads, \
       int32_t kv_heads, int32_t scale_bits) {                                                                         \
     __shared__ __attribute__((aligned(1024))) uint8_t smem[Tile<D>::kLds];                                            \
-    attention_entry<D, CAUSAL, F16>(smem, q, k, v, o, key_lens, batch, t, tk, heads, kv_heads, scale_bits);           \
+    attention_entry<D, CAUSAL, F16>(smem, q, k, v, o, key_lens, nullptr, batch, t, tk, heads, kv_heads, scale_bits);  \
+  }
+
+// Behind the ring, the words of the scanned key mask row: a copy a wave.
+#define SVODK_ATTENTION_MASK_ENTRY(NAME, D, CAUSAL, F16)                                                             \
+  extern "C" __global__ __launch_bounds__(256, (D) <= 64 ? 3 : 2) void NAME(                                          \
+      const uint16_t *__restrict__ q, const uint16_t *__restrict__ k, const uint16_t *__restrict__ v,                 \
+      uint16_t *__restrict__ o, const void *__restrict__ key_mask, int32_t batch, int32_t t, int32_t tk, int32_t heads, \
+      int32_t kv_heads, int32_t scale_bits) {                                                                         \
+    __shared__ __attribute__((aligned(1024))) uint8_t smem[Tile<D>::kLds + 4 * kScannedBlocks * 8];                   \
+    attention_entry<D, CAUSAL, F16>(smem, q, k, v, o, nullptr, key_mask, batch, t, tk, heads, kv_heads, scale_bits);  \
   }
 
 SVODK_ATTENTION_ENTRY(svodk_attention_d32_bf16, 32, false, false)
@@ -1749,7 +1767,16 @@ SVODK_ATTENTION_ENTRY(svodk_attention_d64_f16, 64, false, true)
 SVODK_ATTENTION_ENTRY(svodk_attention_d64_f16_causal, 64, true, true)
 SVODK_ATTENTION_ENTRY(svodk_attention_d128_f16, 128, false, true)
 SVODK_ATTENTION_ENTRY(svodk_attention_d128_f16_causal, 128, true, true)
+SVODK_ATTENTION_MASK_ENTRY(svodk_attention_d64_bf16_mask, 64, false, false)
+SVODK_ATTENTION_MASK_ENTRY(svodk_attention_d64_bf16_causal_mask, 64, true, false)
+SVODK_ATTENTION_MASK_ENTRY(svodk_attention_d128_bf16_mask, 128, false, false)
+SVODK_ATTENTION_MASK_ENTRY(svodk_attention_d128_bf16_causal_mask, 128, true, false)
+SVODK_ATTENTION_MASK_ENTRY(svodk_attention_d64_f16_mask, 64, false, true)
+SVODK_ATTENTION_MASK_ENTRY(svodk_attention_d64_f16_causal_mask, 64, true, true)
+SVODK_ATTENTION_MASK_ENTRY(svodk_attention_d128_f16_mask, 128, false, true)
+SVODK_ATTENTION_MASK_ENTRY(svodk_attention_d128_f16_causal_mask, 128, true, true)
 #undef SVODK_ATTENTION_ENTRY
+#undef SVODK_ATTENTION_MASK_ENTRY
 
 }  // namespace
 }  // namespace svodk

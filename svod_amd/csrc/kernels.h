@@ -92,6 +92,7 @@ struct AttnArgs {
   int32_t kv_head_start;
   const void *row_map;
   int32_t row_map_i64;
+  int32_t cache_rows;  // k's leading dim: mapped rows are clamped into it
   const void *k_app, *v_app;
   int32_t app_rows;
   const void *app_lens;

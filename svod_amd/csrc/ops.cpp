@@ -530,8 +530,13 @@ static int attend(const svodk_tensor *q, const svodk_tensor *k, const svodk_tens
     a.kv_head_start = (int32_t)cache->head_start;
     if (cache->row_map != nullptr) {
       if (cache->row_map->data == nullptr) return fail(SVODK_ERR_ARGUMENT, "%s: a null device pointer", op);
+      if (k->shape[0] > 0x7fffffff) return ran_graph(op, SVODK_GRAPH_SHAPE);
       a.row_map = cache->row_map->data;
       a.row_map_i64 = cache->row_map->dtype == SVODK_I64;
+      a.cache_rows = (int32_t)k->shape[0];
+      Span pair[2] = {{"row_map", a.row_map, (size_t)numel(cache->row_map) * dtype_bytes(cache->row_map->dtype), false},
+                      spans[3]};
+      if (int rc = check_aliasing(op, pair, 2)) return rc;
     }
     if (cache->k_app != nullptr) {
       if (cache->k_app->data == nullptr || cache->v_app->data == nullptr ||
@@ -548,6 +553,10 @@ static int attend(const svodk_tensor *q, const svodk_tensor *k, const svodk_tens
       if (cache->app_lens != nullptr) {
         a.app_lens = cache->app_lens->data;
         a.app_lens_i64 = cache->app_lens->dtype == SVODK_I64;
+        Span pair[2] = {{"appended lens", a.app_lens, (size_t)numel(cache->app_lens) * dtype_bytes(cache->app_lens->dtype),
+                         false},
+                        spans[3]};
+        if (int rc = check_aliasing(op, pair, 2)) return rc;
       }
     }
   }
@@ -628,7 +637,8 @@ int svodk_attention_packed(const svodk_tensor *qkv, int32_t heads, int32_t kv_he
 
 void svodk_tune_streaming(int32_t workgroups_per_xcd) { svodk::attention_stream_slots(workgroups_per_xcd); }
 
-// The workspace of a split call (tk/src/ops/attention.rs:285-293).
+// The batch rows by descending key count, for svodk_attn.row_order (no counterpart in the reference,
+// whose grid fixes what a block computes and leaves the order of blocks to the hardware).
 int svodk_order_rows(const svodk_tensor *keys, const svodk_tensor *order, void *hip_stream) {
   const char *op = "order_rows";
   if (!well_formed(keys) || !well_formed(order))
@@ -657,6 +667,7 @@ int svodk_order_rows(const svodk_tensor *keys, const svodk_tensor *order, void *
   return SVODK_KERNEL;
 }
 
+// The workspace of a split call (tk/src/ops/attention.rs:285-293).
 int64_t svodk_attention_workspace(const svodk_tensor *q, const svodk_tensor *k, const svodk_attn *opts) {
   if (!well_formed(q) || !well_formed(k) || opts == nullptr || q->rank != 4 || k->rank != 4) return 0;
   const int64_t batch = opts->batch_live > 0 ? opts->batch_live : q->shape[0];

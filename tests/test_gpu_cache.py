@@ -106,6 +106,24 @@ def test_a_cache_without_appended_rows_is_a_view_of_its_heads(device):
         assert np.array_equal(bits(cached), bits(plain))
 
 
+def test_a_mapped_row_outside_the_cache_reads_its_nearest_row(device):
+    """The map is device data no host check sees: rows past the cache's ends are held inside it, so a
+    bad map gives the result of a clamped one instead of a read of memory that is not there."""
+    t, d, h, tk = 40, 64, 4, 300
+    q, k, v, _, _, _, lens, _, _ = operands(t, d, h, tk, 1)
+    dev = lambda x: bf16_tensor(x, device)
+    ints = lambda a, dt=torch.int32: torch.tensor(a, dtype=dt, device=device)
+    rows = k.shape[0]
+    wild = np.array([-3, rows, 0, 2 ** 31 - 1, rows - 1][:B] + [0] * max(0, B - 5))
+    tame = np.clip(wild, 0, rows - 1)
+    for dt in (torch.int32, torch.int64):
+        got = svod_amd.attention(dev(q), dev(k), dev(v), Attn(keys=KeyMask.lens(ints(lens)),
+                                                             cache=Cache(2 * h, h, row_map=ints(wild, dt))))
+        want = svod_amd.attention(dev(q), dev(k), dev(v), Attn(keys=KeyMask.lens(ints(lens)),
+                                                              cache=Cache(2 * h, h, row_map=ints(tame, dt))))
+        assert np.array_equal(bits(got), bits(want))
+
+
 def test_what_the_cache_has_no_kernel_for_keeps_the_graph(device):
     t, d, h, tk = 4, 64, 4, 100
     q, k, v, _, _, _, lens, row_map, _ = operands(t, d, h, tk, 1)

@@ -99,6 +99,29 @@ def test_attention_code_object_equals_the_library(device, runtime, name, b, t, t
     assert np.array_equal(bits(got), bits(want))
 
 
+@pytest.mark.parametrize("d,causal,f16,tk", [(64, False, False, 200), (128, True, False, 300), (64, True, True, 130),
+                                             (128, False, True, 70), (64, False, False, 64 * 300)],
+                         ids=["d 64", "d 128 causal", "f16 d 64 causal", "f16 d 128", "a row too long to scan up front"])
+def test_key_mask_code_object_equals_the_library(device, runtime, d, causal, f16, tk):
+    """The fixture of tk/src/test/unit/attention.rs:80: key j of batch row b is hidden iff (b + j) % 5 == 2;
+    one row sees nothing."""
+    b, t, h, hkv = 3, min(tk, 200), 4, 2
+    g = Lcg(5)
+    q, k, v = (tensor(g.bf16(s), device, f16) for s in ((b, t, h, d), (b, tk, hkv, d), (b, tk, hkv, d)))
+    mask = np.array([[(i + j) % 5 != 2 for j in range(tk)] for i in range(b)])
+    mask[1] = False
+    mask_t = torch.from_numpy(mask).to(device)
+    want = svod_amd.attention(q, k, v, Attn(causal=causal, keys=KeyMask.bool(mask_t), splits=1))
+    assert "flash_attention" in svod_amd.chosen()
+    got = torch.full_like(want, 7.0)
+    kernel = f"svodk_attention_d{d}_{'f16' if f16 else 'bf16'}" + ("_causal" if causal else "") + "_mask"
+    runtime.launch(kernel, {"q": q.data_ptr(), "k": k.data_ptr(), "v": v.data_ptr(), "o": got.data_ptr(),
+                            "key_mask": mask_t.data_ptr(), "batch": b, "t": t, "tk": tk, "heads": h, "kv_heads": hkv,
+                            "scale_bits": f32_bits(d ** -0.5)})
+    assert np.array_equal(bits(got), bits(want))
+    assert not bits(got[1]).any()
+
+
 @pytest.mark.parametrize("d,f16,rope,norms", [(128, False, 1, True), (64, False, 2, True), (128, True, 1, False),
                                               (64, True, 0, True)],
                          ids=["d 128, shared table", "d 64, a table row per token", "f16 without norms", "f16 without rope"])

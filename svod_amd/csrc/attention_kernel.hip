@@ -89,21 +89,35 @@ std::atomic<uint32_t> g_queue_turn{0};
 //     over 4 rows modulo the period.
 // K runs one block ahead of V, so each has its own pair of slots:
 // LDS = [K slot 0][K slot 1][V slot 0][V slot 1].
+// A head of 48 takes the 64-wide tile: a row's last two chunks are never fetched (their lanes
+// read past the descriptor's bound and land zeros), the score product stops at the third
+// k-step, and the second half of O^T's second row block is dropped at the store.
 template <int D>
 struct Tile {
-  static constexpr int kRowBytes = D * 2;
-  static constexpr int kCpr = D / 8;  // 16-byte chunks per row
+  static constexpr int kWide = D == 48 ? 64 : D;  // the head size the tile is laid out for
+  static constexpr int kRowBytes = kWide * 2;
+  static constexpr int kCpr = kWide / 8;   // 16-byte chunk places per row of the tile
+  static constexpr int kChunks = D / 8;    // chunks a row holds in memory
   static constexpr int kBytes = kBkv * kRowBytes;
   static constexpr int kLds = 4 * kBytes;
   static constexpr int kInstrs = kBytes / 1024;  // wave-wide 1 KiB fills per tile
-  // D = 32: rows are 64 bytes, four to the bank period, so 16 rows at one logical chunk spread over
+  // 32 wide: rows are 64 bytes, four to the bank period, so 16 rows at one logical chunk spread over
   // the period's 16 chunk places when the chunk is xor-ed with row / 4; a V row is one 64-byte
   // group and four consecutive rows are the whole period as they lie.
   __device__ static constexpr int swz_k(int row) {
-    return D == 32 ? ((row >> 2) & 3) : D == 64 ? ((row >> 1) & 7) : (row & 15);
+    return kWide == 32 ? ((row >> 2) & 3) : kWide == 64 ? ((row >> 1) & 7) : (row & 15);
   }
   // In units of 64-byte groups (4 chunks).
-  __device__ static constexpr int swz_v(int row) { return D == 32 ? 0 : D == 64 ? ((row >> 1) & 1) : (row & 3); }
+  __device__ static constexpr int swz_v(int row) {
+    return kWide == 32 ? 0 : kWide == 64 ? ((row >> 1) & 1) : (row & 3);
+  }
+  // The byte offset, from a fill instruction's first row, of what the lane at chunk place `pc` of
+  // tile row `row` fetches: logical chunk pc ^ swizzle of that row of memory, or an offset past any
+  // descriptor's bound where the row has no such chunk.
+  __device__ static int source(int row, int pc, int row_bytes, bool v) {
+    const int chunk = pc ^ (v ? swz_v(row) << 2 : swz_k(row));
+    return chunk < kChunks ? row * row_bytes + (chunk << 4) : (int)0xfffffff0u;
+  }
 };
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
@@ -171,8 +185,8 @@ constexpr unsigned kBiased = 4;  // an additive bias joins the scaled scores
 // Everything a wave carries through the key loop.
 template <int D, int NW, bool F16, unsigned FLAGS>
 struct Wave {
-  static constexpr int KS = D / 16;  // k-steps of the score product
-  static constexpr int DB = D / 32;  // 32-row blocks of O^T
+  static constexpr int KS = D / 16;               // k-steps of the score product
+  static constexpr int DB = Tile<D>::kWide / 32;  // 32-row blocks of O^T
   static constexpr int CH = Tile<D>::kInstrs / NW;  // fills per wave per tile
   // block constants
   const uint8_t *k_base, *v_base;
@@ -891,8 +905,8 @@ __device__ __forceinline__ void flash_fwd_body(
   {
     const int row = w.wave * kRowsPer + w.lane / TL::kCpr;
     const int pc = w.lane % TL::kCpr;
-    w.k_src = row * w.kv_row_bytes + ((pc ^ TL::swz_k(row)) << 4);
-    w.v_src = row * w.kv_row_bytes + ((pc ^ (TL::swz_v(row) << 2)) << 4);
+    w.k_src = TL::source(row, pc, w.kv_row_bytes, false);
+    w.v_src = TL::source(row, pc, w.kv_row_bytes, true);
   }
   // ---- K(0), V(0), K(1) go first: everything below runs in the shadow of their flight.
   w.nxt_end = 0;  // one item a workgroup
@@ -1037,8 +1051,8 @@ __device__ __forceinline__ void flash_fwd_body(
       {
         const int frow = w.wave * kRowsPer + w.lane / TL::kCpr;
         const int pc = w.lane % TL::kCpr;
-        const int k_src = frow * app_row_bytes + ((pc ^ TL::swz_k(frow)) << 4);
-        const int v_src = frow * app_row_bytes + ((pc ^ (TL::swz_v(frow) << 2)) << 4);
+        const int k_src = TL::source(frow, pc, app_row_bytes, false);
+        const int v_src = TL::source(frow, pc, app_row_bytes, true);
         fill_tile<D, NW>(w, (const uint8_t *)(rg.k_app + at), bytes, 0, w.lds0, k_src, app_row_bytes);
         fill_tile<D, NW>(w, (const uint8_t *)(rg.v_app + at), bytes, 0, w.lds0 + 2 * TL::kBytes, v_src, app_row_bytes);
       }
@@ -1084,6 +1098,7 @@ __device__ __forceinline__ void flash_fwd_body(
       for (int db = 0; db < DB; db++) {
 #pragma unroll
         for (int c = 0; c < 4; c++) {
+          if (32 * db + 8 * c >= D) continue;  // the tile's columns past the head
           const f32x4 x = {w.acc[db][4 * c], w.acc[db][4 * c + 1], w.acc[db][4 * c + 2], w.acc[db][4 * c + 3]};
           *reinterpret_cast<f32x4 *>(o_ptr + 32 * db + 8 * c) = x;
         }
@@ -1099,6 +1114,7 @@ __device__ __forceinline__ void flash_fwd_body(
     for (int db = 0; db < DB; db++) {
 #pragma unroll
       for (int c = 0; c < 4; c++) {
+        if (32 * db + 8 * c >= D) continue;  // the tile's columns past the head
         u32x2 x;
         x[0] = pack2<F16>(w.acc[db][4 * c] * inv, w.acc[db][4 * c + 1] * inv);
         x[1] = pack2<F16>(w.acc[db][4 * c + 2] * inv, w.acc[db][4 * c + 3] * inv);
@@ -1248,8 +1264,8 @@ __global__ __launch_bounds__(NW * 64, 3) void flash_stream_kernel(
   {
     const int row = w.wave * kRowsPer + w.lane / TL::kCpr;
     const int pc = w.lane % TL::kCpr;
-    w.k_src = row * w.kv_row_bytes + ((pc ^ TL::swz_k(row)) << 4);
-    w.v_src = row * w.kv_row_bytes + ((pc ^ (TL::swz_v(row) << 2)) << 4);
+    w.k_src = TL::source(row, pc, w.kv_row_bytes, false);
+    w.v_src = TL::source(row, pc, w.kv_row_bytes, true);
   }
 #pragma unroll
   for (int ks = 0; ks < KS; ks++) w.k_read[ks] = ln * TL::kRowBytes + (((2 * ks + w.g) ^ TL::swz_k(ln)) << 4);
@@ -1654,7 +1670,7 @@ hipError_t launch_order_rows(const void *keys, int32_t elem_bytes, int32_t n, in
   return hipGetLastError();
 }
 
-bool attention_supports(int32_t d) { return d == 32 || d == 64 || d == 128; }
+bool attention_supports(int32_t d) { return d == 32 || d == 48 || d == 64 || d == 128; }
 
 bool attention_groups(const AttnArgs &a) {
   const bool ranged = a.win_left >= 0 || a.chunk_size > 0 || a.seg_start != nullptr;
@@ -1680,6 +1696,7 @@ const char *attention_config(const AttnArgs &a) {
 hipError_t launch_attention(const AttnArgs &a, hipStream_t stream) {
   switch (a.d) {
     case 32: return launch_d<32>(a, stream);
+    case 48: return launch_d<48>(a, stream);
     case 64: return launch_d<64>(a, stream);
     case 128: return launch_d<128>(a, stream);
     default: return hipErrorInvalidValue;

@@ -80,6 +80,7 @@ hipError_t launch_combine(const CombineArgs &a, hipStream_t stream) {
   if (a.splits < 1) return hipErrorInvalidValue;
   switch (a.d) {
     case 32: return a.f16 ? launch<32, true>(a, stream) : launch<32, false>(a, stream);
+    case 48: return a.f16 ? launch<48, true>(a, stream) : launch<48, false>(a, stream);
     case 64: return a.f16 ? launch<64, true>(a, stream) : launch<64, false>(a, stream);
     case 128: return a.f16 ? launch<128, true>(a, stream) : launch<128, false>(a, stream);
     default: return hipErrorInvalidValue;

@@ -47,8 +47,10 @@ def run(device, t, d, h, tk, splits, appended, counted, biased, int_dtype=torch.
     return got, p
 
 
-# ([t, d, h, tk], splits, appended, counted, biased): ops.rs:585-591, d 48 run at 64
+# ([t, d, h, tk], splits, appended, counted, biased): ops.rs:585-591 (the d 48 cases also at 64)
 CASES = [
+    ("a streaming chunk: eight queries, eight appended, d 48", [8, 48, 16, 128], None, 8, False, False),
+    ("sixteen counted appended, two splits, d 48", [16, 48, 16, 128], 2, 16, True, False),
     ("one query, 1500 keys, four splits", [1, 64, 20, 1500], 4, 1, False, False),
     ("d 128 unsplit", [1, 128, 8, 300], None, 1, False, False),
     ("three queries, two splits", [3, 64, 4, 200], 2, 1, False, False),

@@ -38,6 +38,8 @@ CASES = [
      dict(causal=True, window=(50, 0), chunk=(32, 3, 0), seg=40, key_mask=True), [128, 100], None),      # attention.rs:288-295
     ("causal packed segments, gqa", 2, 200, 200, 4, 2, 64, dict(causal=True, seg=30), None, None),       # ops.rs:444
     ("chunks of 8, sixteen behind, lens", 2, 300, 300, 4, 4, 64, dict(chunk=(8, 16, 0)), [300, 171], None),  # ops.rs:452
+    ("d48 chunks of 8, sixteen behind, lens", 2, 300, 300, 4, 4, 48, dict(chunk=(8, 16, 0)), [300, 171], None),  # ops.rs:452
+    ("d48 causal segments bool mask", 1, 96, 96, 4, 4, 48, dict(causal=True, seg=40, key_mask=True), None, None),  # ops.rs:445
     ("chunks of 24, every earlier one and one ahead", 2, 200, 200, 4, 2, 64, dict(chunk=(24, None, 1)), None, None),
     ("d128 chunks with a bool mask", 1, 100, 100, 4, 4, 128, dict(chunk=(16, 1, 0), key_mask=True), None, None),
     ("long segments, d128", 1, 900, 900, 2, 1, 128, dict(causal=True, seg=333), None, None),

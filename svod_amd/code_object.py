@@ -58,7 +58,7 @@ def entries() -> Dict[str, dict]:
     the config it stands for in the reference's terms."""
     out: Dict[str, dict] = {}
     for dtype in ("bf16", "f16"):
-        for d in (32, 64, 128):
+        for d in (32, 48, 64, 128):
             for causal in (False, True):
                 out[f"svodk_attention_d{d}_{dtype}" + ("_causal" if causal else "")] = {
                     "file": "svodk_attention.co", "source": "attention_kernel.hip", "params": _ATTENTION,
@@ -67,7 +67,7 @@ def entries() -> Dict[str, dict]:
                     "op": "attention", "dtype": dtype, "head_dim": d, "causal": causal,
                     "cfg": f"FaCfg {{ bq: 128, bkv: 64, stages: 2, splits: 1, forms: {{ raw_max, skip_rescale }}, "
                            f"warp_rows: 32, core: mfma_f32_32x32x16_{dtype} }}"}
-                if d != 32:  # with a [batch, tk] byte mask in place of the lengths
+                if d >= 64:  # with a [batch, tk] byte mask in place of the lengths
                     plain = out[f"svodk_attention_d{d}_{dtype}" + ("_causal" if causal else "")]
                     out[f"svodk_attention_d{d}_{dtype}" + ("_causal" if causal else "") + "_mask"] = {
                         **plain, "params": _ATTENTION_MASK, "key_mask": True}

@@ -1774,12 +1774,16 @@ __device__ __forceinline__ void attention_entry(uint8_t *smem, const uint16_t *q
 
 SVODK_ATTENTION_ENTRY(svodk_attention_d32_bf16, 32, false, false)
 SVODK_ATTENTION_ENTRY(svodk_attention_d32_bf16_causal, 32, true, false)
+SVODK_ATTENTION_ENTRY(svodk_attention_d48_bf16, 48, false, false)
+SVODK_ATTENTION_ENTRY(svodk_attention_d48_bf16_causal, 48, true, false)
 SVODK_ATTENTION_ENTRY(svodk_attention_d64_bf16, 64, false, false)
 SVODK_ATTENTION_ENTRY(svodk_attention_d64_bf16_causal, 64, true, false)
 SVODK_ATTENTION_ENTRY(svodk_attention_d128_bf16, 128, false, false)
 SVODK_ATTENTION_ENTRY(svodk_attention_d128_bf16_causal, 128, true, false)
 SVODK_ATTENTION_ENTRY(svodk_attention_d32_f16, 32, false, true)
 SVODK_ATTENTION_ENTRY(svodk_attention_d32_f16_causal, 32, true, true)
+SVODK_ATTENTION_ENTRY(svodk_attention_d48_f16, 48, false, true)
+SVODK_ATTENTION_ENTRY(svodk_attention_d48_f16_causal, 48, true, true)
 SVODK_ATTENTION_ENTRY(svodk_attention_d64_f16, 64, false, true)
 SVODK_ATTENTION_ENTRY(svodk_attention_d64_f16_causal, 64, true, true)
 SVODK_ATTENTION_ENTRY(svodk_attention_d128_f16, 128, false, true)

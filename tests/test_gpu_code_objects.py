@@ -78,6 +78,7 @@ ATTENTION = [
     ("Qwen3's kind: causal, grouped heads, d 128", 2, 300, 300, 8, 2, 128, True, [300, 130], False, None),
     ("no lengths (address 0), 11 units over 8 XCDs", 11, 130, 130, 1, 1, 64, False, None, False, None),
     ("f16, d 32, causal", 2, 100, 100, 4, 2, 32, True, None, True, None),
+    ("d 48, lengths", 2, 150, 150, 4, 4, 48, False, [150, 100], False, None),
     ("f16 d 128, a scale of its own", 1, 64, 257, 2, 2, 128, False, [201], True, 0.05),
     ("cross attention, d 64 causal, queries longer than keys", 2, 260, 70, 2, 1, 64, True, None, False, None),
 ]

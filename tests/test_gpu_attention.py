@@ -223,3 +223,44 @@ def test_a_key_mask_row_too_long_to_scan(device):
     split = svod_amd.attention(dq, dk, dv, Attn(keys=keys))  # split unasked: every split scans its share
     assert "combine_splits" in svod_amd.chosen()
     assert max_abs(to_np(split), want) < 2e-2
+
+
+@pytest.mark.parametrize("per_key,causal,d", [(0.1, False, 64), (1.0, False, 64), (0.1, True, 64), (0.4, False, 128),
+                                               (-0.5, False, 64)],
+                         ids=["a slow climb", "a steep climb", "a slow causal climb", "d 128", "a descent"])
+def test_climbing_scores_rescale_the_accumulator(device, per_key, causal, d):
+    """attention.rs:457-472 with the climb in the scores themselves (its bias-ramp form is in
+    test_gpu_bias.py): key j scores per_key * j in log2 units against every query, so a row keeps its
+    stale maximum for several blocks and then adopts a new one (slowly), or adopts one every block
+    (steeply); the accumulator is rescaled while it holds earlier blocks' work.  A descent never rescales."""
+    b, t, tk, h = 2, 256, 512, 2
+    g = Lcg(5)
+    q, k, v = g.bf16((b, t, h, d)), g.bf16((b, tk, h, d)), g.bf16((b, tk, h, d))
+    # One coordinate carries the ramp: q[..., 0] = 1, k[j, ..., 0] = ramp(j); the others stay small noise.
+    q[..., 0] = 1.0
+    ramp = oracle.round_bf16((per_key * np.arange(tk) / (d ** -0.5 * 1.4426950408889634)).astype(np.float32))
+    k[..., 0] = ramp[None, :, None]
+    q[..., 1:] *= 0.25
+    lens = [tk, 300]
+    got = to_np(run(device, q, k, v, causal=causal, lens=lens))
+    p = oracle.AttnProblem(q, k, v, causal=causal, key_lens=np.asarray(lens))
+    assert_bf16_parity("climbing scores", got, oracle.attention_direct(p), oracle.attention_flash(p, bq=128, bkv=64))
+
+
+def test_a_non_finite_unread_element_never_reaches_the_output(device):
+    """attention.rs:572-592 on plain operands: rows of K and V at and past a batch row's length may
+    hold anything, an infinity or a NaN included, as memory nothing initialised does; the kernel reads
+    zeros there (the last key block is partial), never those elements."""
+    b, t, tk, h, d = 2, 100, 200, 4, 64
+    q, k, v = reference_case(t, tk, d, heads=h, kv_heads=h, batch=b)
+    lens = [100, 37]
+    clean = run(device, q, k, v, lens=lens)
+    for x in (k, v):
+        x[0, 100:] = np.nan
+        x[1, 37:] = np.inf
+        x[1, 38::2] = np.nan
+    dirty = run(device, q, k, v, lens=lens)
+    assert np.isfinite(to_np(dirty)).all()
+    assert np.array_equal(bits(dirty), bits(clean))
+    for causal in (True,):
+        assert np.isfinite(to_np(run(device, q, k, v, causal=causal, lens=lens))).all()

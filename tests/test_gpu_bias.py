@@ -121,3 +121,22 @@ def test_a_bias_off_the_stream_dtype_keeps_the_graph(device):
         svod_amd.attention(bf16_tensor(q, device), bf16_tensor(k, device), bf16_tensor(v, device),
                            Attn(bias=torch.from_numpy(bias).to(torch.float16).to(device)))
     assert e.value.why == svod_amd.Fallback.Dtype
+
+
+@pytest.mark.parametrize("per_key,causal", [(0.1, False), (1.0, False), (0.1, True)],
+                         ids=["a slow climb", "a steep climb", "a slow causal climb"])
+def test_climbing_scores_rescale_the_accumulator(device, per_key, causal):
+    """attention.rs:457-472: a bias ramp along the keys (per_key * j, rounded to bf16).  Slowly, a row keeps
+    its stale maximum for several blocks and then adopts a new one; steeply, it adopts one every block.
+    Either way the accumulator is rescaled while it holds earlier blocks' work.  384 keys here (the
+    reference's 128 are two of this kernel's key blocks)."""
+    b, t, tk, h, d = 2, 128, 384, 2, 64
+    q, k, v, _ = case(b, t, tk, h, h, d, b)
+    ramp = oracle.round_bf16((per_key * np.arange(tk)).astype(np.float32))
+    bias = np.ascontiguousarray(np.broadcast_to(ramp, (b, h, t, tk))).astype(np.float32)
+    got = svod_amd.attention(bf16_tensor(q, device), bf16_tensor(k, device), bf16_tensor(v, device),
+                             Attn(causal=causal, bias=bf16_tensor(bias, device)))
+    torch.cuda.synchronize()
+    assert svod_amd.chosen().startswith('Kernel { op: "attention"'), svod_amd.chosen()
+    p = oracle.AttnProblem(q, k, v, causal=causal, bias=bias)
+    assert_bf16_parity("climbing bias", to_np(got), oracle.attention_direct(p), oracle.attention_flash(p, bq=128, bkv=64))

@@ -138,3 +138,34 @@ def test_what_the_cache_has_no_kernel_for_keeps_the_graph(device):
         with pytest.raises(svod_amd.GraphFallback) as e:
             svod_amd.attention(dev(q), dev(k), dev(v), opts)
         assert e.value.why == svod_amd.Fallback.Config
+
+
+@pytest.mark.parametrize("splits", [None, 4], ids=["whole", "a decoder step over four splits"])
+def test_a_non_finite_unread_element_never_reaches_the_output(device, splits):
+    """attention.rs:572-592: the cache's first row, which no lane's map reaches, and every row past a
+    lane's keys hold an infinity and NaNs, as memory nothing initialised may; the last key block is
+    partial.  The kernel reads zeros past the keys and never the unmapped row: same bits as with clean memory."""
+    t, d, h, tk = 1, 64, 4, 100
+    q, k, v, _, _, _, _, _, _ = operands(t, d, h, tk, 1)
+    lens = np.array([100, 37, 1, 99, 64])
+    row_map = np.ones(B, dtype=np.int64)
+    dev = lambda x: bf16_tensor(x, device)
+    ints = lambda a: torch.tensor(a, dtype=torch.int32, device=device)
+
+    def call(kk, vv):
+        out = svod_amd.attention(dev(q), dev(kk), dev(vv), Attn(keys=KeyMask.lens(ints(lens)), splits=splits,
+                                                              cache=Cache(h, h, row_map=ints(row_map))))
+        torch.cuda.synchronize()
+        return out
+
+    clean = call(k, v)
+    k2, v2 = k.copy(), v.copy()
+    for x in (k2, v2):
+        x[0] = np.nan
+        x[0, 0, 0, 0] = np.inf
+        x[1, 37:, :h] = np.nan      # heads before the launch's and rows past the shortest lane's keys:
+        x[1, 100:] = np.inf         # the longest lane sees rows 0..99 of heads h..2h-1 only
+    k2[1, :100, h:2 * h], v2[1, :100, h:2 * h] = k[1, :100, h:2 * h], v[1, :100, h:2 * h]
+    dirty = call(k2, v2)
+    assert np.isfinite(to_np(dirty)).all()
+    assert np.array_equal(bits(dirty), bits(clean))

@@ -61,6 +61,21 @@ class _Qkv(ctypes.Structure):
 
 _lib: Optional[ctypes.CDLL] = None
 
+# Fill the outputs and workspaces this module allocates with NaN bit patterns before the call, so that
+# an element a kernel leaves unwritten shows (the reference's tests do the same to their outputs,
+# tk/src/test/unit/device.rs:44-50).  Off by default; the test suite turns it on.
+POISON = False
+
+
+def _fresh(shape, dtype, device) -> torch.Tensor:
+    out = torch.empty(shape, dtype=dtype, device=device)
+    if POISON and out.numel():
+        if out.dtype.is_floating_point:
+            out.fill_(float("nan"))
+        else:
+            out.view(torch.uint8).fill_(0xFF)
+    return out
+
 
 def load_library() -> ctypes.CDLL:
     """The shared library, loaded once.  Missing library = hard error: there is
@@ -279,7 +294,7 @@ def _lend_workspace(lib, a: _Attn, qd: _Tensor, kd: _Tensor, device, workspace, 
         return
     need = int(lib.svodk_attention_workspace(ctypes.byref(qd), ctypes.byref(kd), ctypes.byref(a)))
     if workspace is None and need > 0:
-        workspace = torch.empty(need, dtype=torch.uint8, device=device)
+        workspace = _fresh(need, torch.uint8, device)
     if workspace is not None:
         keep.append(workspace)
         a.workspace, a.workspace_bytes = workspace.data_ptr(), workspace.numel() * workspace.element_size()
@@ -294,7 +309,7 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, opts: Optional[
     lib = load_library()
     if out is None:
         # The op allocates its output at capacity (tk/src/ops/mod.rs:423-429).
-        out = torch.empty_like(q)
+        out = _fresh(q.shape, q.dtype, q.device)
     keep: list = []
     a = _attn_options(opts, keep)
     qd, kd, vd, od = _desc(q), _desc(k), _desc(v), _desc(out)
@@ -320,7 +335,7 @@ def attention_packed(qkv: torch.Tensor, heads: int, kv_heads: int, opts: Optiona
     lib = load_library()
     slots = heads + 2 * kv_heads
     if out is None and qkv.dim() == 3 and slots > 0 and qkv.shape[2] % slots == 0:
-        out = torch.empty((qkv.shape[0], qkv.shape[1], heads, qkv.shape[2] // slots), dtype=qkv.dtype, device=qkv.device)
+        out = _fresh((qkv.shape[0], qkv.shape[1], heads, qkv.shape[2] // slots), qkv.dtype, qkv.device)
     if out is None:
         out = torch.empty((1, 1, 1, 1), dtype=qkv.dtype, device=qkv.device)  # the op rejects the shape itself
     keep: list = []
@@ -343,7 +358,7 @@ def heads(qkv: torch.Tensor, opts: Qkv, out: Optional[Tuple[torch.Tensor, torch.
     lib = load_library()
     if qkv.dim() == 3 and out is None:
         b, t = qkv.shape[0], qkv.shape[1]
-        mk = lambda n: torch.empty((b, t, n, opts.head_dim), dtype=qkv.dtype, device=qkv.device)
+        mk = lambda n: _fresh((b, t, n, opts.head_dim), qkv.dtype, qkv.device)
         out = (mk(opts.heads), mk(opts.kv_heads), mk(opts.kv_heads))
     elif out is None:
         # Let the library word the shape error; the outputs are never touched.
@@ -369,7 +384,8 @@ def _norm(name: str, x, residual, w, b, eps, batch_live, out):
     keep: list = []
     fused = residual is not None
     if out is None:
-        out = (torch.empty_like(x), torch.empty_like(x)) if fused else torch.empty_like(x)
+        out = ((_fresh(x.shape, x.dtype, x.device), _fresh(x.shape, x.dtype, x.device)) if fused
+               else _fresh(x.shape, x.dtype, x.device))
     none = ctypes.POINTER(_Tensor)()
     args = [_ref(keep, x)]
     if fused:
@@ -425,7 +441,7 @@ def order_rows(keys: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.
     rows run grouped by length ends on its short tiles."""
     lib = load_library()
     if out is None:
-        out = torch.empty(keys.shape[:1], dtype=torch.int32, device=keys.device)
+        out = _fresh(keys.shape[:1], torch.int32, keys.device)
     keep: list = []
     status = lib.svodk_order_rows(_ref(keep, keys), _ref(keep, out), ctypes.c_void_p(_stream(keys)))
     _finish("order_rows", status)

@@ -23,4 +23,8 @@ def device():
     assert torch.cuda.is_available(), "the gpu-marked tests need a GPU"
     svod_amd.load_library()
     assert svod_amd.supported(), "the current device is not a gfx950 this library has kernels for"
+    # Outputs the harness allocates start as NaN: an element a kernel leaves unwritten fails its comparison.
+    import svod_amd.ops
+
+    svod_amd.ops.POISON = True
     return torch.device("cuda:0")

@@ -40,19 +40,29 @@ def hipcc() -> str:
     raise RuntimeError("hipcc not found (looked at $HIPCC, PATH and /opt/rocm/bin)")
 
 
+# The attention source is compiled once per head size and once for what does not depend on it
+# (its SVODK_HEAD macro), side by side: one translation unit of every instantiation takes minutes.
+ATTENTION_PARTS = [0, 32, 48, 64, 128]
+
+
 def build(verbose: bool = False) -> str:
+    from concurrent.futures import ThreadPoolExecutor
+
     cc = hipcc()
     objdir = os.path.join(HERE, "build")
     os.makedirs(objdir, exist_ok=True)
-    objs = []
+    jobs = []
     for src in SOURCES:
-        obj = os.path.join(objdir, os.path.splitext(src)[0] + ".o")
-        cmd = [cc, "-x", "hip", *DEVICE_FLAGS, *COMMON_FLAGS, *EXTRA_FLAGS.get(src, []),
-               *os.environ.get("SVODK_CXXFLAGS", "").split(), "-c",
-               os.path.join(CSRC, src), "-o", obj]
-        _run(cmd, verbose)
-        objs.append(obj)
-    _run([cc, *DEVICE_FLAGS, "-shared", "-fPIC", "-o", LIB, *objs], verbose)
+        stem = os.path.splitext(src)[0]
+        parts = [(f"_h{h}", [f"-DSVODK_HEAD={h}"]) for h in ATTENTION_PARTS] if src == "attention_kernel.hip" else [("", [])]
+        for suffix, defines in parts:
+            obj = os.path.join(objdir, stem + suffix + ".o")
+            jobs.append((obj, [cc, "-x", "hip", *DEVICE_FLAGS, *COMMON_FLAGS, *EXTRA_FLAGS.get(src, []), *defines,
+                               *os.environ.get("SVODK_CXXFLAGS", "").split(), "-c", os.path.join(CSRC, src), "-o", obj]))
+    workers = max(1, min(len(jobs), os.cpu_count() or 1, int(os.environ.get("MAX_JOBS", "8"))))
+    with ThreadPoolExecutor(max_workers=workers) as pool:
+        list(pool.map(lambda job: _run(job[1], verbose), jobs))
+    _run([cc, *DEVICE_FLAGS, "-shared", "-fPIC", "-o", LIB, *[obj for obj, _ in jobs]], verbose)
     return LIB
 
 

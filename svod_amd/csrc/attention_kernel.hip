@@ -36,12 +36,19 @@
 #include "kernels.h"
 
 namespace svodk {
+#if !defined(SVODK_CODE_OBJECT)
+// Workgroups per XCD of the streaming form (<= 0: a workgroup per query tile instead), and the
+// streaming launches so far: each takes the next set of shared counters.
+extern std::atomic<int> g_stream_slots;
+extern std::atomic<uint32_t> g_queue_turn;
+#endif
 namespace {
 
 // The kernel's body is compiled for the device only (see flash_fwd_kernel): to the host pass
 // the helpers below have no caller.
-#if !defined(__HIP_DEVICE_COMPILE__)
+#if !defined(__HIP_DEVICE_COMPILE__) || defined(SVODK_HEAD)  // nor, to a part of the build, what other parts use
 #pragma clang diagnostic ignored "-Wunused-function"
+#pragma clang diagnostic ignored "-Wunused-variable"
 #pragma clang diagnostic ignored "-Wunused-const-variable"
 #pragma clang diagnostic ignored "-Wunneeded-internal-declaration"
 #pragma clang diagnostic ignored "-Wunused-template"
@@ -69,11 +76,15 @@ constexpr int kXcds = 8;       // accelerator dies of an MI355X, each with its o
 constexpr float kLog2e = 1.44269504088896340736f;
 constexpr float kRescaleAbove = 8.0f;  // tk/src/kernels/attention.rs:379
 
-#if !defined(SVODK_CODE_OBJECT)
-// Workgroups per XCD of the streaming form; <= 0 = a workgroup per query tile instead.
-std::atomic<int> g_stream_slots{0};
-// Streaming launches so far: each takes the next set of shared counters.
-std::atomic<uint32_t> g_queue_turn{0};
+// The library's build compiles this file once per head size (SVODK_HEAD = 32, 48, 64, 128: that
+// size's instantiations) and once for what does not depend on it (SVODK_HEAD = 0), side by side;
+// without the macro one translation unit holds everything.
+#if defined(SVODK_HEAD)
+#define SVODK_HAS_HEAD(D) (SVODK_HEAD == (D))
+#define SVODK_HAS_COMMON (SVODK_HEAD == 0)
+#else
+#define SVODK_HAS_HEAD(D) 1
+#define SVODK_HAS_COMMON 1
 #endif
 
 // A ring slot holds a [64 keys, D] tile, rows unpadded (D*2 bytes), filled by
@@ -1192,7 +1203,11 @@ struct alignas(64) TileQueue {
   uint32_t next, done;
 };
 constexpr int kQueueSets = 256;
+#if SVODK_HAS_HEAD(64)  // the streaming form exists at head size 64 only
 __device__ __attribute__((unused)) TileQueue g_tile_queues[kQueueSets][kXcds];
+#else
+extern __device__ TileQueue g_tile_queues[kQueueSets][kXcds];  // named by the template, never instantiated here
+#endif
 
 template <int D, int NW, bool CAUSAL, bool F16>
 __global__ __launch_bounds__(NW * 64, 3) void flash_stream_kernel(
@@ -1621,6 +1636,7 @@ hipError_t launch_d(const AttnArgs &a, hipStream_t stream) {
   return a.f16 ? launch_t<D, true>(a, stream) : launch_t<D, false>(a, stream);
 }
 
+#if SVODK_HAS_COMMON
 // The batch rows in descending order of their key counts, ties by row: order[p] = the row with
 // the p-th most keys.  A row's count is its length, or with a [n, tk] key mask the place after its
 // last visible key (what a tile's key blocks run to).  One workgroup; a thread ranks its rows
@@ -1659,8 +1675,26 @@ __global__ __launch_bounds__(256) void order_rows_kernel(const void *__restrict_
     order[ahead] = i;
   }
 }
+#endif  // SVODK_HAS_COMMON
 
 }  // namespace
+
+#if SVODK_HAS_HEAD(32)
+hipError_t launch_attention_d32(const AttnArgs &a, hipStream_t stream) { return launch_d<32>(a, stream); }
+#endif
+#if SVODK_HAS_HEAD(48)
+hipError_t launch_attention_d48(const AttnArgs &a, hipStream_t stream) { return launch_d<48>(a, stream); }
+#endif
+#if SVODK_HAS_HEAD(64)
+hipError_t launch_attention_d64(const AttnArgs &a, hipStream_t stream) { return launch_d<64>(a, stream); }
+#endif
+#if SVODK_HAS_HEAD(128)
+hipError_t launch_attention_d128(const AttnArgs &a, hipStream_t stream) { return launch_d<128>(a, stream); }
+#endif
+
+#if SVODK_HAS_COMMON
+std::atomic<int> g_stream_slots{0};
+std::atomic<uint32_t> g_queue_turn{0};
 
 hipError_t launch_order_rows(const void *keys, int32_t elem_bytes, int32_t n, int32_t tk, int32_t *order,
                              hipStream_t stream) {
@@ -1695,13 +1729,14 @@ const char *attention_config(const AttnArgs &a) {
 
 hipError_t launch_attention(const AttnArgs &a, hipStream_t stream) {
   switch (a.d) {
-    case 32: return launch_d<32>(a, stream);
-    case 48: return launch_d<48>(a, stream);
-    case 64: return launch_d<64>(a, stream);
-    case 128: return launch_d<128>(a, stream);
+    case 32: return launch_attention_d32(a, stream);
+    case 48: return launch_attention_d48(a, stream);
+    case 64: return launch_attention_d64(a, stream);
+    case 128: return launch_attention_d128(a, stream);
     default: return hipErrorInvalidValue;
   }
 }
+#endif  // SVODK_HAS_COMMON
 
 }  // namespace svodk
 

@@ -113,6 +113,11 @@ bool attention_supports(int32_t d);
 // Whether launch_attention runs `a` on grouped tiles: the heads of a KV head's group side by side
 // in one query tile (a decoder step under GQA: no causal or per-row mask, group * t <= 128).
 bool attention_groups(const AttnArgs &a);
+// One head size's kernels each (launch_attention picks by AttnArgs::d).
+hipError_t launch_attention_d32(const AttnArgs &a, hipStream_t stream);
+hipError_t launch_attention_d48(const AttnArgs &a, hipStream_t stream);
+hipError_t launch_attention_d64(const AttnArgs &a, hipStream_t stream);
+hipError_t launch_attention_d128(const AttnArgs &a, hipStream_t stream);
 // order[p] = the batch row with the p-th most keys (ties by row), for AttnArgs::row_order.  `keys` is
 // [n] lengths (tk < 0; elements of 4 or 8 bytes) or an [n, tk] key mask (elements of 1 or 4 bytes).
 constexpr int32_t kMaxOrderedRows = 8192;

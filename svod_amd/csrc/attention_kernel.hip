@@ -938,6 +938,7 @@ __device__ __forceinline__ void flash_fwd_body(
   w.mask_next = 0;
   if (w.scanned) {
     bool open = true;
+    int visible = 0, last_key = 0;  // keys the row shows, and the place after the last of them
     for (int base = 0; base < end; base += 8) {
       int words[8];
 #pragma unroll
@@ -947,13 +948,27 @@ __device__ __forceinline__ void flash_fwd_body(
         if (base + i >= end) break;
         const uint64_t bits = __builtin_amdgcn_ballot_w64(words[i] != 0);
         if (w.lane == 0) w.mask_words[base + i] = bits;
-        if (bits != 0) seen_end = base + i + 1;
+        if (bits != 0) {
+          seen_end = base + i + 1;
+          last_key = (base + i) * kBkv + 64 - __builtin_clzll(bits);
+        }
+        visible += __builtin_popcountll(bits);
         open = open && bits == ~0ull;
         lead_open += open ? 1 : 0;
       }
     }
     end = min(end, seen_end);
     w.end = end;
+    if (visible == last_key) {
+      // The row shows exactly its first `last_key` keys (a padding mask): that is a length, and
+      // from here on the row runs as one with a length does: no mask word per block, rows past
+      // the length never fetched.
+      len = min(len, last_key);
+      w.len = len;
+      w.key_mask = nullptr;
+      w.scanned = false;
+      w.kv_bytes = len > 0 ? (int64_t)(len - 1) * w.kv_row_bytes + D * 2 : 0;
+    }
   } else if (key_mask != nullptr) {
     word0 = mask_lane<D, NW>(w, 0);
     w.mask_next = mask_lane<D, NW>(w, 1);
@@ -1023,7 +1038,7 @@ __device__ __forceinline__ void flash_fwd_body(
   // for a causal wave, below its first row's diagonal.  A key mask puts every block on the
   // edge path.  Step j is hot when block j+1 is such a block.
   int full = 0;
-  if (w.positive && (key_mask == nullptr || w.scanned)) {
+  if (w.positive && (w.key_mask == nullptr || w.scanned)) {
     full = min(my_end, len / kBkv);
     if (w.scanned) full = min(full, lead_open);
     if (RANGED)

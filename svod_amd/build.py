@@ -74,29 +74,36 @@ def build_code_objects(verbose: bool = False) -> str:
 
     from . import code_object as co
 
+    from concurrent.futures import ThreadPoolExecutor
+
     cc = hipcc()
     os.makedirs(co.CO_DIR, exist_ok=True)
     table = co.entries()
-    built = {}
+    jobs = {}
     for name, e in table.items():
-        if e["file"] in built:
+        if e["file"] in jobs:
             continue
         path = os.path.join(co.CO_DIR, e["file"])
         # No argument preload here: a loader that writes its own user registers passes the record's address only.
         extra = [f for f in EXTRA_FLAGS.get(e["source"], []) if "kernarg-preload" not in f]
         extra = [f for i, f in enumerate(extra) if not (f == "-mllvm" and (i + 1 == len(extra) or extra[i + 1] == "-mllvm"))]
-        cmd = [cc, "-x", "hip", *DEVICE_FLAGS, "--offload-device-only", "--no-gpu-bundle-output", "-DSVODK_CODE_OBJECT",
-               "-O3", "-std=c++17", "-Wall", "-Wno-unused-command-line-argument", *extra,
-               os.path.join(CSRC, e["source"]), "-o", path]
-        _run(cmd, verbose)
-        with open(path, "rb") as f:
-            built[e["file"]] = f.read()
+        head = [f"-DSVODK_HEAD={e['head']}"] if "head" in e else []  # one head size's full family a file
+        jobs[e["file"]] = [cc, "-x", "hip", *DEVICE_FLAGS, "--offload-device-only", "--no-gpu-bundle-output",
+                           "-DSVODK_CODE_OBJECT", *head, "-O3", "-std=c++17", "-Wall", "-Wno-unused-command-line-argument",
+                           *extra, os.path.join(CSRC, e["source"]), "-o", path]
+    workers = max(1, min(len(jobs), os.cpu_count() or 1, int(os.environ.get("MAX_JOBS", "8"))))
+    with ThreadPoolExecutor(max_workers=workers) as pool:
+        list(pool.map(lambda cmd: _run(cmd, verbose), jobs.values()))
+    built = {}
+    for f in jobs:
+        with open(os.path.join(co.CO_DIR, f), "rb") as fh:
+            built[f] = fh.read()
     manifest = {"arch": "gfx950", "record": "buffers are 8-byte addresses, scalars 4-byte integers, in this order at "
                                             "natural alignment; *_bits scalars are an f32's bit pattern",
                 "kernels": {}}
     for name, e in table.items():
         kd = co.check(built[e["file"]], name, e["params"])
-        manifest["kernels"][name] = {**{k: v for k, v in e.items() if k != "source"},
+        manifest["kernels"][name] = {**{k: v for k, v in e.items() if k not in ("source", "head")},
                                      "kernarg_size": kd.kernarg_size, "lds_bytes": kd.group_segment_fixed_size}
     for f in built:
         unlisted = set(co.CodeObject.parse(built[f]).kernels()) - set(table)

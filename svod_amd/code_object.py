@@ -43,6 +43,32 @@ B, S = "buffer", "scalar"
 _ATTENTION = [("q", B), ("k", B), ("v", B), ("o", B), ("key_lens", B),
               ("batch", S), ("t", S), ("tk", S), ("heads", S), ("kv_heads", S), ("scale_bits", S)]
 _ATTENTION_MASK = [p if p[0] != "key_lens" else ("key_mask", B) for p in _ATTENTION]
+_FULL = ([(n, B) for n in ("q", "k", "v", "o", "key_lens", "key_mask", "seg_start", "row_map", "k_app", "v_app", "app_lens",
+                            "bias", "o_part", "m_part", "l_part")] +
+         [(n, S) for n in ("batch", "t", "tk", "heads", "kv_heads", "scale_bits", "lens_i64", "mask_bytes", "q_row_elems",
+                           "kv_row_elems", "splits", "win_left", "win_right", "chunk_size", "chunk_left", "chunk_right",
+                           "seg_i64", "bias_per_batch", "kv_head_start", "row_map_i64", "cache_rows", "app_rows",
+                           "app_lens_i64")])
+_COMBINE = [("o_part", B), ("m_part", B), ("l_part", B), ("o", B), ("rows", S), ("splits", S)]
+
+
+def full_forms():
+    """(causal, split, ranged, biased, cached, grouped) of every instantiation the library's own
+    dispatch reaches: a cache excludes per-row ranges; grouped tiles take neither a causal mask
+    nor ranges."""
+    for ranged, biased, cached in ((0, 0, 0), (0, 1, 0), (1, 0, 0), (1, 1, 0), (0, 0, 1), (0, 1, 1)):
+        for causal in (0, 1):
+            for split in (0, 1):
+                yield causal, split, ranged, biased, cached, 0
+        if not ranged:
+            for split in (0, 1):
+                yield 0, split, 0, biased, cached, 1
+
+
+def full_name(d: int, dtype: str, causal, split, ranged, biased, cached, grouped) -> str:
+    return f"svodk_attention_full_d{d}_{dtype}_c{causal}s{split}r{ranged}b{biased}k{cached}g{grouped}"
+
+
 _HEADS = [("qkv", B), ("q_w", B), ("k_w", B), ("cos", B), ("sin", B), ("q", B), ("k", B), ("v", B),
           ("rows", S), ("t", S), ("heads", S), ("kv_heads", S), ("eps_bits", S), ("rope", S)]
 _TAIL = [("rows", S), ("d", S), ("eps_bits", S)]
@@ -71,6 +97,20 @@ def entries() -> Dict[str, dict]:
                     plain = out[f"svodk_attention_d{d}_{dtype}" + ("_causal" if causal else "")]
                     out[f"svodk_attention_d{d}_{dtype}" + ("_causal" if causal else "") + "_mask"] = {
                         **plain, "params": _ATTENTION_MASK, "key_mask": True}
+        for d in (32, 48, 64, 128):
+            for c, s, r, b, k, g in full_forms():
+                per = ("1" if g else "(heads // kv_heads) * ((t + 127) // 128)") + (" * splits" if s else "")
+                out[full_name(d, dtype, c, s, r, b, k, g)] = {
+                    "file": f"svodk_attention_full_d{d}.co", "source": "attention_kernel.hip", "head": d, "params": _FULL,
+                    "local": [256, 1, 1], "workgroups": f"(batch * kv_heads + 7) // 8 * 8 * {per}",
+                    "op": "attention", "dtype": dtype, "head_dim": d, "causal": bool(c), "split": bool(s),
+                    "ranged": bool(r), "biased": bool(b), "cached": bool(k), "grouped": bool(g), "key_mask": True,
+                    "cfg": f"FaCfg {{ bq: 128, bkv: 64, stages: 2, splits: {'n' if s else 1}, forms: {{ raw_max, "
+                           f"skip_rescale }}, warp_rows: 32, core: mfma_f32_32x32x16_{dtype} }}"}
+            out[f"svodk_combine_d{d}_{dtype}"] = {
+                "file": "svodk_combine.co", "source": "combine_kernel.hip", "params": _COMBINE, "local": [256, 1, 1],
+                "workgroups": f"(rows * {d // 4} + 255) // 256", "op": "combine_splits", "dtype": dtype, "head_dim": d,
+                "cfg": "NormCfg { br: 4 }"}
         for d in (64, 128):
             out[f"svodk_heads_d{d}_{dtype}"] = {
                 "file": "svodk_heads.co", "source": "heads_kernel.hip", "params": _HEADS, "local": [256, 1, 1],

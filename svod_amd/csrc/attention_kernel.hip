@@ -1803,6 +1803,104 @@ __device__ __forceinline__ void attention_entry(uint8_t *smem, const uint16_t *q
 }
 #endif
 
+// ---- every form the library has, one kernel an instantiation (svodk_attention_full_d<D>_<type>_
+// c<causal>s<split>r<ranged>b<biased>k<cached>g<grouped>), all with one record.  Buffers, in the
+// reference kernel's order (tk/src/kernels/attention.rs:308-327, 452-459), an address of 0 for what
+// a call does not have: q, k, v, o, key_lens, key_mask, seg_start, row_map, k_app, v_app, app_lens,
+// bias, then the partial states of a split call o_part, m_part, l_part.  Scalars: batch, t, tk,
+// heads, kv_heads, scale_bits, lens_i64, mask_bytes (1 or 4), q_row_elems, kv_row_elems (0: heads * D
+// and kv_heads * D; a fused projection's or a cache's row otherwise), splits, win_left (< 0: no
+// window), win_right, chunk_size (0: none), chunk_left (< 0: every earlier chunk), chunk_right,
+// seg_i64, bias_per_batch, kv_head_start, row_map_i64, cache_rows, app_rows, app_lens_i64.
+// A kernel reads what its flags name and ignores the rest.  Launch: ceil(batch * kv_heads, 8) * per
+// workgroups of 256 threads, per = (g ? 1 : heads / kv_heads) * (g ? 1 : ceil(t / 128)) * (s ? splits : 1).
+// LDS: the ring and the scanned mask words.  The caller keeps the op layer's checks, the caps on the
+// window's and the chunks' reaches included (at most t + tk, and the chunks of t + tk).
+#define SVODK_FULL_PARAMS                                                                                             \
+  const uint16_t *__restrict__ q, const uint16_t *__restrict__ k, const uint16_t *__restrict__ v,                     \
+      uint16_t *__restrict__ o, const void *__restrict__ key_lens, const void *__restrict__ key_mask,                 \
+      const void *__restrict__ seg_start, const void *__restrict__ row_map, const uint16_t *__restrict__ k_app,       \
+      const uint16_t *__restrict__ v_app, const void *__restrict__ app_lens, const uint16_t *__restrict__ bias,       \
+      float *__restrict__ o_part, float *__restrict__ m_part, float *__restrict__ l_part, int32_t batch, int32_t t,   \
+      int32_t tk, int32_t heads, int32_t kv_heads, int32_t scale_bits, int32_t lens_i64, int32_t mask_bytes,          \
+      int32_t q_row_elems, int32_t kv_row_elems, int32_t splits, int32_t win_left, int32_t win_right,                 \
+      int32_t chunk_size, int32_t chunk_left, int32_t chunk_right, int32_t seg_i64, int32_t bias_per_batch,           \
+      int32_t kv_head_start, int32_t row_map_i64, int32_t cache_rows, int32_t app_rows, int32_t app_lens_i64
+#define SVODK_FULL_ARGS                                                                                               \
+  q, k, v, o, key_lens, key_mask, seg_start, row_map, k_app, v_app, app_lens, bias, o_part, m_part, l_part, batch, t, \
+      tk, heads, kv_heads, scale_bits, lens_i64, mask_bytes, q_row_elems, kv_row_elems, splits, win_left, win_right,  \
+      chunk_size, chunk_left, chunk_right, seg_i64, bias_per_batch, kv_head_start, row_map_i64, cache_rows, app_rows, \
+      app_lens_i64
+
+#if defined(__HIP_DEVICE_COMPILE__)
+template <int D, bool CAUSAL, bool SPLIT, bool RANGED, bool BIASED, bool CACHED, bool GROUPED, bool F16>
+__device__ __forceinline__ void attention_entry_full(uint8_t *smem, SVODK_FULL_PARAMS) {
+  constexpr int NW = 4;
+  if (batch <= 0 || t <= 0 || tk < 0 || kv_heads <= 0 || heads < kv_heads) return;
+  const uint32_t group = (uint32_t)heads / (uint32_t)kv_heads;
+  const uint32_t count = SPLIT ? (uint32_t)(splits > 0 ? splits : 1) : 1u;
+  const uint32_t nqt = (GROUPED ? 1u : ((uint32_t)t + NW * kWaveRows - 1) / (NW * kWaveRows)) * count;
+  const uint32_t unit_size = (GROUPED ? 1u : group) * nqt;
+  const Splits sp = {count, rcp_for(count), o_part, m_part, l_part, (uint32_t)batch};
+  Ranges rg = {};
+  rg.win_left = RANGED ? win_left : -1;
+  rg.win_right = win_right;
+  rg.chunk_size = RANGED ? chunk_size : 0;
+  rg.chunk_left = chunk_left;
+  rg.chunk_right = chunk_right;
+  rg.seg_start = RANGED ? seg_start : nullptr;
+  rg.seg_i64 = seg_i64;
+  rg.bias = bias;
+  rg.bias_per_batch = bias_per_batch;
+  rg.bias_cols = tk + (CACHED ? app_rows : 0);
+  rg.kv_head_start = kv_head_start;
+  rg.row_map = row_map;
+  rg.row_map_i64 = row_map_i64;
+  rg.cache_rows = cache_rows;
+  rg.k_app = k_app;
+  rg.v_app = v_app;
+  rg.app_rows = app_rows;
+  rg.app_lens = app_lens;
+  rg.app_lens_i64 = app_lens_i64;
+  flash_fwd_body<D, NW, CAUSAL, SPLIT, RANGED, BIASED, CACHED, GROUPED, F16>(
+      smem, unit_size, rcp_for(unit_size), nqt, rcp_for(nqt), (uint32_t)kv_heads, rcp_for((uint32_t)kv_heads),
+      (uint32_t)kv_heads * (uint32_t)batch, (uint32_t)heads | group << 16, key_lens, nullptr, t,
+      (uint32_t)tk | (lens_i64 ? 0x80000000u : 0u), q, k, v, o, key_mask, mask_bytes, __builtin_bit_cast(float, scale_bits),
+      sp, q_row_elems > 0 ? q_row_elems : heads * D, kv_row_elems > 0 ? kv_row_elems : kv_heads * D, rg);
+}
+#endif
+
+#define SVODK_FULL_ENTRY(D, T, F16, C, S, R, B, K, G)                                                                 \
+  extern "C" __global__ __launch_bounds__(256, ((D) <= 64 && !(B)) ? 3 : 2) void                                      \
+      svodk_attention_full_d##D##_##T##_c##C##s##S##r##R##b##B##k##K##g##G(SVODK_FULL_PARAMS) {                       \
+    __shared__ __attribute__((aligned(1024))) uint8_t smem[Tile<D>::kLds + 4 * kScannedBlocks * 8];                   \
+    attention_entry_full<D, C, S, R, B, K, G, F16>(smem, SVODK_FULL_ARGS);                                            \
+  }
+// The instantiations the library's own dispatch reaches: a cache excludes per-row ranges; grouped
+// tiles take neither a causal mask nor ranges.
+#define SVODK_FULL_SPLITS(D, T, F16, C, R, B, K, G) \
+  SVODK_FULL_ENTRY(D, T, F16, C, 0, R, B, K, G) SVODK_FULL_ENTRY(D, T, F16, C, 1, R, B, K, G)
+#define SVODK_FULL_TILES(D, T, F16, R, B, K)                                                  \
+  SVODK_FULL_SPLITS(D, T, F16, 0, R, B, K, 0) SVODK_FULL_SPLITS(D, T, F16, 1, R, B, K, 0)
+#define SVODK_FULL_FAMILY(D, T, F16)                                                          \
+  SVODK_FULL_TILES(D, T, F16, 0, 0, 0) SVODK_FULL_SPLITS(D, T, F16, 0, 0, 0, 0, 1)           \
+  SVODK_FULL_TILES(D, T, F16, 0, 1, 0) SVODK_FULL_SPLITS(D, T, F16, 0, 0, 1, 0, 1)           \
+  SVODK_FULL_TILES(D, T, F16, 1, 0, 0) SVODK_FULL_TILES(D, T, F16, 1, 1, 0)                   \
+  SVODK_FULL_TILES(D, T, F16, 0, 0, 1) SVODK_FULL_SPLITS(D, T, F16, 0, 0, 0, 1, 1)           \
+  SVODK_FULL_TILES(D, T, F16, 0, 1, 1) SVODK_FULL_SPLITS(D, T, F16, 0, 0, 1, 1, 1)
+
+#if defined(SVODK_HEAD)  // one head size's whole family a file
+#if SVODK_HEAD == 32
+SVODK_FULL_FAMILY(32, bf16, false) SVODK_FULL_FAMILY(32, f16, true)
+#elif SVODK_HEAD == 48
+SVODK_FULL_FAMILY(48, bf16, false) SVODK_FULL_FAMILY(48, f16, true)
+#elif SVODK_HEAD == 64
+SVODK_FULL_FAMILY(64, bf16, false) SVODK_FULL_FAMILY(64, f16, true)
+#elif SVODK_HEAD == 128
+SVODK_FULL_FAMILY(128, bf16, false) SVODK_FULL_FAMILY(128, f16, true)
+#endif
+#else  // the short records: lengths or a key mask, causal or not
+
 #define SVODK_ATTENTION_ENTRY(NAME, D, CAUSAL, F16)                                                                  \
   extern "C" __global__ __launch_bounds__(256, (D) <= 64 ? 3 : 2) void NAME(                                          \
       const uint16_t *__restrict__ q, const uint16_t *__restrict__ k, const uint16_t *__restrict__ v,                 \
@@ -1848,6 +1946,7 @@ SVODK_ATTENTION_MASK_ENTRY(svodk_attention_d128_f16_mask, 128, false, true)
 SVODK_ATTENTION_MASK_ENTRY(svodk_attention_d128_f16_causal_mask, 128, true, true)
 #undef SVODK_ATTENTION_ENTRY
 #undef SVODK_ATTENTION_MASK_ENTRY
+#endif  // SVODK_HEAD
 
 }  // namespace
 }  // namespace svodk

@@ -32,11 +32,11 @@ __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
 }
 
+// The workgroup's program, for the kernels below to inline.
 template <int D, bool F16>
-__global__ __launch_bounds__(kThreads) void combine_kernel(const float *__restrict__ o_part,
-                                                           const float *__restrict__ m_part,
-                                                           const float *__restrict__ l_part, uint16_t *__restrict__ o,
-                                                           int64_t rows, int32_t splits) {
+__device__ __forceinline__ void combine_body(const float *__restrict__ o_part, const float *__restrict__ m_part,
+                                             const float *__restrict__ l_part, uint16_t *__restrict__ o, int64_t rows,
+                                             int32_t splits) {
 #pragma clang fp contract(off)
   constexpr int kLanes = D / 4;  // lanes sharing a row
   const int64_t gid = (int64_t)__builtin_amdgcn_workgroup_id_x() * kThreads + __builtin_amdgcn_workitem_id_x();
@@ -61,6 +61,15 @@ __global__ __launch_bounds__(kThreads) void combine_kernel(const float *__restri
   out[0] = pack2<F16>(acc[0] / ll, acc[1] / ll);
   out[1] = pack2<F16>(acc[2] / ll, acc[3] / ll);
   *(reinterpret_cast<u32x2 *>(o + row * D) + part) = out;
+}
+
+#if !defined(SVODK_CODE_OBJECT)  // the library's kernel and its launch: not part of a code object build
+template <int D, bool F16>
+__global__ __launch_bounds__(kThreads) void combine_kernel(const float *__restrict__ o_part,
+                                                           const float *__restrict__ m_part,
+                                                           const float *__restrict__ l_part, uint16_t *__restrict__ o,
+                                                           int64_t rows, int32_t splits) {
+  combine_body<D, F16>(o_part, m_part, l_part, o, rows, splits);
 }
 
 template <int D, bool F16>
@@ -88,3 +97,29 @@ hipError_t launch_combine(const CombineArgs &a, hipStream_t stream) {
 }
 
 }  // namespace svodk
+
+#else  // SVODK_CODE_OBJECT
+// The merge as kernels for a loader that takes a code object and a flat argument record
+// (device/src/amd/program.rs:403-414, 655-675; device/src/hcq.rs:1262-1285): o_part [splits, rows, D],
+// m_part and l_part [splits, rows] (f32, what a split attention kernel wrote), o [rows, D], then rows
+// (batch * t * heads) and splits.  Launch: ceil(rows * (D / 4) / 256) workgroups of 256 threads.
+#define SVODK_COMBINE_ENTRY(NAME, D, F16)                                                                             \
+  extern "C" __global__ __launch_bounds__(kThreads) void NAME(const float *__restrict__ o_part,                       \
+                                                              const float *__restrict__ m_part,                       \
+                                                              const float *__restrict__ l_part,                       \
+                                                              uint16_t *__restrict__ o, int32_t rows, int32_t splits) { \
+    if (splits >= 1) combine_body<D, F16>(o_part, m_part, l_part, o, rows, splits);                                   \
+  }
+SVODK_COMBINE_ENTRY(svodk_combine_d32_bf16, 32, false)
+SVODK_COMBINE_ENTRY(svodk_combine_d48_bf16, 48, false)
+SVODK_COMBINE_ENTRY(svodk_combine_d64_bf16, 64, false)
+SVODK_COMBINE_ENTRY(svodk_combine_d128_bf16, 128, false)
+SVODK_COMBINE_ENTRY(svodk_combine_d32_f16, 32, true)
+SVODK_COMBINE_ENTRY(svodk_combine_d48_f16, 48, true)
+SVODK_COMBINE_ENTRY(svodk_combine_d64_f16, 64, true)
+SVODK_COMBINE_ENTRY(svodk_combine_d128_f16, 128, true)
+#undef SVODK_COMBINE_ENTRY
+
+}  // namespace
+}  // namespace svodk
+#endif  // SVODK_CODE_OBJECT

@@ -170,3 +170,118 @@ def test_norm_code_objects_equal_the_library(device, runtime, kind, d, f16):
     runtime.launch(f"svodk_{kind}_d{dmax}_{'f16' if f16 else 'bf16'}", values)
     for y, z in zip(got, want):
         assert np.array_equal(bits(y), bits(z))
+
+
+# ---- the full family: every form the library has, one record for all of them.
+def full_record(q, k, v, o, *, batch=None, heads=None, kv_heads=None, scale=None, key_lens=None, key_mask=None, seg_start=None,
+                row_map=None, k_app=None, v_app=None, app_lens=None, bias=None, parts=None, splits=1, window=None,
+                chunk=None, q_row_elems=0, kv_row_elems=0, kv_head_start=0, cache_rows=0):
+    """The record of a full kernel for these operands, as the op layer would fill it
+    (tk/src/ops/attention.rs:216-283: reaches capped where they no longer hide anything)."""
+    ptr = lambda x: 0 if x is None else x.data_ptr()
+    b, t, h, d = q.shape
+    tk = k.shape[1]
+    left, right = (-1, 0) if window is None else (min(window[0], t + tk), min(window[1], t + tk))
+    size, cl, cr = (0, -1, 0) if chunk is None else chunk
+    chunks = (t + tk) // size + 2 if size else 0
+    return {"q": ptr(q), "k": ptr(k), "v": ptr(v), "o": ptr(o), "key_lens": ptr(key_lens), "key_mask": ptr(key_mask),
+            "seg_start": ptr(seg_start), "row_map": ptr(row_map), "k_app": ptr(k_app), "v_app": ptr(v_app),
+            "app_lens": ptr(app_lens), "bias": ptr(bias), "o_part": ptr(parts[0]) if parts else 0,
+            "m_part": ptr(parts[1]) if parts else 0, "l_part": ptr(parts[2]) if parts else 0,
+            "batch": batch or b, "t": t, "tk": tk, "heads": heads or h, "kv_heads": kv_heads or k.shape[2],
+            "scale_bits": f32_bits(scale if scale is not None else d ** -0.5),
+            "lens_i64": int(key_lens is not None and key_lens.dtype == torch.int64),
+            "mask_bytes": 0 if key_mask is None else key_mask.element_size(), "q_row_elems": q_row_elems,
+            "kv_row_elems": kv_row_elems, "splits": splits, "win_left": left, "win_right": right,
+            "chunk_size": size, "chunk_left": -1 if cl is None else min(cl, chunks), "chunk_right": min(cr, chunks),
+            "seg_i64": int(seg_start is not None and seg_start.dtype == torch.int64),
+            "bias_per_batch": int(bias is not None and (bias.shape[0] != 1 or b == 1)), "kv_head_start": kv_head_start,
+            "row_map_i64": int(row_map is not None and row_map.dtype == torch.int64), "cache_rows": cache_rows,
+            "app_rows": 0 if k_app is None else k_app.shape[1],
+            "app_lens_i64": int(app_lens is not None and app_lens.dtype == torch.int64)}
+
+
+def test_full_kernels_with_per_row_ranges_equal_the_library(device, runtime):
+    b, t, tk, h, hkv, d = 2, 300, 300, 4, 2, 64
+    g = Lcg(5)
+    q, k, v = (bf16_tensor(g.bf16(s), device) for s in ((b, t, h, d), (b, tk, hkv, d), (b, tk, hkv, d)))
+    lens = torch.tensor([300, 171], dtype=torch.int32, device=device)
+    seg = torch.from_numpy(np.tile(np.arange(t) - np.arange(t) % 40, (b, 1))).to(torch.int64).to(device)
+    for causal, window, chunk, seg_start in ((False, (64, 64), None, None), (True, (50, 0), (32, 3, 0), seg),
+                                             (False, None, (24, None, 1), None)):
+        want = svod_amd.attention(q, k, v, Attn(causal=causal, keys=KeyMask.lens(lens), window=window, chunk=chunk,
+                                                seg_start=seg_start, splits=1))
+        got = torch.full_like(want, 7.0)
+        runtime.launch(co.full_name(d, "bf16", int(causal), 0, 1, 0, 0, 0),
+                       full_record(q, k, v, got, key_lens=lens, window=window, chunk=chunk, seg_start=seg_start))
+        assert np.array_equal(bits(got), bits(want)), (causal, window, chunk)
+
+
+def test_full_kernel_with_a_bias_and_a_key_mask_equals_the_library(device, runtime):
+    b, t, tk, h, hkv, d = 2, 130, 130, 4, 2, 128
+    g = Lcg(7)
+    q, k, v = (tensor(g.bf16(s), device, True) for s in ((b, t, h, d), (b, tk, hkv, d), (b, tk, hkv, d)))
+    bias = tensor(g.bf16((1, h, t, tk), mul=2.0), device, True)
+    mask = torch.from_numpy(np.add.outer(np.arange(b), np.arange(tk)) % 5 != 2).to(device)
+    want = svod_amd.attention(q, k, v, Attn(causal=True, keys=KeyMask.bool(mask), bias=bias, splits=1))
+    got = torch.full_like(want, 7.0)
+    runtime.launch(co.full_name(d, "f16", 1, 0, 0, 1, 0, 0), full_record(q, k, v, got, key_mask=mask, bias=bias))
+    assert np.array_equal(bits(got), bits(want))
+
+
+def test_full_split_kernel_and_the_merge_equal_the_library(device, runtime):
+    """A decoder step: one query, 1500 keys, four splits (tk/src/test/unit/ops.rs:585), then combine_splits."""
+    b, t, tk, h, d, splits = 3, 1, 1500, 20, 64, 4
+    g = Lcg(9)
+    q, k, v = (bf16_tensor(g.bf16(s), device) for s in ((b, t, h, d), (b, tk, h, d), (b, tk, h, d)))
+    lens = torch.tensor([1500, 700, 0], dtype=torch.int32, device=device)
+    want = svod_amd.attention(q, k, v, Attn(keys=KeyMask.lens(lens), splits=splits))
+    assert "combine_splits" in svod_amd.chosen()
+    rows = b * t * h
+    parts = (torch.full((splits, rows, d), 7.0, device=device), torch.full((splits, rows), 7.0, device=device),
+             torch.full((splits, rows), 7.0, device=device))
+    scratch = torch.empty_like(want)
+    runtime.launch(co.full_name(d, "bf16", 0, 1, 0, 0, 0, 0),
+                   full_record(q, k, v, scratch, key_lens=lens, parts=parts, splits=splits))
+    got = torch.full_like(want, 7.0)
+    runtime.launch(f"svodk_combine_d{d}_bf16", {"o_part": parts[0].data_ptr(), "m_part": parts[1].data_ptr(),
+                                                "l_part": parts[2].data_ptr(), "o": got.data_ptr(), "rows": rows,
+                                                "splits": splits})
+    assert np.array_equal(bits(got), bits(want))
+    assert not bits(got[2]).any()
+
+
+def test_full_cached_grouped_kernel_equals_the_library(device, runtime):
+    """A decoder step under GQA over a cache of three layers' heads with a row map, appended rows and
+    their counts (tk/src/test/unit/ops.rs:589-590), the KV head's group in one tile."""
+    from svod_amd import Cache
+    b, t, tk, h, hkv, d, rows, layers, appended = 5, 2, 200, 8, 2, 48, 2, 3, 8
+    g = Lcg(40)
+    q = bf16_tensor(g.bf16((b, t, h, d)), device)
+    k, v = (bf16_tensor(g.bf16((rows, tk, layers * hkv, d)), device) for _ in range(2))
+    k_app, v_app = (bf16_tensor(g.bf16((b, appended, hkv, d)), device) for _ in range(2))
+    lens = torch.tensor([tk, 1, 37, tk - 1, 0], dtype=torch.int32, device=device)
+    row_map = torch.tensor([0, 1, 1, 0, 1], dtype=torch.int64, device=device)
+    seen = torch.tensor([8, 7, 6, 8, 1], dtype=torch.int32, device=device)
+    want = svod_amd.attention(q, k, v, Attn(keys=KeyMask.lens(lens), splits=1,
+                                            cache=Cache(hkv, hkv, row_map=row_map, appended=(k_app, v_app), app_lens=seen)))
+    got = torch.full_like(want, 7.0)
+    runtime.launch(co.full_name(d, "bf16", 0, 0, 0, 0, 1, 1),
+                   full_record(q, k, v, got, kv_heads=hkv, key_lens=lens, row_map=row_map, k_app=k_app, v_app=v_app,
+                               app_lens=seen, kv_row_elems=layers * hkv * d, kv_head_start=hkv, cache_rows=rows))
+    assert np.array_equal(bits(got), bits(want))
+
+
+def test_full_kernel_reads_a_fused_projection_in_place(device, runtime):
+    """attention_packed (tk/src/ops/attention.rs:104-122): q, k and v are views of one [B, T, (H + 2 Hkv) D] row."""
+    b, t, h, hkv, d = 2, 150, 4, 2, 32
+    x = tensor(Lcg(3).bf16((b, t, (h + 2 * hkv) * d)), device, False)
+    want = svod_amd.attention_packed(x, h, hkv, Attn(causal=True, splits=1))
+    got = torch.full_like(want, 7.0)
+    row = (h + 2 * hkv) * d
+    q = x.view(b, t, h + 2 * hkv, d)[:, :, :h]  # shapes only: the record takes addresses
+    rec = full_record(q, x.view(b, t, h + 2 * hkv, d)[:, :, h:h + hkv], None, got, heads=h, kv_heads=hkv, q_row_elems=row,
+                      kv_row_elems=row)
+    rec["q"], rec["k"], rec["v"] = x.data_ptr(), x.data_ptr() + h * d * 2, x.data_ptr() + (h + hkv) * d * 2
+    runtime.launch(co.full_name(d, "bf16", 1, 0, 0, 0, 0, 0), rec)
+    assert np.array_equal(bits(got), bits(want))

@@ -13,7 +13,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
-#include <mutex>
+#include <atomic>
 #include <string>
 
 #include "../../include/svodk.h"
@@ -148,12 +148,15 @@ bool current_device_has_kernels() {
     (void)hipGetLastError();
     return false;
   }
-  static std::mutex lock;
-  static int known[64];  // 0 unknown, 1 yes, 2 no
-  std::lock_guard<std::mutex> guard(lock);
+  // 0 unknown, 1 yes, 2 no; two threads that both find it unknown ask the runtime twice and store the same answer.
+  static std::atomic<int> known[64];
   if (device >= 64) return device_is_gfx950(device);
-  if (known[device] == 0) known[device] = device_is_gfx950(device) ? 1 : 2;
-  return known[device] == 1;
+  int state = known[device].load(std::memory_order_acquire);
+  if (state == 0) {
+    state = device_is_gfx950(device) ? 1 : 2;
+    known[device].store(state, std::memory_order_release);
+  }
+  return state == 1;
 }
 
 // ---- shape gates (tk/src/ops/shape.rs).

@@ -23,7 +23,7 @@
 extern "C" {
 #endif
 
-#define SVODK_ABI_VERSION 3
+#define SVODK_ABI_VERSION 4
 
 /* Element types of a tensor descriptor. */
 typedef enum svodk_dtype {
@@ -158,6 +158,25 @@ typedef struct svodk_qkv {
  */
 int svodk_attention(const svodk_tensor *q, const svodk_tensor *k, const svodk_tensor *v, const svodk_attn *opts,
                     const svodk_tensor *out, void *hip_stream);
+
+/*
+ * svodk_attention for callers that cannot allocate device memory (code under HIP graph capture, a
+ * serving loop with a fixed memory plan, a harness that forbids hipMalloc).  It has no counterpart
+ * in the reference, whose op allocates the partial tensors of a split call itself
+ * (tk/src/ops/attention.rs:285-293).  Same operands, options, checks, kernels and results as
+ * svodk_attention; the one difference is where the partial states of a split call live: in a
+ * static device array of the library, svodk_noalloc_scratch_bytes() (8 MiB) on each GPU the library
+ * runs on, held until the process ends.  `opts->workspace` is ignored.  The call and everything
+ * under it allocate nothing.  A call whose splits (named, or chosen for `splits` = 0 as if a workspace
+ * had been lent) need more than the array holds answers SVODK_ERR_ARGUMENT and launches nothing;
+ * svodk_attention_workspace says how much a call needs.  Every call on a GPU shares that GPU's
+ * array: calls that overlap on one GPU (two streams, two threads) race on it and must be ordered
+ * by the caller.  Nothing in the array has to start at zero (a split call writes every partial
+ * state its merge reads).
+ */
+int svodk_attention_noalloc(const svodk_tensor *q, const svodk_tensor *k, const svodk_tensor *v, const svodk_attn *opts,
+                            const svodk_tensor *out, void *hip_stream);
+int64_t svodk_noalloc_scratch_bytes(void);
 
 /*
  * ops::attention_packed (tk/src/ops/attention.rs:104-122): attention over a fused

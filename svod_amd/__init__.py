@@ -18,7 +18,9 @@ from .ops import (  # noqa: F401
     add_layer_norm,
     add_rms_norm,
     attention,
+    attention_noalloc,
     attention_packed,
+    noalloc_scratch_bytes,
     tune_streaming,
     chosen,
     heads,

@@ -8,7 +8,19 @@
 // lanes, each reading one 128-bit chunk per split and writing 8 bytes of bf16.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+
 #include "kernels.h"
+
+#if !defined(SVODK_CODE_OBJECT)
+// The partial states of a split call whose caller cannot lend a workspace because it cannot allocate
+// one (code under graph capture, a serving loop with a fixed memory plan): kSplitScratchBytes of
+// device memory that every GPU the library runs on holds until the process ends.  In host code the
+// array's name is a stand-in, not a device address: each device's copy has its own address, which
+// split_scratch() looks up once with that device current and keeps; kernels take that pointer as an
+// argument.
+static __device__ __align__(256) unsigned char scratch[svodk::kSplitScratchBytes];
+#endif
 
 namespace svodk {
 namespace {
@@ -83,7 +95,25 @@ hipError_t launch(const CombineArgs &a, hipStream_t stream) {
   return hipGetLastError();
 }
 
+std::atomic<void *> g_scratch_at[64];  // `scratch` by device ordinal; devices past 63 ask every time
+
 }  // namespace
+
+hipError_t split_scratch(void **ptr, int64_t *bytes) {
+  int device = -1;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) return e;
+  void *at = device >= 0 && device < 64 ? g_scratch_at[device].load(std::memory_order_acquire) : nullptr;
+  if (at == nullptr) {
+    e = hipGetSymbolAddress(&at, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return e;
+    if (at == nullptr) return hipErrorInvalidSymbol;
+    if (device >= 0 && device < 64) g_scratch_at[device].store(at, std::memory_order_release);
+  }
+  *ptr = at;
+  *bytes = kSplitScratchBytes;
+  return hipSuccess;
+}
 
 hipError_t launch_combine(const CombineArgs &a, hipStream_t stream) {
   if (a.splits < 1) return hipErrorInvalidValue;

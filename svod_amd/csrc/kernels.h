@@ -109,6 +109,11 @@ struct CombineArgs {
   int32_t f16;
 };
 hipError_t launch_combine(const CombineArgs &a, hipStream_t stream);
+// The library's own device memory for the partial states of a split call that brings no workspace:
+// a file-scope array of kSplitScratchBytes per GPU.  `*ptr` is the current device's copy (its
+// address is looked up on the first call on that device), `*bytes` its size.  Allocates nothing.
+constexpr int64_t kSplitScratchBytes = 8ll << 20;
+hipError_t split_scratch(void **ptr, int64_t *bytes);
 bool attention_supports(int32_t d);
 // Whether launch_attention runs `a` on grouped tiles: the heads of a KV head's group side by side
 // in one query tile (a decoder step under GQA: no causal or per-row mask, group * t <= 128).

@@ -284,8 +284,10 @@ static int split_count(const svodk_attn *opts, int64_t batch, int64_t t, int64_t
 
 // attend (tk/src/ops/attention.rs:126-303): attention of q, k and v, or of the `packed` operand
 // they are views of.
+// `own_scratch`: the partial states of a split call go to the library's static device array instead
+// of a lent workspace (svodk_attention_noalloc).
 static int attend(const svodk_tensor *q, const svodk_tensor *k, const svodk_tensor *v, const svodk_tensor *packed,
-                  const svodk_attn *opts, const svodk_tensor *out, void *hip_stream) {
+                  const svodk_attn *opts, const svodk_tensor *out, void *hip_stream, bool own_scratch = false) {
   const char *op = OP_ATTN;
   if (!well_formed(q) || !well_formed(k) || !well_formed(v) || !well_formed(out) || opts == nullptr)
     return fail(SVODK_ERR_ARGUMENT, "%s: a null or malformed tensor descriptor", op);
@@ -565,7 +567,19 @@ static int attend(const svodk_tensor *q, const svodk_tensor *k, const svodk_tens
   }
   // L280-302: key splits.  The partial tensors live in the caller's workspace.
   a.splits = split_count(opts, a.batch, t, heads, kv_heads, tk);
-  if (a.splits > 1) {
+  void *workspace = opts->workspace;
+  if (a.splits > 1 && own_scratch) {
+    // The library's own array holds the partial states: a call that needs more than it has is
+    // refused, not shrunk (the caller asked for a call that allocates nothing, and gets that or an error).
+    const int64_t need = (int64_t)a.splits * a.batch * t * heads * (d + 2) * 4;
+    int64_t have = 0;
+    const hipError_t e = svodk::split_scratch(&workspace, &have);
+    if (e != hipSuccess) return fail(SVODK_ERR_LAUNCH, "%s: the static scratch: %s", op, hipGetErrorString(e));
+    if (need > have)
+      return fail(SVODK_ERR_ARGUMENT,
+                  "%s: %d key splits of %lld rows need %lld bytes of partial states, the static scratch holds %lld", op,
+                  a.splits, (long long)((int64_t)a.batch * t * heads), (long long)need, (long long)have);
+  } else if (a.splits > 1) {
     const int64_t rows = (int64_t)a.batch * t * heads;
     int64_t need = (int64_t)a.splits * rows * (d + 2) * 4;
     const bool lent = opts->workspace != nullptr && opts->workspace_bytes >= need;
@@ -576,13 +590,13 @@ static int attend(const svodk_tensor *q, const svodk_tensor *k, const svodk_tens
   if (a.splits > 1) {
     const int64_t rows = (int64_t)a.batch * t * heads;
     const int64_t need = (int64_t)a.splits * rows * (d + 2) * 4;
-    Span ws[2] = {{"workspace", opts->workspace, (size_t)need, true}, {"o", out->data, (size_t)numel(out) * 2, true}};
+    Span ws[2] = {{"workspace", workspace, (size_t)need, true}, {"o", out->data, (size_t)numel(out) * 2, true}};
     if (int rc = check_aliasing(op, ws, 2)) return rc;
     for (int i = 0; i < 3; i++) {
-      Span pair[2] = {{"workspace", opts->workspace, (size_t)need, true}, spans[i]};
+      Span pair[2] = {{"workspace", workspace, (size_t)need, true}, spans[i]};
       if (int rc = check_aliasing(op, pair, 2)) return rc;
     }
-    a.o_part = (float *)opts->workspace;
+    a.o_part = (float *)workspace;
     a.m_part = a.o_part + (int64_t)a.splits * rows * d;
     a.l_part = a.m_part + (int64_t)a.splits * rows;
   }
@@ -610,6 +624,13 @@ int svodk_attention(const svodk_tensor *q, const svodk_tensor *k, const svodk_te
                     const svodk_tensor *out, void *hip_stream) {
   return attend(q, k, v, nullptr, opts, out, hip_stream);
 }
+
+int svodk_attention_noalloc(const svodk_tensor *q, const svodk_tensor *k, const svodk_tensor *v, const svodk_attn *opts,
+                            const svodk_tensor *out, void *hip_stream) {
+  return attend(q, k, v, nullptr, opts, out, hip_stream, /*own_scratch=*/true);
+}
+
+int64_t svodk_noalloc_scratch_bytes(void) { return svodk::kSplitScratchBytes; }
 
 // attention_packed (tk/src/ops/attention.rs:104-122).
 int svodk_attention_packed(const svodk_tensor *qkv, int32_t heads, int32_t kv_heads, const svodk_attn *opts,

@@ -92,6 +92,9 @@ def load_library() -> ctypes.CDLL:
     tp = ctypes.POINTER(_Tensor)
     lib.svodk_attention.restype = ctypes.c_int
     lib.svodk_attention.argtypes = [tp, tp, tp, ctypes.POINTER(_Attn), tp, ctypes.c_void_p]
+    lib.svodk_attention_noalloc.restype = ctypes.c_int
+    lib.svodk_attention_noalloc.argtypes = [tp, tp, tp, ctypes.POINTER(_Attn), tp, ctypes.c_void_p]
+    lib.svodk_noalloc_scratch_bytes.restype = ctypes.c_int64
     lib.svodk_attention_packed.restype = ctypes.c_int
     lib.svodk_attention_packed.argtypes = [tp, ctypes.c_int32, ctypes.c_int32, ctypes.POINTER(_Attn), tp, ctypes.c_void_p]
     lib.svodk_attention_workspace.restype = ctypes.c_int64
@@ -318,6 +321,24 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, opts: Optional[
                                  ctypes.byref(od), ctypes.c_void_p(_stream(q)))
     _finish("attention", status)
     return out
+
+
+def attention_noalloc(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, opts: Attn, out: torch.Tensor) -> torch.Tensor:
+    """``attention`` through ``svodk_attention_noalloc``: the partial states of a split call live in
+    the library's static device array (``noalloc_scratch_bytes()`` per GPU), nothing is allocated
+    below this call, and the caller brings ``out``.  No counterpart in the reference."""
+    lib = load_library()
+    keep: list = []
+    a = _attn_options(opts, keep)
+    qd, kd, vd, od = _desc(q), _desc(k), _desc(v), _desc(out)
+    status = lib.svodk_attention_noalloc(ctypes.byref(qd), ctypes.byref(kd), ctypes.byref(vd), ctypes.byref(a),
+                                         ctypes.byref(od), ctypes.c_void_p(_stream(q)))
+    _finish("attention", status)
+    return out
+
+
+def noalloc_scratch_bytes() -> int:
+    return int(load_library().svodk_noalloc_scratch_bytes())
 
 
 def tune_streaming(workgroups_per_xcd: int) -> None:

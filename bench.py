@@ -25,12 +25,22 @@ import time
 
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of
-# this file, each scaled by what the counter reads for a 256 MiB device copy (x2.000 and x1.000);
-# the summaries are under profiles/.  Counters cannot be read from inside a timed run.
-HBM_TRAFFIC_BYTES = {"bge_m3": 110.32e6, "qwen3_attention": 176.82e6, "qwen3_prologue": 269.01e6,
-                     "qwen3_add_rms_norm": 268.56e6, "whisper": 245.96e6, "whisper_decode": 124.93e6,
-                     "long": 127.44e6}
+ROOT = os.path.dirname(os.path.abspath(__file__))
+# The workloads a default run times after the headline one, a few steps each, so that one run
+# carries every figure the targets are set on.
+OTHERS = ["qwen3_attention", "qwen3_prologue", "whisper", "long"]
+
+
+def hbm_traffic(workload):
+    """HBM bytes per launch of the workload's dominant kernel, from profiles/traffic.json: rocprofv3
+    --pmc FETCH_SIZE and WRITE_SIZE runs of this file, each scaled by what the counter reads for a 256 MiB
+    device copy (the summaries under profiles/ give the commands).  Counters cannot be read from inside a
+    timed run; a workload that has not been profiled reports null."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            return json.load(f).get("bytes_per_launch", {}).get(workload)
+    except (OSError, ValueError):
+        return None
 
 
 def parse():
@@ -52,67 +62,70 @@ def parse():
                     help="bge_m3, bge_m3_bool: take the batch rows as they come instead of ordering them by length once per step")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="rough budget of the CPU baseline sample")
+    ap.add_argument("--no-others", action="store_true",
+                    help="the default workload only: without the shorter runs of the other configurations that a "
+                         "default run appends under \"others\"")
+    ap.add_argument("--other-steps", type=int, default=4, help="timed steps of each workload under \"others\"")
     return ap.parse_args()
 
 
-def main():
-    args = parse()
-    if args.gpus != 1:
-        print("bench.py measures one GPU: this build has no multi-GPU path (every (batch, head, query tile) block is "
-              "independent, so the op shards over batch and heads without exchange); run with --gpus 1.",
-              file=sys.stderr)
-        sys.exit(2)
+class Workload:
+    """A step of one workload: closures that launch on the current stream, and what a launch is worth."""
 
+    def __init__(self):
+        self.calls, self.extra_calls = [], []  # extra: launches of a step that are not calls of the op measured
+        self.flops_vis = self.flops_nom = 0.0
+        self.bytes_min = 0
+        self.kernel_name, self.bound, self.text = "", "mfma", ""
+        self.cpu_sample = None
+        self.keep = []  # what the closures use
+
+    def step(self):
+        for c in self.extra_calls:
+            c()
+        for c in self.calls:
+            c()
+
+
+def build_workload(name, args, dev, row_order=True):
     import torch
 
     import svod_amd
     from svod_amd import Attn, KeyMask, Qkv, workloads as W
 
-    if not torch.cuda.is_available():
-        print("bench.py needs a GPU (torch.cuda.is_available() is False)", file=sys.stderr)
-        sys.exit(2)
-    svod_amd.load_library()
-    if not svod_amd.supported():
-        print("the current device is not a gfx950 this library has kernels for", file=sys.stderr)
-        sys.exit(2)
-    dev = torch.device("cuda:0")
-    props = torch.cuda.get_device_properties(0)
-
-    # ---- build the step: a list of closures launching on the current stream.
-    calls, flops_vis, flops_nom, bytes_min, kernel_name, bound = [], 0.0, 0.0, 0, "", "mfma"
-    extra_calls = []  # launches of a step that are not calls of the op being measured
-    cpu_sample = None
-    if args.workload in ("bge_m3", "bge_m3_bool"):
+    wl = Workload()
+    calls = wl.calls
+    if name in ("bge_m3", "bge_m3_bool"):
         sets = [W.config2(layer=l, device=dev) for l in range(args.layers)]
         # The lengths belong to the batch, not to a layer (every set has the same ones): as a model would,
         # the step orders the batch rows by length once (one small launch, inside the timed region) and
         # hands the order to its 24 layer calls.  --no-row-order runs the rows as they come.
         order = None
-        if not args.no_row_order:
+        if row_order:
             order = torch.empty(sets[0].key_lens.shape, dtype=torch.int32, device=dev)
-            keys0 = sets[0].key_lens if args.workload == "bge_m3" else sets[0].key_mask()
-            extra_calls.append(lambda: svod_amd.order_rows(keys0, out=order))
+            keys0 = sets[0].key_lens if name == "bge_m3" else sets[0].key_mask()
+            wl.extra_calls.append(lambda: svod_amd.order_rows(keys0, out=order))
         for w in sets:
-            keys = KeyMask.lens(w.key_lens) if args.workload == "bge_m3" else KeyMask.bool(w.key_mask())
+            keys = KeyMask.lens(w.key_lens) if name == "bge_m3" else KeyMask.bool(w.key_mask())
             out = torch.empty_like(w.q)
             calls.append((lambda w=w, keys=keys, out=out: svod_amd.attention(
                 w.q, w.k, w.v, Attn(keys=keys, scale=w.scale, row_order=order), out=out)))
         w0 = sets[0]
-        flops_vis, flops_nom, bytes_min = w0.visible_flops(), w0.nominal_flops(), w0.min_bytes()
-        workload = "BGE-M3 encoder self-attention bf16 B32 H16 D64 S512 key-padding U[64,512], %d layer calls/step%s%s" % (
-            args.layers, " (KeyMask::Bool)" if args.workload == "bge_m3_bool" else " (KeyMask::Lens)",
+        wl.flops_vis, wl.flops_nom, wl.bytes_min = w0.visible_flops(), w0.nominal_flops(), w0.min_bytes()
+        wl.text = "BGE-M3 encoder self-attention bf16 B32 H16 D64 S512 key-padding U[64,512], %d layer calls/step%s%s" % (
+            args.layers, " (KeyMask::Bool)" if name == "bge_m3_bool" else " (KeyMask::Lens)",
             ", batch rows ordered by length once per step (svodk_order_rows, in the timed region)" if order is not None else "")
-        cpu_sample = ("attention", w0)
-        kernel_name = "flash_fwd_kernel<64>"
-    elif args.workload == "hbm_copy":
+        wl.cpu_sample = ("attention", w0)
+        wl.kernel_name = "flash_fwd_kernel<64>"
+    elif name == "hbm_copy":
         srcs = [torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255) for _ in range(2)]
         dsts = [torch.empty_like(x) for x in srcs]
         for i in range(args.calls):
             calls.append(lambda i=i: dsts[i % 2].copy_(srcs[i % 2]))
-        bytes_min = 2 * srcs[0].numel()
-        workload = "plain device copy of 256 MiB (torch copy_), counter calibration"
-        kernel_name, bound = "torch elementwise copy", "hbm"
-    elif args.workload == "qwen3_prologue":
+        wl.bytes_min = 2 * srcs[0].numel()
+        wl.text = "plain device copy of 256 MiB (torch copy_), counter calibration"
+        wl.kernel_name, wl.bound = "torch elementwise copy", "hbm"
+    elif name == "qwen3_prologue":
         p = W.config3_prologue(device=dev)
         opts = Qkv(p.heads, p.kv_heads, p.head_dim, p.q_w, p.k_w, p.eps, (p.cos, p.sin))
         ins = [p.qkv] + [p.qkv.clone() for _ in range(3)]
@@ -120,11 +133,11 @@ def main():
                 for _ in range(4)]
         for i in range(args.calls):
             calls.append(lambda i=i: svod_amd.heads(ins[i % 4], opts, out=outs[i % 4]))
-        bytes_min = p.min_bytes()
-        workload = "Qwen3-Embedding prologue bf16 qkv[8,2048,4096] -> q,k,v (RMSNorm eps 1e-6 + RoPE theta 1e6)"
-        cpu_sample = ("heads", p)
-        kernel_name, bound = "heads_kernel<128>", "hbm"
-    elif args.workload == "whisper_decode":
+        wl.bytes_min = p.min_bytes()
+        wl.text = "Qwen3-Embedding prologue bf16 qkv[8,2048,4096] -> q,k,v (RMSNorm eps 1e-6 + RoPE theta 1e6)"
+        wl.cpu_sample = ("heads", p)
+        wl.kernel_name, wl.bound = "heads_kernel<128>", "hbm"
+    elif name == "whisper_decode":
         # One decoder step of Whisper-large-v3's cross-attention (model/src/whisper/decoder.rs:441-477): a query
         # per lane against the 1500 encoder keys of its layer, read from a cache that holds every layer's heads.
         from svod_amd import Cache
@@ -140,11 +153,11 @@ def main():
             calls.append(lambda layer=layer: svod_amd.attention(
                 qs[layer], k_cache, v_cache, Attn(keys=KeyMask.lens(lens), cache=Cache(layer * h, h)), out=outs[layer],
                 workspace=ws))
-        bytes_min = 2 * b * tk * h * d * 2 + 2 * b * h * d * 2  # the layer's K and V heads read once, q and o
-        workload = ("Whisper-large-v3 decoder step, cross-attention bf16 B16 T1 H20 D64 over 1500 cached keys, "
-                    "32 layer calls/step on one cache [16,1500,640,64] (splits chosen by the library)")
-        kernel_name, bound = "flash_fwd_kernel<64, split, cached> + combine_kernel<64>", "hbm"
-    elif args.workload == "qwen3_add_rms_norm":
+        wl.bytes_min = 2 * b * tk * h * d * 2 + 2 * b * h * d * 2  # the layer's K and V heads read once, q and o
+        wl.text = ("Whisper-large-v3 decoder step, cross-attention bf16 B16 T1 H20 D64 over 1500 cached keys, "
+                   "32 layer calls/step on one cache [16,1500,640,64] (splits chosen by the library)")
+        wl.kernel_name, wl.bound = "flash_fwd_kernel<64, split, cached> + combine_kernel<64>", "hbm"
+    elif name == "qwen3_add_rms_norm":
         # The residual add + RMSNorm between Qwen3-Embedding's layers: hidden size 16 heads x 128 = 2048.
         g = torch.Generator(device=dev).manual_seed(0x5EED0030)
         shape = (8, 2048, 2048)
@@ -154,46 +167,49 @@ def main():
         outs = [(torch.empty_like(xs[0]), torch.empty_like(xs[0])) for _ in range(4)]
         for i in range(args.calls):
             calls.append(lambda i=i: svod_amd.add_rms_norm(xs[i % 4], rs[i % 4], wn, 1e-6, out=outs[i % 4]))
-        bytes_min = 4 * xs[0].numel() * 2 + 2 * 2048  # x and residual read, sum and out written, the weight
-        workload = "Qwen3-Embedding residual add + RMSNorm bf16 x,residual [8,2048,2048] -> sum, out (eps 1e-6)"
-        cpu_sample = ("norm", (xs[0], rs[0], wn))
-        kernel_name, bound = "rows_kernel<4, rms, residual>", "hbm"
+        wl.bytes_min = 4 * xs[0].numel() * 2 + 2 * 2048  # x and residual read, sum and out written, the weight
+        wl.text = "Qwen3-Embedding residual add + RMSNorm bf16 x,residual [8,2048,2048] -> sum, out (eps 1e-6)"
+        wl.cpu_sample = ("norm", (xs[0], rs[0], wn))
+        wl.kernel_name, wl.bound = "rows_kernel<4, rms, residual>", "hbm"
     else:
-        if args.workload == "qwen3_attention":
+        if name == "qwen3_attention":
             p = W.config3_prologue(device=dev)
             q, k, v = svod_amd.heads(p.qkv, Qkv(p.heads, p.kv_heads, p.head_dim, p.q_w, p.k_w, p.eps, (p.cos, p.sin)))
             w = W.config3_attention(q, k, v)
-            workload = "Qwen3-Embedding causal GQA attention bf16 B8 S2048 Hq16 Hkv8 D128, right padding U[512,2048]"
-            kernel_name = "flash_fwd_kernel<128, causal>"
-        elif args.workload == "whisper":
+            wl.text = "Qwen3-Embedding causal GQA attention bf16 B8 S2048 Hq16 Hkv8 D128, right padding U[512,2048]"
+            wl.kernel_name = "flash_fwd_kernel<128, causal>"
+        elif name == "whisper":
             w = W.config4(device=dev)
-            workload = "Whisper-large-v3 encoder attention bf16 B16 H20 D64 S1500, no mask"
-            kernel_name = "flash_fwd_kernel<64>"
+            wl.text = "Whisper-large-v3 encoder attention bf16 B16 H20 D64 S1500, no mask"
+            wl.kernel_name = "flash_fwd_kernel<64>"
         else:
             w = W.config5(device=dev)
-            workload = "long-context pair attention bf16 B2 H16 D64 S8192, lens {8192, 5000}"
-            kernel_name = "flash_fwd_kernel<64>"
+            wl.text = "long-context pair attention bf16 B2 H16 D64 S8192, lens {8192, 5000}"
+            wl.kernel_name = "flash_fwd_kernel<64>"
         keys = KeyMask.lens(w.key_lens) if w.key_lens is not None else KeyMask.none()
         ins = [(w.q, w.k, w.v)] + [(w.q.clone(), w.k.clone(), w.v.clone()) for _ in range(3)]
         outs = [torch.empty_like(w.q) for _ in range(4)]
         opts = Attn(causal=w.causal, keys=keys, scale=w.scale)
         for i in range(args.calls):
             calls.append(lambda i=i: svod_amd.attention(*ins[i % 4], opts, out=outs[i % 4]))
-        flops_vis, flops_nom, bytes_min = w.visible_flops(), w.nominal_flops(), w.min_bytes()
-        cpu_sample = ("attention", w)
+        wl.flops_vis, wl.flops_nom, wl.bytes_min = w.visible_flops(), w.nominal_flops(), w.min_bytes()
+        wl.cpu_sample = ("attention", w)
+    return wl
 
-    def step():
-        for c in extra_calls:
-            c()
-        for c in calls:
-            c()
 
+def measure(wl, steps, warmup, use_graph=True, spread=True, warm=True):
+    """Times `steps` steps of the workload between synchronisations, after `warmup` untimed ones and a
+    clock warm-up.  Every launch goes to torch's current stream, which is also where the events are
+    recorded.  Returns ms per step, the average launch duration and the extras asked for."""
+    import torch
+
+    step = wl.step
     # ---- warm-up (also loads the code objects and sets kernel attributes), then capture.
-    for _ in range(max(1, args.warmup)):
+    for _ in range(max(1, warmup)):
         step()
     torch.cuda.synchronize()
     graph = None
-    if not args.no_graph:
+    if use_graph:
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
@@ -229,86 +245,149 @@ def main():
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     wall0 = time.perf_counter()
     e0.record()
-    for _ in range(args.steps):
+    for _ in range(steps):
         run()
     e1.record()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - wall0) * 1e3
     gpu_ms = e0.elapsed_time(e1)
-    ms_per_step = max(wall_ms, gpu_ms) / args.steps
-    launches = len(calls) * args.steps
-    kernel_us = gpu_ms * 1e3 / launches  # average launch duration over the timed region (HIP events)
+    res = {"ms_per_step": max(wall_ms, gpu_ms) / steps,
+           "kernel_us": gpu_ms * 1e3 / (len(wl.calls) * steps),  # average launch duration over the timed region (HIP events)
+           "launch": "hip graph replay" if graph is not None else "eager"}
 
-    # Five more rounds of K steps for the spread (min and median, after the reference tuner's
-    # reporting, runtime/src/benchmark.rs:13-52); the headline stays the timed region above.
-    rounds = []
-    for _ in range(5):
-        r0, r1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        r0.record()
-        for _ in range(args.steps):
-            run()
-        r1.record()
-        r1.synchronize()
-        rounds.append(r0.elapsed_time(r1) / args.steps)
-    rounds.sort()
+    if spread:
+        # Five more rounds of K steps for the spread (min and median, after the reference tuner's
+        # reporting, runtime/src/benchmark.rs:13-52); the headline stays the timed region above.
+        rounds = []
+        for _ in range(5):
+            r0, r1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            r0.record()
+            for _ in range(steps):
+                run()
+            r1.record()
+            r1.synchronize()
+            rounds.append(r0.elapsed_time(r1) / steps)
+        rounds.sort()
+        res["rounds"] = rounds
+    if warm:
+        # The same call back to back on one operand set: operands warm in the Infinity Cache (the
+        # reference's tuner times cold, its probes warm; both are reported, the headline is cold).
+        for c in wl.extra_calls:
+            c()
+        n_warm = max(len(wl.calls) * steps // 4, 8)
+        for _ in range(4):
+            wl.calls[0]()
+        w0, w1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        w0.record()
+        for _ in range(n_warm):
+            wl.calls[0]()
+        w1.record()
+        w1.synchronize()
+        res["warm_us"] = w0.elapsed_time(w1) * 1e3 / n_warm
+    return res
 
-    # The same call back to back on one operand set: operands warm in the Infinity Cache (the
-    # reference's tuner times cold, its probes warm; both are reported, the headline is cold).
-    for c in extra_calls:
-        c()
-    n_warm = max(len(calls) * args.steps // 4, 8)
-    for _ in range(4):
-        calls[0]()
-    w0, w1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    w0.record()
-    for _ in range(n_warm):
-        calls[0]()
-    w1.record()
-    w1.synchronize()
-    warm_us = w0.elapsed_time(w1) * 1e3 / n_warm
 
-    if bound == "mfma":
-        value = flops_vis * len(calls) / (ms_per_step * 1e-3) / 1e12
-        achieved = flops_vis / (kernel_us * 1e-6) / 1e12
-        roof = {"bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": HBM_TRAFFIC_BYTES.get(args.workload),
-                "traffic_unit": "bytes per launch", "kernel": kernel_name,
-                "kernel_us": round(kernel_us, 3), "flops_per_launch_visible": flops_vis,
-                "flops_per_launch_nominal": flops_nom,
-                "nominal_tflops": round(flops_nom / (kernel_us * 1e-6) / 1e12, 2),
-                "hbm_gbs_at_min_bytes": round(bytes_min / (kernel_us * 1e-6) / 1e9, 1)}
+def roofline(name, wl, kernel_us):
+    if wl.bound == "mfma":
+        achieved = wl.flops_vis / (kernel_us * 1e-6) / 1e12
+        return {"bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": hbm_traffic(name),
+                "traffic_unit": "bytes per launch", "kernel": wl.kernel_name,
+                "kernel_us": round(kernel_us, 3), "flops_per_launch_visible": wl.flops_vis,
+                "flops_per_launch_nominal": wl.flops_nom,
+                "nominal_tflops": round(wl.flops_nom / (kernel_us * 1e-6) / 1e12, 2),
+                "hbm_gbs_at_min_bytes": round(wl.bytes_min / (kernel_us * 1e-6) / 1e9, 1)}
+    achieved = wl.bytes_min / (kernel_us * 1e-6) / 1e9
+    return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": hbm_traffic(name),
+            "traffic_unit": "bytes per launch", "kernel": wl.kernel_name,
+            "kernel_us": round(kernel_us, 3), "bytes_per_launch": wl.bytes_min}
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (every (batch, head, query tile) block is "
+              "independent, so the op shards over batch and heads without exchange); run with --gpus 1.",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    import svod_amd
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (torch.cuda.is_available() is False)", file=sys.stderr)
+        sys.exit(2)
+    svod_amd.load_library()
+    if not svod_amd.supported():
+        print("the current device is not a gfx950 this library has kernels for", file=sys.stderr)
+        sys.exit(2)
+    dev = torch.device("cuda:0")
+    props = torch.cuda.get_device_properties(0)
+
+    name = args.workload
+    wl = build_workload(name, args, dev, row_order=not args.no_row_order)
+    m = measure(wl, args.steps, args.warmup, use_graph=not args.no_graph)
+    ms_per_step, kernel_us, rounds = m["ms_per_step"], m["kernel_us"], m["rounds"]
+    roof = roofline(name, wl, kernel_us)
+    calls = wl.calls
+    if wl.bound == "mfma":
+        value = wl.flops_vis * len(calls) / (ms_per_step * 1e-3) / 1e12
         metric, unit = "flash-attn fwd TFLOP/s (visible-pair FLOPs) on 1 MI355X", "TFLOP/s"
     else:
-        value = bytes_min * len(calls) / (ms_per_step * 1e-3) / 1e9
-        achieved = bytes_min / (kernel_us * 1e-6) / 1e9
-        roof = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": HBM_TRAFFIC_BYTES.get(args.workload),
-                "traffic_unit": "bytes per launch", "kernel": kernel_name,
-                "kernel_us": round(kernel_us, 3), "bytes_per_launch": bytes_min}
+        value = wl.bytes_min * len(calls) / (ms_per_step * 1e-3) / 1e9
         metric = {"qwen3_add_rms_norm": "row norm GB/s on 1 MI355X",
                   "whisper_decode": "decoder-step attention GB/s of K and V on 1 MI355X"}.get(
-                      args.workload, "attention prologue GB/s on 1 MI355X")
+                      name, "attention prologue GB/s on 1 MI355X")
         unit = "GB/s"
+
+    config = {"workload": wl.text, "calls_per_step": len(calls), "ms_per_call": round(ms_per_step / len(calls), 5),
+              "launch": m["launch"],
+              "ms_per_step_min": round(rounds[0], 5), "ms_per_step_median": round(rounds[2], 5),
+              "us_per_call_warm": round(m["warm_us"], 2),
+              "operands": "cold: the calls of a step rotate over operand sets larger than the 256 MB Infinity Cache "
+                          "(us_per_call_warm: one set back to back, eager launches)",
+              "device": props.name or props.gcnArchName, "compute_units": props.multi_processor_count,
+              "clock_mhz": props.clock_rate // 1000 if hasattr(props, "clock_rate") else None}
 
     # ---- CPU baseline: the oracle's restatement of the reference graph path, bounded sample.
     cpu = None
-    if not args.no_cpu_baseline and cpu_sample is not None:
-        cpu = cpu_baseline(cpu_sample, args.cpu_seconds, bound)
+    if not args.no_cpu_baseline and wl.cpu_sample is not None:
+        cpu = cpu_baseline(wl.cpu_sample, args.cpu_seconds, wl.bound)
+
+    others = None
+    if name == "bge_m3" and not args.no_others:
+        # The same calls with the batch rows as the caller gave them (no svodk_order_rows, no row_order): the
+        # figure of the op exactly as the reference has it, beside the headline.
+        if not args.no_row_order:
+            plain = build_workload(name, args, dev, row_order=False)
+            pm = measure(plain, max(2, args.steps // 4), 1, use_graph=not args.no_graph, spread=False, warm=False)
+            config["us_per_call_rows_as_given"] = round(pm["kernel_us"], 3)
+            config["frac_rows_as_given"] = roofline(name, plain, pm["kernel_us"])["frac"]
+            del plain
+        del wl
+        torch.cuda.empty_cache()
+        others = []
+        for other in OTHERS:
+            ow = build_workload(other, args, dev)
+            om = measure(ow, args.other_steps, 2, use_graph=not args.no_graph, spread=False, warm=False)
+            r = roofline(other, ow, om["kernel_us"])
+            others.append({"workload": ow.text, "name": other, "calls_per_step": len(ow.calls), "steps": args.other_steps,
+                           "kernel": r["kernel"], "kernel_us": r["kernel_us"], "bound": r["bound"],
+                           "achieved": r["achieved"], "unit": r["unit"], "peak": r["peak"], "frac": r["frac"],
+                           "traffic": r["traffic"]})
+            del ow
+            torch.cuda.empty_cache()
 
     line = {
         "metric": metric, "value": round(value, 3), "unit": unit, "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": workload, "calls_per_step": len(calls), "ms_per_call": round(ms_per_step / len(calls), 5),
-                   "launch": "hip graph replay" if graph is not None else "eager",
-                   "ms_per_step_min": round(rounds[0], 5), "ms_per_step_median": round(rounds[2], 5),
-                   "us_per_call_warm": round(warm_us, 2),
-                   "operands": "cold: the calls of a step rotate over operand sets larger than the 256 MB Infinity Cache "
-                               "(us_per_call_warm: one set back to back, eager launches)",
-                   "device": props.name or props.gcnArchName, "compute_units": props.multi_processor_count,
-                   "clock_mhz": props.clock_rate // 1000 if hasattr(props, "clock_rate") else None},
-        "roofline": roof, "cpu_baseline": cpu,
+        "config": config, "roofline": roof, "cpu_baseline": cpu,
     }
+    if others is not None:
+        line["others"] = others
     print(json.dumps(line))
 
 

@@ -35,6 +35,24 @@
 
 #include "kernels.h"
 
+// A timeline build (-DSVODK_TIMELINE, never the shipped library: svod_amd/probes/timeline.py makes and
+// reads one): thread 0 of every workgroup of flash_fwd_kernel leaves five stamps of the 100 MHz clock
+// (entry, first barrier, last computed step, last step, stores landed), where it ran and what it had to
+// do in the buffer svodk_debug_timeline_h<head size> names, eight 64-bit words a workgroup.
+#if defined(SVODK_TIMELINE) && defined(SVODK_HEAD) && !defined(SVODK_CODE_OBJECT)
+static __device__ unsigned long long *g_timeline = nullptr;
+#define SVODK_TL_CAT2(a, b) a##b
+#define SVODK_TL_CAT(a, b) SVODK_TL_CAT2(a, b)
+extern "C" int SVODK_TL_CAT(svodk_debug_timeline_h, SVODK_HEAD)(void *buf) {
+  return (int)hipMemcpyToSymbol(HIP_SYMBOL(g_timeline), &buf, sizeof(buf));
+}
+#define SVODK_TL_STAMPS unsigned long long tl_stamp[5] = {0, 0, 0, 0, 0}
+#define SVODK_TL(i) asm volatile("s_memrealtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(tl_stamp[i])::"memory")
+#else
+#define SVODK_TL_STAMPS
+#define SVODK_TL(i)
+#endif
+
 namespace svodk {
 #if !defined(SVODK_CODE_OBJECT)
 // Workgroups per XCD of the streaming form (<= 0: a workgroup per query tile instead), and the
@@ -755,6 +773,8 @@ __device__ __forceinline__ void flash_fwd_body(
   // is tile-major, every unit's longest tile, then every unit's next (span = the XCD's units * group
   // workgroups a place), so that the launch ends on short tiles everywhere.
   const uint32_t wg = __builtin_amdgcn_workgroup_id_x();
+  SVODK_TL_STAMPS;
+  SVODK_TL(0);
   const uint32_t local = wg / kXcds;
   uint32_t round, head_in_group;
   int order;
@@ -1022,6 +1042,7 @@ __device__ __forceinline__ void flash_fwd_body(
   // them lands inside the loop, where it would also wait out the fills in flight.
   __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
   __syncthreads();
+  SVODK_TL(1);
 
   // ---- the first block's scores, masked, and their row maximum.
   // A causal wave past its last visible key has nothing to add from a block: it only keeps
@@ -1078,7 +1099,9 @@ __device__ __forceinline__ void flash_fwd_body(
     hot_step<D, NW, 1>(w, smem, blk + 1, nv, sv, bm);
   }
   for (; blk < my_end; blk++) edge_step<D, NW, CAUSAL>(w, smem, blk, my_end, sv, bm);
+  SVODK_TL(2);
   for (; blk < end; blk++) idle_step<D, NW>(w, blk);
+  SVODK_TL(3);
 
   // ---- the appended rows (L739-755, L827-846): one more block of keys, from their own tensors,
   // which only the last split scores; the first `seen` of them are visible and no other mask
@@ -1167,6 +1190,19 @@ __device__ __forceinline__ void flash_fwd_body(
       }
     }
   }
+#if defined(SVODK_TIMELINE) && defined(SVODK_HEAD) && !defined(SVODK_CODE_OBJECT)
+  __builtin_amdgcn_s_waitcnt(0x0f70);  // the stores have landed
+  SVODK_TL(4);
+  if (g_timeline != nullptr && tid == 0) {
+    unsigned hw, xcc;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)\n\ts_getreg_b32 %1, hwreg(HW_REG_XCC_ID)" : "=s"(hw), "=s"(xcc));
+    unsigned long long *at = g_timeline + (size_t)wg * 8;
+    for (int i = 0; i < 5; i++) at[i] = tl_stamp[i];
+    at[5] = ((unsigned long long)xcc << 32) | hw;
+    at[6] = ((unsigned long long)(unsigned)end << 32) | (unsigned)my_end;
+    at[7] = ((unsigned long long)(unsigned)b << 32) | (unsigned)(h << 8 | qt);
+  }
+#endif
 }
 #endif  // __HIP_DEVICE_COMPILE__
 

@@ -77,13 +77,14 @@ def _fresh(shape, dtype, device) -> torch.Tensor:
     return out
 
 
-def load_library() -> ctypes.CDLL:
+def load_library(path: Optional[str] = None) -> ctypes.CDLL:
     """The shared library, loaded once.  Missing library = hard error: there is
-    no other implementation behind these ops."""
+    no other implementation behind these ops.  ``path`` names another build of the same
+    library (the timeline build of ``svod_amd.probes.timeline``) and only counts on the first call."""
     global _lib
     if _lib is not None:
         return _lib
-    path = library_path()
+    path = path or library_path()
     if not os.path.exists(path):
         raise ImportError(
             f"{path} is missing: build it with `python -m svod_amd.build` (hipcc, gfx950). "

@@ -42,7 +42,7 @@ def hipcc() -> str:
 
 # The attention source is compiled once per head size and once for what does not depend on it
 # (its SVODK_HEAD macro), side by side: one translation unit of every instantiation takes minutes.
-ATTENTION_PARTS = [0, 32, 48, 64, 128]
+ATTENTION_PARTS = [0, 32, 48, 64, 128, 256]
 
 
 def build(verbose: bool = False) -> str:

@@ -84,7 +84,7 @@ def entries() -> Dict[str, dict]:
     the config it stands for in the reference's terms."""
     out: Dict[str, dict] = {}
     for dtype in ("bf16", "f16"):
-        for d in (32, 48, 64, 128):
+        for d in (32, 48, 64, 128, 256):
             for causal in (False, True):
                 out[f"svodk_attention_d{d}_{dtype}" + ("_causal" if causal else "")] = {
                     "file": "svodk_attention.co", "source": "attention_kernel.hip", "params": _ATTENTION,
@@ -97,7 +97,7 @@ def entries() -> Dict[str, dict]:
                     plain = out[f"svodk_attention_d{d}_{dtype}" + ("_causal" if causal else "")]
                     out[f"svodk_attention_d{d}_{dtype}" + ("_causal" if causal else "") + "_mask"] = {
                         **plain, "params": _ATTENTION_MASK, "key_mask": True}
-        for d in (32, 48, 64, 128):
+        for d in (32, 48, 64, 128, 256):
             for c, s, r, b, k, g in full_forms():
                 per = ("1" if g else "(heads // kv_heads) * ((t + 127) // 128)") + (" * splits" if s else "")
                 out[full_name(d, dtype, c, s, r, b, k, g)] = {

@@ -133,6 +133,8 @@ struct Tile {
   // 32 wide: rows are 64 bytes, four to the bank period, so 16 rows at one logical chunk spread over
   // the period's 16 chunk places when the chunk is xor-ed with row / 4; a V row is one 64-byte
   // group and four consecutive rows are the whole period as they lie.
+  // 256 wide: rows are two bank periods, every row starts on a period, and row & 15 spreads 16 rows
+  // over the 16 chunk places of a half row as it does for 128.
   __device__ static constexpr int swz_k(int row) {
     return kWide == 32 ? ((row >> 2) & 3) : kWide == 64 ? ((row >> 1) & 7) : (row & 15);
   }
@@ -143,10 +145,15 @@ struct Tile {
   // The byte offset, from a fill instruction's first row, of what the lane at chunk place `pc` of
   // tile row `row` fetches: logical chunk pc ^ swizzle of that row of memory, or an offset past any
   // descriptor's bound where the row has no such chunk.
-  __device__ static int source(int row, int pc, int row_bytes, bool v) {
-    const int chunk = pc ^ (v ? swz_v(row) << 2 : swz_k(row));
+  // `ahead` rows lie between the fill instruction's first row and the tile row the swizzle is the one of
+  // (a wave's later fills of a tile, where they do not share the first's swizzle).
+  __device__ static int source(int row, int pc, int row_bytes, bool v, int ahead = 0) {
+    const int chunk = pc ^ (v ? swz_v(row + ahead) << 2 : swz_k(row + ahead));
     return chunk < kChunks ? row * row_bytes + (chunk << 4) : (int)0xfffffff0u;
   }
+  // A wave's fills of a tile are NW instructions apart; where that is not a whole period of the swizzle
+  // (16 rows) its even and odd fills have a swizzle each.
+  __device__ static constexpr int sources(int nw) { return (nw * (64 / kCpr)) % 16 == 0 ? 1 : 2; }
 };
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
@@ -245,7 +252,9 @@ struct Wave {
   int row_lo, row_hi;
   int lo_last, hi_first, hi_last;
   // per-lane addressing
-  int k_src, v_src;  // global byte offsets of this lane's chunk in this wave's first fill of a tile
+  // global byte offsets of this lane's chunk in this wave's fills of a tile (one per swizzle phase)
+  static constexpr int NS = Tile<D>::sources(NW);
+  int k_src[NS], v_src[NS];
   int k_read[KS], v_read[DB];
   // state
   u32x4 qf[KS];
@@ -271,11 +280,12 @@ struct Wave {
 // the barrier that ends a step).  m0 carries the LDS address of a wave instruction's 1 KiB.
 template <int D, int NW, bool F16, unsigned FLAGS>
 __device__ __forceinline__ void fill_tile(const Wave<D, NW, F16, FLAGS> &w, const uint8_t *base, int64_t bytes, int blk,
-                                          int lds_at, int src, int row_bytes) {
-  // This wave's fills of a tile are NW instructions apart; the swizzle repeats with that period,
-  // so they share the lanes' offsets and differ in the descriptor's base.
+                                          int lds_at, const int (&src)[Tile<D>::sources(NW)], int row_bytes) {
+  // This wave's fills of a tile are NW instructions apart; the swizzle repeats with that period (or
+  // with twice it), so they share the lanes' offsets and differ in the descriptor's base.
   constexpr int kRowsPer = 64 / Tile<D>::kCpr;  // rows a wave instruction covers
-  static_assert((NW * kRowsPer) % 16 == 0, "the swizzle repeats from one of a wave's fills to its next");
+  constexpr int NS = Tile<D>::sources(NW);
+  static_assert((NS * NW * kRowsPer) % 16 == 0, "the swizzle repeats over a wave's fills");
   const int64_t off = (int64_t)blk * kBkv * row_bytes;
 #pragma unroll
   for (int i = 0; i < Wave<D, NW, F16, FLAGS>::CH; i++) {
@@ -283,7 +293,7 @@ __device__ __forceinline__ void fill_tile(const Wave<D, NW, F16, FLAGS> &w, cons
     const i32x4 r = make_rsrc(base + at, bytes - at);
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
                  :
-                 : "s"(lds_at + (w.wave + NW * i) * 1024), "v"(src), "s"(r)
+                 : "s"(lds_at + (w.wave + NW * i) * 1024), "v"(src[i % NS]), "s"(r)
                  : "memory");
   }
 }
@@ -955,8 +965,11 @@ __device__ __forceinline__ void flash_fwd_body(
   {
     const int row = w.wave * kRowsPer + w.lane / TL::kCpr;
     const int pc = w.lane % TL::kCpr;
-    w.k_src = TL::source(row, pc, w.kv_row_bytes, false);
-    w.v_src = TL::source(row, pc, w.kv_row_bytes, true);
+#pragma unroll
+    for (int j = 0; j < W::NS; j++) {
+      w.k_src[j] = TL::source(row, pc, w.kv_row_bytes, false, j * NW * kRowsPer);
+      w.v_src[j] = TL::source(row, pc, w.kv_row_bytes, true, j * NW * kRowsPer);
+    }
   }
   // ---- K(0), V(0), K(1) go first: everything below runs in the shadow of their flight.
   w.nxt_end = 0;  // one item a workgroup
@@ -1119,8 +1132,12 @@ __device__ __forceinline__ void flash_fwd_body(
       {
         const int frow = w.wave * kRowsPer + w.lane / TL::kCpr;
         const int pc = w.lane % TL::kCpr;
-        const int k_src = TL::source(frow, pc, app_row_bytes, false);
-        const int v_src = TL::source(frow, pc, app_row_bytes, true);
+        int k_src[W::NS], v_src[W::NS];
+#pragma unroll
+        for (int j = 0; j < W::NS; j++) {
+          k_src[j] = TL::source(frow, pc, app_row_bytes, false, j * NW * kRowsPer);
+          v_src[j] = TL::source(frow, pc, app_row_bytes, true, j * NW * kRowsPer);
+        }
         fill_tile<D, NW>(w, (const uint8_t *)(rg.k_app + at), bytes, 0, w.lds0, k_src, app_row_bytes);
         fill_tile<D, NW>(w, (const uint8_t *)(rg.v_app + at), bytes, 0, w.lds0 + 2 * TL::kBytes, v_src, app_row_bytes);
       }
@@ -1207,7 +1224,7 @@ __device__ __forceinline__ void flash_fwd_body(
 #endif  // __HIP_DEVICE_COMPILE__
 
 template <int D, int NW, bool CAUSAL, bool SPLIT, bool RANGED, bool BIASED, bool CACHED, bool GROUPED, bool F16>
-__global__ __launch_bounds__(NW * 64, (D <= 64 && !BIASED) ? 3 : 2) void flash_fwd_kernel(
+__global__ __launch_bounds__(NW * 64, (D <= 64 && !BIASED) ? 3 : (D <= 128 ? 2 : 1)) void flash_fwd_kernel(
     uint32_t unit_size, uint32_t unit_rcp, uint32_t nqt_u, uint32_t nqt_rcp, uint32_t kvh_u, uint32_t kvh_rcp,
     uint32_t units, uint32_t heads_group, const void *__restrict__ key_lens, const int32_t *__restrict__ row_order,
     int32_t t, uint32_t tk_lens64, const uint16_t *__restrict__ q, const uint16_t *__restrict__ k,
@@ -1349,8 +1366,11 @@ __global__ __launch_bounds__(NW * 64, 3) void flash_stream_kernel(
   {
     const int row = w.wave * kRowsPer + w.lane / TL::kCpr;
     const int pc = w.lane % TL::kCpr;
-    w.k_src = TL::source(row, pc, w.kv_row_bytes, false);
-    w.v_src = TL::source(row, pc, w.kv_row_bytes, true);
+#pragma unroll
+    for (int j = 0; j < W::NS; j++) {
+      w.k_src[j] = TL::source(row, pc, w.kv_row_bytes, false, j * NW * kRowsPer);
+      w.v_src[j] = TL::source(row, pc, w.kv_row_bytes, true, j * NW * kRowsPer);
+    }
   }
 #pragma unroll
   for (int ks = 0; ks < KS; ks++) w.k_read[ks] = ln * TL::kRowBytes + (((2 * ks + w.g) ^ TL::swz_k(ln)) << 4);
@@ -1764,6 +1784,9 @@ hipError_t launch_attention_d64(const AttnArgs &a, hipStream_t stream) { return 
 #if SVODK_HAS_HEAD(128)
 hipError_t launch_attention_d128(const AttnArgs &a, hipStream_t stream) { return launch_d<128>(a, stream); }
 #endif
+#if SVODK_HAS_HEAD(256)
+hipError_t launch_attention_d256(const AttnArgs &a, hipStream_t stream) { return launch_d<256>(a, stream); }
+#endif
 
 #if SVODK_HAS_COMMON
 std::atomic<int> g_stream_slots{0};
@@ -1777,7 +1800,7 @@ hipError_t launch_order_rows(const void *keys, int32_t elem_bytes, int32_t n, in
   return hipGetLastError();
 }
 
-bool attention_supports(int32_t d) { return d == 32 || d == 48 || d == 64 || d == 128; }
+bool attention_supports(int32_t d) { return d == 32 || d == 48 || d == 64 || d == 128 || d == 256; }
 
 bool attention_groups(const AttnArgs &a) {
   const bool ranged = a.win_left >= 0 || a.chunk_size > 0 || a.seg_start != nullptr;
@@ -1806,6 +1829,7 @@ hipError_t launch_attention(const AttnArgs &a, hipStream_t stream) {
     case 48: return launch_attention_d48(a, stream);
     case 64: return launch_attention_d64(a, stream);
     case 128: return launch_attention_d128(a, stream);
+    case 256: return launch_attention_d256(a, stream);
     default: return hipErrorInvalidValue;
   }
 }
@@ -1931,7 +1955,7 @@ __device__ __forceinline__ void attention_entry_full(uint8_t *smem, SVODK_FULL_P
 #endif
 
 #define SVODK_FULL_ENTRY(D, T, F16, C, S, R, B, K, G)                                                                 \
-  extern "C" __global__ __launch_bounds__(256, ((D) <= 64 && !(B)) ? 3 : 2) void                                      \
+  extern "C" __global__ __launch_bounds__(256, ((D) <= 64 && !(B)) ? 3 : ((D) <= 128 ? 2 : 1)) void                   \
       svodk_attention_full_d##D##_##T##_c##C##s##S##r##R##b##B##k##K##g##G(SVODK_FULL_PARAMS) {                       \
     __shared__ __attribute__((aligned(1024))) uint8_t smem[Tile<D>::kLds + 4 * kScannedBlocks * 8];                   \
     attention_entry_full<D, C, S, R, B, K, G, F16>(smem, SVODK_FULL_ARGS);                                            \
@@ -1958,11 +1982,13 @@ SVODK_FULL_FAMILY(48, bf16, false) SVODK_FULL_FAMILY(48, f16, true)
 SVODK_FULL_FAMILY(64, bf16, false) SVODK_FULL_FAMILY(64, f16, true)
 #elif SVODK_HEAD == 128
 SVODK_FULL_FAMILY(128, bf16, false) SVODK_FULL_FAMILY(128, f16, true)
+#elif SVODK_HEAD == 256
+SVODK_FULL_FAMILY(256, bf16, false) SVODK_FULL_FAMILY(256, f16, true)
 #endif
 #else  // the short records: lengths or a key mask, causal or not
 
 #define SVODK_ATTENTION_ENTRY(NAME, D, CAUSAL, F16)                                                                  \
-  extern "C" __global__ __launch_bounds__(256, (D) <= 64 ? 3 : 2) void NAME(                                          \
+  extern "C" __global__ __launch_bounds__(256, (D) <= 64 ? 3 : ((D) <= 128 ? 2 : 1)) void NAME(                       \
       const uint16_t *__restrict__ q, const uint16_t *__restrict__ k, const uint16_t *__restrict__ v,                 \
       uint16_t *__restrict__ o, const void *__restrict__ key_lens, int32_t batch, int32_t t, int32_t tk, int32_t heads, \
       int32_t kv_heads, int32_t scale_bits) {                                                                         \
@@ -1972,7 +1998,7 @@ SVODK_FULL_FAMILY(128, bf16, false) SVODK_FULL_FAMILY(128, f16, true)
 
 // Behind the ring, the words of the scanned key mask row: a copy a wave.
 #define SVODK_ATTENTION_MASK_ENTRY(NAME, D, CAUSAL, F16)                                                             \
-  extern "C" __global__ __launch_bounds__(256, (D) <= 64 ? 3 : 2) void NAME(                                          \
+  extern "C" __global__ __launch_bounds__(256, (D) <= 64 ? 3 : ((D) <= 128 ? 2 : 1)) void NAME(                       \
       const uint16_t *__restrict__ q, const uint16_t *__restrict__ k, const uint16_t *__restrict__ v,                 \
       uint16_t *__restrict__ o, const void *__restrict__ key_mask, int32_t batch, int32_t t, int32_t tk, int32_t heads, \
       int32_t kv_heads, int32_t scale_bits) {                                                                         \
@@ -1988,6 +2014,8 @@ SVODK_ATTENTION_ENTRY(svodk_attention_d64_bf16, 64, false, false)
 SVODK_ATTENTION_ENTRY(svodk_attention_d64_bf16_causal, 64, true, false)
 SVODK_ATTENTION_ENTRY(svodk_attention_d128_bf16, 128, false, false)
 SVODK_ATTENTION_ENTRY(svodk_attention_d128_bf16_causal, 128, true, false)
+SVODK_ATTENTION_ENTRY(svodk_attention_d256_bf16, 256, false, false)
+SVODK_ATTENTION_ENTRY(svodk_attention_d256_bf16_causal, 256, true, false)
 SVODK_ATTENTION_ENTRY(svodk_attention_d32_f16, 32, false, true)
 SVODK_ATTENTION_ENTRY(svodk_attention_d32_f16_causal, 32, true, true)
 SVODK_ATTENTION_ENTRY(svodk_attention_d48_f16, 48, false, true)
@@ -1996,14 +2024,20 @@ SVODK_ATTENTION_ENTRY(svodk_attention_d64_f16, 64, false, true)
 SVODK_ATTENTION_ENTRY(svodk_attention_d64_f16_causal, 64, true, true)
 SVODK_ATTENTION_ENTRY(svodk_attention_d128_f16, 128, false, true)
 SVODK_ATTENTION_ENTRY(svodk_attention_d128_f16_causal, 128, true, true)
+SVODK_ATTENTION_ENTRY(svodk_attention_d256_f16, 256, false, true)
+SVODK_ATTENTION_ENTRY(svodk_attention_d256_f16_causal, 256, true, true)
 SVODK_ATTENTION_MASK_ENTRY(svodk_attention_d64_bf16_mask, 64, false, false)
 SVODK_ATTENTION_MASK_ENTRY(svodk_attention_d64_bf16_causal_mask, 64, true, false)
 SVODK_ATTENTION_MASK_ENTRY(svodk_attention_d128_bf16_mask, 128, false, false)
 SVODK_ATTENTION_MASK_ENTRY(svodk_attention_d128_bf16_causal_mask, 128, true, false)
+SVODK_ATTENTION_MASK_ENTRY(svodk_attention_d256_bf16_mask, 256, false, false)
+SVODK_ATTENTION_MASK_ENTRY(svodk_attention_d256_bf16_causal_mask, 256, true, false)
 SVODK_ATTENTION_MASK_ENTRY(svodk_attention_d64_f16_mask, 64, false, true)
 SVODK_ATTENTION_MASK_ENTRY(svodk_attention_d64_f16_causal_mask, 64, true, true)
 SVODK_ATTENTION_MASK_ENTRY(svodk_attention_d128_f16_mask, 128, false, true)
 SVODK_ATTENTION_MASK_ENTRY(svodk_attention_d128_f16_causal_mask, 128, true, true)
+SVODK_ATTENTION_MASK_ENTRY(svodk_attention_d256_f16_mask, 256, false, true)
+SVODK_ATTENTION_MASK_ENTRY(svodk_attention_d256_f16_causal_mask, 256, true, true)
 #undef SVODK_ATTENTION_ENTRY
 #undef SVODK_ATTENTION_MASK_ENTRY
 #endif  // SVODK_HEAD

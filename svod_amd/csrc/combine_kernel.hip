@@ -122,6 +122,7 @@ hipError_t launch_combine(const CombineArgs &a, hipStream_t stream) {
     case 48: return a.f16 ? launch<48, true>(a, stream) : launch<48, false>(a, stream);
     case 64: return a.f16 ? launch<64, true>(a, stream) : launch<64, false>(a, stream);
     case 128: return a.f16 ? launch<128, true>(a, stream) : launch<128, false>(a, stream);
+    case 256: return a.f16 ? launch<256, true>(a, stream) : launch<256, false>(a, stream);
     default: return hipErrorInvalidValue;
   }
 }
@@ -144,10 +145,12 @@ SVODK_COMBINE_ENTRY(svodk_combine_d32_bf16, 32, false)
 SVODK_COMBINE_ENTRY(svodk_combine_d48_bf16, 48, false)
 SVODK_COMBINE_ENTRY(svodk_combine_d64_bf16, 64, false)
 SVODK_COMBINE_ENTRY(svodk_combine_d128_bf16, 128, false)
+SVODK_COMBINE_ENTRY(svodk_combine_d256_bf16, 256, false)
 SVODK_COMBINE_ENTRY(svodk_combine_d32_f16, 32, true)
 SVODK_COMBINE_ENTRY(svodk_combine_d48_f16, 48, true)
 SVODK_COMBINE_ENTRY(svodk_combine_d64_f16, 64, true)
 SVODK_COMBINE_ENTRY(svodk_combine_d128_f16, 128, true)
+SVODK_COMBINE_ENTRY(svodk_combine_d256_f16, 256, true)
 #undef SVODK_COMBINE_ENTRY
 
 }  // namespace

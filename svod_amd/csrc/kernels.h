@@ -123,6 +123,7 @@ hipError_t launch_attention_d32(const AttnArgs &a, hipStream_t stream);
 hipError_t launch_attention_d48(const AttnArgs &a, hipStream_t stream);
 hipError_t launch_attention_d64(const AttnArgs &a, hipStream_t stream);
 hipError_t launch_attention_d128(const AttnArgs &a, hipStream_t stream);
+hipError_t launch_attention_d256(const AttnArgs &a, hipStream_t stream);
 // order[p] = the batch row with the p-th most keys (ties by row), for AttnArgs::row_order.  `keys` is
 // [n] lengths (tk < 0; elements of 4 or 8 bytes) or an [n, tk] key mask (elements of 1 or 4 bytes).
 constexpr int32_t kMaxOrderedRows = 8192;

@@ -50,11 +50,9 @@ def test_every_op_falls_back_alike(has_target, dtypes, static_dims, why):
     assert svod_amd.plan_heads(has_target, dtypes, x, 64) == why
 
 
-# ---- ops_plan.rs:1241-1262 (attention_plans).  The reference plans d in {32, 48, 64, 128, 256}
-# and sends d = 40 to the graph; this library's kernel is built for d in {32, 48, 64, 128} and sends
-# 256 to the graph with the same reason, Fallback::Shape.
-@pytest.mark.parametrize("d,want", [(32, None), (48, None), (64, None), (128, None), (40, Fallback.Shape),
-                                    (256, Fallback.Shape)])
+# ---- ops_plan.rs:1241-1262 (attention_plans): d in {32, 48, 64, 128, 256} plan a kernel, d = 40 goes to the graph.
+@pytest.mark.parametrize("d,want", [(32, None), (48, None), (64, None), (128, None), (256, None), (40, Fallback.Shape),
+                                    (512, Fallback.Shape)])
 def test_attention_plans(d, want):
     assert svod_amd.plan_attention(True, [BF16] * 3, [2, 100, 8, d], [2, 37, 2, d]) == want
 

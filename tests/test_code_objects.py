@@ -41,7 +41,7 @@ def test_the_record_is_packed_as_the_loader_packs_it():
 
 def test_every_kernel_meets_the_loaders_conditions(built):
     table = co.entries()
-    assert len(table) == 52 + 4 * 2 * 32 + 8  # the short records, every form of every head size and type, the merges
+    assert len(table) == 60 + 5 * 2 * 32 + 10  # the short records, every form of every head size and type, the merges
     assert len(list(co.full_forms())) == 32
     for name, e in table.items():
         kd = co.check(built[e["file"]], name, e["params"])

@@ -28,7 +28,7 @@ HBM_PEAK_GBS = 8000.0
 ROOT = os.path.dirname(os.path.abspath(__file__))
 # The workloads a default run times after the headline one, a few steps each, so that one run
 # carries every figure the targets are set on.
-OTHERS = ["qwen3_attention", "qwen3_prologue", "whisper", "long"]
+OTHERS = ["qwen3_attention", "qwen3_prologue", "whisper", "long", "qwen3_projection"]
 
 
 def hbm_traffic(workload):
@@ -50,7 +50,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="bge_m3",
                     choices=["bge_m3", "bge_m3_bool", "qwen3_attention", "qwen3_prologue", "qwen3_add_rms_norm",
-                             "whisper", "whisper_decode", "long", "hbm_copy"],
+                             "whisper", "whisper_decode", "long", "qwen3_projection", "qwen3_projection_plain", "hbm_copy"],
                     help="hbm_copy is a plain 256 MiB device copy: the known-size kernel the HBM counters "
                          "(FETCH_SIZE, WRITE_SIZE) are calibrated on")
     ap.add_argument("--layers", type=int, default=24, help="calls per step for the bge_m3 workloads")
@@ -137,6 +137,28 @@ def build_workload(name, args, dev, row_order=True):
         wl.text = "Qwen3-Embedding prologue bf16 qkv[8,2048,4096] -> q,k,v (RMSNorm eps 1e-6 + RoPE theta 1e6)"
         wl.cpu_sample = ("heads", p)
         wl.kernel_name, wl.bound = "heads_kernel<128>", "hbm"
+    elif name in ("qwen3_projection", "qwen3_projection_plain"):
+        # The fused q/k/v projection at Qwen3-Embedding's shape with the rope applied in the GEMM's store (what a
+        # model without QK norms runs, tk/src/ops/linear.rs:47-58): x [8,2048,1024] . w [4096,1024]^T, 16 + 8 heads
+        # of 128 turned.  The plain form is the same GEMM without the turn.
+        from svod_amd import Linear, Rotary
+        g = torch.Generator(device=dev).manual_seed(0x5EED0038)
+        b, t, k, h, hkv, d = 8, 2048, 1024, 16, 8, 128
+        n = (h + 2 * hkv) * d
+        xs = [torch.randn((b, t, k), generator=g, device=dev).to(torch.bfloat16) for _ in range(4)]
+        wt = (torch.randn((n, k), generator=g, device=dev) / 32).to(torch.bfloat16)
+        cos, sin = W.rope_table(1e6, t, d, dev)
+        cos, sin = (a.to(torch.bfloat16).reshape(1, t, 1, d // 2) for a in (cos, sin))
+        outs = [torch.empty((b, t, n), dtype=torch.bfloat16, device=dev) for _ in range(4)]
+        opts = Linear(rope=Rotary(cos, sin, h + hkv, d)) if name == "qwen3_projection" else Linear()
+        for i in range(args.calls):
+            calls.append(lambda i=i: svod_amd.linear(xs[i % 4], wt, opts, out=outs[i % 4]))
+        wl.flops_vis = wl.flops_nom = 2.0 * b * t * n * k
+        wl.bytes_min = (xs[0].numel() + wt.numel() + outs[0].numel()) * 2
+        wl.text = ("fused q/k/v projection bf16 x[8,2048,1024] . w[4096,1024]^T" +
+                   (", 24 heads of 128 turned in the store (rope theta 1e6)" if name == "qwen3_projection" else ", no turn"))
+        wl.kernel_name = "linear_kernel<rope 128>" if name == "qwen3_projection" else "linear_kernel"
+        wl.cpu_sample = ("linear", (xs[0], wt, cos, sin, h + hkv, d))
     elif name == "whisper_decode":
         # One decoder step of Whisper-large-v3's cross-attention (model/src/whisper/decoder.rs:441-477): a query
         # per lane against the 1500 encoder keys of its layer, read from a cache that holds every layer's heads.
@@ -335,6 +357,8 @@ def main():
     if wl.bound == "mfma":
         value = wl.flops_vis * len(calls) / (ms_per_step * 1e-3) / 1e12
         metric, unit = "flash-attn fwd TFLOP/s (visible-pair FLOPs) on 1 MI355X", "TFLOP/s"
+        if name.startswith("qwen3_projection"):
+            metric = "fused projection GEMM TFLOP/s on 1 MI355X"
     else:
         value = wl.bytes_min * len(calls) / (ms_per_step * 1e-3) / 1e9
         metric = {"qwen3_add_rms_norm": "row norm GB/s on 1 MI355X",
@@ -413,6 +437,20 @@ def cpu_baseline(sample, seconds, bound):
         return {"value": round(nbytes / dt / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
                 "sample": f"{rows} rows of one call (x, residual [{rows},2048]), f32 restatement of the graph path, "
                           f"scalar C, {reps} reps"}
+    if kind == "linear":
+        x, wt, cos, sin, heads, d = w
+        rows = 4
+        xs = x[:1, :rows].float().cpu().numpy()
+        wn = wt.float().cpu().numpy()
+        rope = (cos[0, :rows, 0].float().cpu().numpy(), sin[0, :rows, 0].float().cpu().numpy(), heads, d)
+        t0 = time.perf_counter()
+        reps = 0
+        while time.perf_counter() - t0 < min(seconds, 5.0):
+            oracle.linear_kernel(xs, wn, None, rope)
+            reps += 1
+        dt = (time.perf_counter() - t0) / reps
+        return {"value": round(2.0 * rows * wn.shape[0] * wn.shape[1] / dt / 1e12, 6), "unit": "TFLOP/s", "cores": 1,
+                "kind": "port", "sample": f"{rows} rows of batch 0, f32 restatement of the kernel's arithmetic, scalar C, {reps} reps"}
     if kind == "heads":
         rows = 256
         qkv = w.qkv[:1, :rows].float().cpu().numpy()

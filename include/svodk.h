@@ -23,7 +23,7 @@
 extern "C" {
 #endif
 
-#define SVODK_ABI_VERSION 4
+#define SVODK_ABI_VERSION 5
 
 /* Element types of a tensor descriptor. */
 typedef enum svodk_dtype {
@@ -215,6 +215,51 @@ int64_t svodk_attention_workspace(const svodk_tensor *q, const svodk_tensor *k, 
  */
 int svodk_heads(const svodk_tensor *qkv, const svodk_qkv *opts, const svodk_tensor *q, const svodk_tensor *k,
                 const svodk_tensor *v, void *hip_stream);
+
+/*
+ * Rotary of tk/src/ops/linear.rs:47-58: the output's first `heads` heads of `head_dim` columns are
+ * turned by the tables' row of the token's position, halves paired as in svodk_heads; tables
+ * [1, T, 1, head_dim/2] of the operands' type.
+ */
+typedef struct svodk_rotary {
+  const svodk_tensor *cos, *sin;
+  int32_t heads, head_dim;
+} svodk_rotary;
+
+/* Act of tk/src/ops/mod.rs (the activation of a Linear). */
+typedef enum svodk_act { SVODK_ACT_NONE = 0, SVODK_ACT_GELU = 1, SVODK_ACT_SILU = 2 } svodk_act;
+
+/*
+ * Linear of tk/src/ops/linear.rs:24-45.  Zero-initialise, then set fields.  This library's GEMM
+ * carries a bias and the rope; an activation, a gated weight, a residual, a scale (the rest of the
+ * reference's GEMM family) answer SVODK_GRAPH_CONFIG, as does a rope with a head size other than 64
+ * or 128 (no tile of the kernel holds its heads: the reference then rotates on the graph after a
+ * plain kernel, tk/src/ops/linear.rs:176-184).
+ */
+typedef struct svodk_linear_opts {
+  const svodk_tensor *bias; /* [N] or NULL */
+  int32_t act;              /* svodk_act */
+  int32_t gated;
+  const svodk_tensor *residual; /* [B, T, N] or NULL */
+  int32_t has_scale;
+  float scale;
+  const svodk_rotary *rope; /* or NULL */
+  int32_t batch_live;       /* as in svodk_attn */
+} svodk_linear_opts;
+
+/*
+ * ops::linear (tk/src/ops/linear.rs:60-231) for a fused projection: x [B, T, K] . w [N, K]^T
+ * (+ bias) -> out [B, T, N], the rope applied in the GEMM's store (tk/src/kernels/gemm.rs:604-645,
+ * 666-716): a model without QK norms gets its rotated queries and keys and its plain values from the
+ * projection itself and needs no svodk_heads pass (svodk_attention_packed then reads `out` in place).
+ * f32 accumulators, one rounding at the store.  N a multiple of 8 (tk/src/ops/shape.rs:133-136);
+ * K a multiple of 32 here (others answer SVODK_GRAPH_SHAPE).
+ */
+int svodk_linear(const svodk_tensor *x, const svodk_tensor *w, const svodk_linear_opts *opts, const svodk_tensor *out,
+                 void *hip_stream);
+/* shape::linear (tk/src/ops/shape.rs:120-139) as a pure function: x_dims [.., K], n the output's columns. */
+int svodk_plan_linear(int32_t has_target, const int32_t *dtypes, int32_t n_dtypes, const int64_t *x_dims, int32_t x_rank,
+                      int64_t n);
 
 /*
  * ops::layer_norm, add_layer_norm, rms_norm, add_rms_norm (tk/src/ops/norm.rs:16-42 -> norm, :44-98):

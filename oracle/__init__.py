@@ -133,6 +133,11 @@ def _declare(l: ctypes.CDLL) -> None:
     l.svod_oracle_attention_flash.argtypes = common + [_i32, _i32, _i32, _f32p, _f32p, _f32p, _f32p, _i32]
     l.svod_oracle_attention_flash_split.restype = ctypes.c_int
     l.svod_oracle_attention_flash_split.argtypes = common + [_i32, _i32, _i32, _i32, _f32p, _f32p, _f32p, _f32p, _i32]
+    lin = [ctypes.c_int64, _i32, _i32, _i32, _f32p, _f32p, _f32p, _i32, _i32, _f32p, _f32p]
+    l.svod_oracle_linear_direct.restype = ctypes.c_int
+    l.svod_oracle_linear_direct.argtypes = lin + [_f64p]
+    l.svod_oracle_linear_kernel.restype = ctypes.c_int
+    l.svod_oracle_linear_kernel.argtypes = lin + [_f32p]
     heads = [_i32] * 5 + [_i32, _i32, ctypes.c_double, _i32] + [_f32p] * 5 + [_f32p] * 3
     for name in ("svod_oracle_heads_direct", "svod_oracle_heads_kernel", "svod_oracle_heads_graph"):
         getattr(l, name).restype = ctypes.c_int
@@ -466,3 +471,37 @@ def norm_f32(kind: int, x, w, b=None, residual=None, eps: float = 1e-5):
     if rc:
         raise ValueError(f"oracle norm_f32 rejected the problem (rc={rc})")
     return out, total
+
+
+# --------------------------------------------------------------------------
+# linear with the rope epilogue
+# --------------------------------------------------------------------------
+def _linear(fn_name: str, x, w, bias, rope, out_dtype, out_ptr):
+    x, w = _f32(x), _f32(w)
+    if x.ndim != 3 or w.ndim != 2 or w.shape[1] != x.shape[2]:
+        raise ValueError("linear: x [B, T, K] and w [N, K]")
+    b, t, k = x.shape
+    n = w.shape[0]
+    bias = None if bias is None else _f32(bias)
+    heads = head_dim = 0
+    cos = sin = None
+    if rope is not None:
+        cos, sin, heads, head_dim = rope
+        cos, sin = _f32(cos).reshape(t, head_dim // 2), _f32(sin).reshape(t, head_dim // 2)
+    out = np.empty((b, t, n), dtype=out_dtype)
+    rc = getattr(lib(), fn_name)(b * t, t, k, n, _ptr(x, _f32p), _ptr(w, _f32p), _ptr(bias, _f32p), heads, head_dim,
+                                  _ptr(cos, _f32p), _ptr(sin, _f32p), _ptr(out, out_ptr))
+    if rc:
+        raise ValueError(f"oracle {fn_name} rejected the problem (rc={rc})")
+    return out
+
+
+def linear_direct(x, w, bias=None, rope=None) -> np.ndarray:
+    """``x [B,T,K] . w [N,K]^T + bias`` with the first ``heads`` heads turned, ``rope = (cos, sin, heads, head_dim)``
+    with tables ``[T, head_dim/2]``: the unrounded f64 reference of tk/src/test/unit/ops.rs:148-158."""
+    return _linear("svod_oracle_linear_direct", x, w, bias, rope, np.float64, _f64p)
+
+
+def linear_kernel(x, w, bias=None, rope=None) -> np.ndarray:
+    """The same in the kernel's f32 arithmetic (tk/src/kernels/gemm.rs:604-716), rounded once to the stream dtype."""
+    return _linear("svod_oracle_linear_kernel", x, w, bias, rope, np.float32, _f32p)

@@ -61,6 +61,15 @@
  *       (tk/src/test/unit/rows.rs:223); the ORDER of its row sums is this
  *       file's own (neither the kernel nor the graph fixes one), so its bit
  *       patterns are "parity unpinned" below that tolerance.
+ *   svod_oracle_linear_direct
+ *       pinned by an independent numpy float64 evaluation (a matmul, and the
+ *       rotation as a complex product (y1 + i y2)(cos + i sin)) and closed
+ *       forms (zero angles leave the product, a turn preserves each pair's
+ *       norm, columns past the turned heads are the plain product).
+ *   svod_oracle_linear_kernel
+ *       pinned against svod_oracle_linear_direct within the reference's 2e-2
+ *       (tk/src/test/unit/ops.rs:312); the ORDER of its f32 dot products is this
+ *       file's own, so its bit patterns are "parity unpinned" below that.
  *   svod_oracle_rope_table
  *       restates tensor/src/transformer.rs:130-164 with libm powf/cosf/sinf;
  *       the reference evaluates pow/cos/sin through its own f32 graph
@@ -1001,5 +1010,78 @@ int svod_oracle_norm_f32(int32_t kind, int64_t rows, int32_t d, double eps, cons
     }
   }
   free(row);
+  return 0;
+}
+
+/* ------------------------------------------------------------------ */
+/* linear with the rope epilogue: y = x . w^T + bias, the first `heads` */
+/* heads of `head_dim` columns turned by the tables' row of the token's */
+/* position (tk/src/ops/linear.rs:47-58, 303-347; the turn is           */
+/* apply_rotary_emb on split halves, tensor/src/transformer.rs:72-117:  */
+/* y1' = y1 cos - y2 sin, y2' = y2 cos + y1 sin).  x [rows, k] with     */
+/* row r at position r % t, w [n, k], bias [n] or NULL, cos and sin     */
+/* [t, head_dim / 2] or NULL (no turn), out [rows, n].                  */
+/* ------------------------------------------------------------------ */
+
+/* The reference of tk/src/test/unit/ops.rs:148-158 (the graph over unrounded copies), in f64. */
+int svod_oracle_linear_direct(int64_t rows, int32_t t, int32_t k, int32_t n, const float *x, const float *w,
+                              const float *bias, int32_t heads, int32_t head_dim, const float *cos_t, const float *sin_t,
+                              double *out) {
+  if (rows < 0 || t <= 0 || k <= 0 || n <= 0) return -1;
+  const int turn = cos_t != NULL && sin_t != NULL;
+  if (turn && (head_dim <= 0 || head_dim % 2 != 0 || (int64_t)heads * head_dim > n)) return -2;
+  const int32_t half = head_dim / 2;
+  for (int64_t r = 0; r < rows; r++) {
+    double *y = out + r * n;
+    for (int32_t c = 0; c < n; c++) {
+      double acc = 0.0;
+      for (int32_t i = 0; i < k; i++) acc += (double)x[r * k + i] * (double)w[(int64_t)c * k + i];
+      y[c] = acc + (bias ? (double)bias[c] : 0.0);
+    }
+    if (!turn) continue;
+    const int64_t pos = r % t;
+    for (int32_t h = 0; h < heads; h++) {
+      for (int32_t i = 0; i < half; i++) {
+        const double c = cos_t[pos * half + i], sn = sin_t[pos * half + i];
+        const double y1 = y[h * head_dim + i], y2 = y[h * head_dim + half + i];
+        y[h * head_dim + i] = y1 * c - y2 * sn;
+        y[h * head_dim + half + i] = y2 * c + y1 * sn;
+      }
+    }
+  }
+  return 0;
+}
+
+/* The kernel's arithmetic (tk/src/kernels/gemm.rs:604-645 finish, :666-716 turn): f32 accumulators,
+ * the bias added in f32, x cos rounded to f32 and the partner's product joined by one fused
+ * multiply-add, sin negated over a head's first half; one rounding to the stream dtype at the store. */
+int svod_oracle_linear_kernel(int64_t rows, int32_t t, int32_t k, int32_t n, const float *x, const float *w,
+                              const float *bias, int32_t heads, int32_t head_dim, const float *cos_t, const float *sin_t,
+                              float *out) {
+  if (rows < 0 || t <= 0 || k <= 0 || n <= 0) return -1;
+  const int turn = cos_t != NULL && sin_t != NULL;
+  if (turn && (head_dim <= 0 || head_dim % 2 != 0 || (int64_t)heads * head_dim > n)) return -2;
+  const int32_t half = head_dim / 2;
+  float *y = (float *)malloc(sizeof(float) * (size_t)n);
+  for (int64_t r = 0; r < rows; r++) {
+    for (int32_t c = 0; c < n; c++) {
+      float acc = 0.0f;
+      for (int32_t i = 0; i < k; i++) acc = fmaf(x[r * k + i], w[(int64_t)c * k + i], acc);
+      y[c] = bias ? acc + bias[c] : acc;
+    }
+    const int64_t pos = r % t;
+    for (int32_t c = 0; c < n; c++) {
+      float v = y[c];
+      if (turn && c < heads * head_dim) {
+        const int32_t in_head = c % head_dim, i = in_head % half;
+        const int first = in_head < half;
+        const float partner = y[first ? c + half : c - half];
+        const float sn = first ? -sin_t[pos * half + i] : sin_t[pos * half + i];
+        v = fmaf(partner, sn, y[c] * cos_t[pos * half + i]);
+      }
+      out[r * n + c] = round_stream(v);
+    }
+  }
+  free(y);
   return 0;
 }

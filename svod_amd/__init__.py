@@ -8,11 +8,14 @@ the HIP kernels under ``csrc/``.  PyTorch is used for device memory and streams
 only.
 """
 from .ops import (  # noqa: F401
+    Act,
     Attn,
     Cache,
     Fallback,
     GraphFallback,
     KeyMask,
+    Linear,
+    Rotary,
     OpError,
     Qkv,
     add_layer_norm,
@@ -25,6 +28,8 @@ from .ops import (  # noqa: F401
     chosen,
     heads,
     layer_norm,
+    linear,
+    plan_linear,
     library_path,
     load_library,
     order_rows,

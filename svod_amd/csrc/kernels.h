@@ -43,6 +43,25 @@ hipError_t launch_norm(const NormArgs &a, hipStream_t stream);
 // Row widths the norm kernel is built for.
 bool norm_supports(int64_t d);
 
+// linear with the rope epilogue: tk/src/kernels/gemm.rs (gemm_body, finish :604-645, turn :666-716).
+struct LinearArgs {
+  const void *x;     // [rows, k]
+  const void *w;     // [n, k]
+  const void *bias;  // [n] or null
+  const void *cos;   // [seq, head_dim / 2] or null: no turn
+  const void *sin;
+  void *y;           // [rows, n]
+  int64_t rows;      // live batches * seq
+  int32_t n, k;
+  int32_t seq;       // row r is the token at position r % seq
+  int32_t heads, head_dim;  // the first heads * head_dim columns are turned
+  int32_t f16;
+};
+hipError_t launch_linear(const LinearArgs &a, hipStream_t stream);
+// Shapes the GEMM kernel takes (n a multiple of 8, k a multiple of 32), and head sizes it turns.
+bool linear_supports(int64_t n, int64_t k);
+bool linear_turns(int32_t head_dim);
+
 // Flash attention forward: tk/src/kernels/attention.rs:466-924 (attention_body).
 struct AttnArgs {
   const void *q;  // [batch, t, heads, d] bf16

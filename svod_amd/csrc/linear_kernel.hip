@@ -1,0 +1,337 @@
+// linear with the rope epilogue for gfx950 (MI355X): y = x . w^T + bias over x [rows, K] and w [N, K]
+// (both K-contiguous), the first `heads` heads of `head_dim` output columns turned by the rotary tables'
+// row of the token's position before the one rounding at the store.  The algorithm is the reference GEMM
+// kernel's epilogue (tk/src/kernels/gemm.rs:604-645 `finish`, :666-716 `turn`): f32 accumulators, the bias
+// added in f32, then per turned column  y = fma(partner, +-sin, x * cos)  with the partner half a head
+// along and sin negated over a head's first half, then the cast.  A fused projection's queries and keys
+// come out rotated and its values plain, so a model without QK norms needs no prologue pass at all
+// (tk/src/ops/linear.rs:47-58).
+//
+// The mapping onto CDNA4 is this file's own.  A workgroup of 8 waves owns a 256 x 256 output tile; a wave
+// owns 64 rows x 128 columns as 2 x 4 accumulators of v_mfma_f32_32x32x16.  The product runs transposed,
+// C^T = W . X^T, so that a lane owns one output ROW and, per accumulator register quad, four CONSECUTIVE
+// columns: the store is 8-byte runs, the rotation's partner column (32 or 64 columns along) is the same
+// lane's register of another accumulator, and the tables are read as 8-byte runs of the lane's row.
+// X and W tiles of 32 k-columns stream through a four-stage LDS ring (32 KiB a stage), filled global -> LDS
+// by buffer_load_dwordx4 ... lds three stages ahead; rows are 64 bytes, their four 16-byte chunks
+// XOR-swizzled by (row / 4) % 4 through the lanes' source addresses so that a ds_read_b128 of 16 rows at one
+// logical chunk touches every bank once.  Rows past the operands' ends read as zeros through the buffer
+// descriptors' bounds.  One barrier a stage (16 MFMAs a wave).
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+
+#include "kernels.h"
+
+namespace svodk {
+namespace {
+
+#if !defined(__HIP_DEVICE_COMPILE__)
+#pragma clang diagnostic ignored "-Wunused-function"
+#pragma clang diagnostic ignored "-Wunused-const-variable"
+#endif
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+typedef __attribute__((ext_vector_type(4))) int i32x4;
+
+constexpr int kXcds = 8;
+constexpr int kWaves = 8;               // 4 along the rows x 2 along the columns
+constexpr int kBm = 256, kBn = 256;     // the workgroup's output tile
+constexpr int kBk = 32;                 // k-columns a stage
+constexpr int kStages = 4;
+constexpr int kRowBytes = kBk * 2;      // a tile row in LDS
+constexpr int kTileBytes = kBm * kRowBytes;           // one operand's tile: 16 KiB
+constexpr int kStageBytes = 2 * kTileBytes;           // W tile, then X tile
+constexpr int kLds = kStages * kStageBytes;           // 128 KiB
+constexpr int kFills = 2 * (kTileBytes / 1024) / kWaves;  // wave instructions of 1 KiB per wave and stage: 4
+
+template <bool F16>
+__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+  f32x2 f = {lo, hi};
+  if constexpr (F16)
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, f16x2));
+  else
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
+}
+
+// One 16-bit element of the operands' type as f32.
+template <bool F16>
+__device__ __forceinline__ float widen(uint32_t bits16) {
+  if constexpr (F16) return (float)__builtin_bit_cast(_Float16, (uint16_t)bits16);
+  return __builtin_bit_cast(float, bits16 << 16);
+}
+
+template <bool F16>
+__device__ __forceinline__ f32x16 mma(const u32x4 &a, const u32x4 &b, const f32x16 &c) {
+  if constexpr (F16)
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+
+// A raw buffer descriptor over `bytes` bytes at `base`: loads past the end return zero.
+__device__ __forceinline__ i32x4 make_rsrc(const void *base, int64_t bytes) {
+  const int64_t clamped = bytes < 0 ? 0 : (bytes > 0xffffffffLL ? 0xffffffffLL : bytes);
+  const uint64_t addr = (uint64_t)(uintptr_t)base;
+  i32x4 r;
+  r[0] = (int)(uint32_t)addr;
+  r[1] = (int)(uint32_t)((addr >> 32) & 0xffffu);
+  r[2] = (int)(uint32_t)clamped;
+  r[3] = 0x00020000;
+  return r;
+}
+
+// Four 16-bit elements at `p` (8-byte aligned) as f32.
+template <bool F16>
+__device__ __forceinline__ void load4(const uint16_t *p, float (&out)[4]) {
+  const u32x2 x = *reinterpret_cast<const u32x2 *>(p);
+  out[0] = widen<F16>(x[0] & 0xffffu);
+  out[1] = widen<F16>(x[0] >> 16);
+  out[2] = widen<F16>(x[1] & 0xffffu);
+  out[3] = widen<F16>(x[1] >> 16);
+}
+
+#if defined(__HIP_DEVICE_COMPILE__)
+// HD: the head size a turning kernel is built for (64 or 128), 0: no turn.
+template <bool F16, int HD>
+__device__ __forceinline__ void linear_body(uint8_t *smem, const uint16_t *__restrict__ x, const uint16_t *__restrict__ w,
+                                            const uint16_t *__restrict__ bias, const uint16_t *__restrict__ cos_t,
+                                            const uint16_t *__restrict__ sin_t, uint16_t *__restrict__ y, int64_t rows,
+                                            int32_t n, int32_t k, int32_t seq, int32_t heads, uint32_t tiles_n,
+                                            uint32_t tiles, uint32_t per_xcd) {
+  const int tid = __builtin_amdgcn_workitem_id_x();
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int g = lane >> 5, ln = lane & 31;
+  // Workgroups are dealt to the 8 XCDs in turn, so XCD x takes a run of consecutive tiles, column tile
+  // fastest: its workgroups share x's row tile and walk w through one L2.
+  const uint32_t wg = __builtin_amdgcn_workgroup_id_x();
+  const uint32_t tile = (wg % kXcds) * per_xcd + wg / kXcds;
+  if (wg / kXcds >= per_xcd || tile >= tiles) return;
+  const uint32_t tm = tile / tiles_n, tn = tile - tm * tiles_n;
+  const int64_t m0 = (int64_t)tm * kBm;
+  const int32_t n0 = (int32_t)tn * kBn;
+  const int64_t row_bytes = (int64_t)k * 2;
+
+  // ---- this wave's fills of a stage: 16 rows x 4 chunk places an instruction, rows 16 * wave and
+  // 128 + 16 * wave of the W tile and of the X tile.  The swizzle's period is 16 rows, so one lane
+  // offset serves all four; the descriptors' bases differ.
+  const int frow = lane >> 2, place = lane & 3;
+  const int src = frow * (int)row_bytes + ((place ^ ((frow >> 2) & 3)) << 4);
+  i32x4 rsrc[kFills];
+  int lds_at[kFills];
+#pragma unroll
+  for (int f = 0; f < kFills; f++) {
+    const bool is_x = f >= kFills / 2;
+    const int block_row = 16 * wave + 128 * (f & 1);
+    const int64_t first = (is_x ? m0 : (int64_t)n0) + block_row;
+    const int64_t limit = is_x ? rows : (int64_t)n;
+    const uint16_t *base = is_x ? x : w;
+    rsrc[f] = make_rsrc((const uint8_t *)base + first * row_bytes, (limit - first) * row_bytes);
+    lds_at[f] = (int)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)(smem) + (is_x ? kTileBytes : 0) +
+                block_row * kRowBytes;
+  }
+  const int nk = k / kBk;
+  // Stage `s` of the k loop into its ring slot; past the last stage an empty descriptor (zeros land in a
+  // slot nothing reads any more) keeps the count of fills in flight the same in every iteration.
+  auto fill = [&](int s) {
+    const int slot = (s % kStages) * kStageBytes;
+    const int voff = src + s * kRowBytes;
+#pragma unroll
+    for (int f = 0; f < kFills; f++) {
+      i32x4 r = rsrc[f];
+      if (s >= nk) r[2] = 0;
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                   :
+                   : "s"(lds_at[f] + slot), "v"(voff), "s"(r)
+                   : "memory");
+    }
+  };
+#pragma unroll
+  for (int s = 0; s < kStages - 1; s++) fill(s);
+
+  // ---- operand reads: A = W rows (the output's columns), B = X rows (the output's rows); fragment
+  // (block of 32 rows, k-step ks): row ln of the block, logical chunk 2 * ks + g.
+  const int wave_m = wave & 3, wave_n = wave >> 2;  // 64-row and 128-column shares of the tile
+  int a_read[4], b_read[2];
+#pragma unroll
+  for (int cb = 0; cb < 4; cb++) a_read[cb] = (wave_n * 128 + cb * 32 + ln) * kRowBytes;
+#pragma unroll
+  for (int rb = 0; rb < 2; rb++) b_read[rb] = kTileBytes + (wave_m * 64 + rb * 32 + ln) * kRowBytes;
+  const int swz = (ln >> 2) & 3;  // every block starts on a multiple of 16 rows
+  int chunk_at[2];
+#pragma unroll
+  for (int ks = 0; ks < 2; ks++) chunk_at[ks] = ((2 * ks + g) ^ swz) << 4;
+
+  f32x16 acc[2][4];
+  const f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+  for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+    for (int cb = 0; cb < 4; cb++) acc[rb][cb] = zero;
+
+  for (int s = 0; s < nk; s++) {
+    // This wave's fills of stage s have landed (two younger stages may still fly); after the barrier so
+    // have every wave's, and every wave is done reading stage s - 1, whose slot stage s + 3 takes.
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kFills * (kStages - 2)) : "memory");
+    __syncthreads();
+    fill(s + kStages - 1);
+    const uint8_t *st = smem + (s % kStages) * kStageBytes;
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++) {
+      u32x4 af[4], bf[2];
+#pragma unroll
+      for (int cb = 0; cb < 4; cb++) af[cb] = *reinterpret_cast<const u32x4 *>(st + a_read[cb] + chunk_at[ks]);
+#pragma unroll
+      for (int rb = 0; rb < 2; rb++) bf[rb] = *reinterpret_cast<const u32x4 *>(st + b_read[rb] + chunk_at[ks]);
+#pragma unroll
+      for (int cb = 0; cb < 4; cb++)
+#pragma unroll
+        for (int rb = 0; rb < 2; rb++) acc[rb][cb] = mma<F16>(af[cb], bf[rb], acc[rb][cb]);
+    }
+  }
+  // The empty fills still in flight write LDS: they land before the workgroup's LDS is given away.
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+  // ---- epilogue.  Accumulator (rb, cb) register i: row m0 + 64 wave_m + 32 rb + ln, column
+  // n0 + 128 wave_n + 32 cb + 8 (i / 4) + 4 g + i % 4.
+  const int col_base = n0 + wave_n * 128 + 4 * g;
+  if (bias != nullptr) {
+#pragma unroll
+    for (int cb = 0; cb < 4; cb++) {
+#pragma unroll
+      for (int q = 0; q < 4; q++) {
+        const int col = col_base + 32 * cb + 8 * q;
+        if (col >= n) continue;
+        float b4[4];
+        load4<F16>(bias + col, b4);
+#pragma unroll
+        for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+          for (int e = 0; e < 4; e++) acc[rb][cb][4 * q + e] += b4[e];
+      }
+    }
+  }
+  const int turned = HD > 0 ? heads * HD : 0;
+  if (HD > 0 && n0 + wave_n * 128 < turned) {
+    // The head size is 64 or 128: a head's halves are whole 32-column blocks of this wave's 128 columns,
+    // the partner of block cb is block cb +- nb, and a head never straddles two waves.
+    constexpr int head_dim = HD > 0 ? HD : 64;
+    constexpr int half = head_dim >> 1, nb = half >> 5;
+#pragma unroll
+    for (int rb = 0; rb < 2; rb++) {
+      const int64_t row = m0 + wave_m * 64 + rb * 32 + ln;
+      const int64_t pos = row % seq;  // gemm.rs:685: the table row of the token's position
+      const uint16_t *cos_row = cos_t + pos * half, *sin_row = sin_t + pos * half;
+#pragma unroll
+      for (int cb = 0; cb < 4; cb++) {
+        constexpr int kBlocks = 4;
+        const int in_head = (cb * 32) & (head_dim - 1);  // the block's first column within its head
+        if (in_head >= half) continue;                   // second halves are turned with their first
+        if (n0 + wave_n * 128 + cb * 32 >= turned) continue;
+        const int pb = (cb + nb) % kBlocks;  // the partner block (a head's halves lie in one wave)
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+          const int at = in_head + 8 * q + 4 * g;  // index into the table row, < half
+          float c4[4], s4[4];
+          if (row < rows) {
+            load4<F16>(cos_row + at, c4);
+            load4<F16>(sin_row + at, s4);
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++) c4[e] = 1.0f, s4[e] = 0.0f;
+          }
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            const float y1 = acc[rb][cb][4 * q + e], y2 = acc[rb][pb][4 * q + e];
+            // gemm.rs:702-705: x cos, then the partner's product joined by one fused multiply-add.
+            const float y1c = y1 * c4[e], y2c = y2 * c4[e];
+            acc[rb][cb][4 * q + e] = __builtin_fmaf(y2, -s4[e], y1c);
+            acc[rb][pb][4 * q + e] = __builtin_fmaf(y1, s4[e], y2c);
+          }
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int rb = 0; rb < 2; rb++) {
+    const int64_t row = m0 + wave_m * 64 + rb * 32 + ln;
+    if (row >= rows) continue;
+    uint16_t *y_row = y + row * (int64_t)n;
+#pragma unroll
+    for (int cb = 0; cb < 4; cb++) {
+#pragma unroll
+      for (int q = 0; q < 4; q++) {
+        const int col = col_base + 32 * cb + 8 * q;
+        if (col >= n) continue;  // n is a multiple of 8: a run of four lies inside or outside
+        u32x2 out;
+        out[0] = pack2<F16>(acc[rb][cb][4 * q], acc[rb][cb][4 * q + 1]);
+        out[1] = pack2<F16>(acc[rb][cb][4 * q + 2], acc[rb][cb][4 * q + 3]);
+        *reinterpret_cast<u32x2 *>(y_row + col) = out;
+      }
+    }
+  }
+}
+#endif  // __HIP_DEVICE_COMPILE__
+
+template <bool F16, int HD>
+__global__ __launch_bounds__(kWaves * 64, 1) void linear_kernel(const uint16_t *__restrict__ x, const uint16_t *__restrict__ w,
+                                                                const uint16_t *__restrict__ bias,
+                                                                const uint16_t *__restrict__ cos_t,
+                                                                const uint16_t *__restrict__ sin_t, uint16_t *__restrict__ y,
+                                                                int64_t rows, int32_t n, int32_t k, int32_t seq, int32_t heads,
+                                                                uint32_t tiles_n, uint32_t tiles, uint32_t per_xcd) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+  linear_body<F16, HD>(smem, x, w, bias, cos_t, sin_t, y, rows, n, k, seq, heads, tiles_n, tiles, per_xcd);
+#endif
+}
+
+template <bool F16, int HD>
+hipError_t launch(const LinearArgs &a, hipStream_t stream) {
+  const int64_t tiles_m = (a.rows + kBm - 1) / kBm, tiles_n = (a.n + kBn - 1) / kBn;
+  const int64_t tiles = tiles_m * tiles_n;
+  if (tiles == 0) return hipSuccess;
+  const int64_t per_xcd = (tiles + kXcds - 1) / kXcds;
+  if (per_xcd * kXcds > 0x7fffffffLL) return hipErrorInvalidConfiguration;
+  auto kernel = linear_kernel<F16, HD>;
+  static std::atomic<uint64_t> configured{0};  // a bit per device ordinal, devices past 63 always ask
+  int device = 0;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) return e;
+  const uint64_t bit = device < 64 ? 1ull << device : 0;
+  if ((configured.load(std::memory_order_acquire) & bit) == 0) {
+    e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
+    if (e != hipSuccess) return e;
+    configured.fetch_or(bit, std::memory_order_release);
+  }
+  hipLaunchKernelGGL(kernel, dim3((uint32_t)(per_xcd * kXcds)), dim3(kWaves * 64), kLds, stream, (const uint16_t *)a.x,
+                     (const uint16_t *)a.w, (const uint16_t *)a.bias, (const uint16_t *)a.cos, (const uint16_t *)a.sin,
+                     (uint16_t *)a.y, a.rows, a.n, a.k, a.seq, a.heads, (uint32_t)tiles_n, (uint32_t)tiles,
+                     (uint32_t)per_xcd);
+  return hipGetLastError();
+}
+
+}  // namespace
+
+bool linear_supports(int64_t n, int64_t k) { return n > 0 && n % 8 == 0 && k >= kBk && k % kBk == 0 && k <= 0x3fffffff; }
+
+bool linear_turns(int32_t head_dim) { return head_dim == 64 || head_dim == 128; }
+
+hipError_t launch_linear(const LinearArgs &a, hipStream_t stream) {
+  if (!linear_supports(a.n, a.k)) return hipErrorInvalidValue;
+  if (a.cos != nullptr && (!linear_turns(a.head_dim) || a.seq <= 0 || (int64_t)a.heads * a.head_dim > a.n))
+    return hipErrorInvalidValue;
+  const int hd = a.cos != nullptr ? a.head_dim : 0;
+  if (a.f16) return hd == 0 ? launch<true, 0>(a, stream) : hd == 64 ? launch<true, 64>(a, stream) : launch<true, 128>(a, stream);
+  return hd == 0 ? launch<false, 0>(a, stream) : hd == 64 ? launch<false, 64>(a, stream) : launch<false, 128>(a, stream);
+}
+
+}  // namespace svodk

@@ -927,6 +927,151 @@ int svodk_add_rms_norm(const svodk_tensor *x, const svodk_tensor *residual, cons
   return norm(false, x, residual, w, nullptr, eps, batch_live, sum, out, hip_stream);
 }
 
+// shape::linear (tk/src/ops/shape.rs:120-139): the gate, a reduced dim, columns in vector runs
+// of 8, rows; then this library's own: the k-columns in whole stages of the kernel's ring.
+static int plan_linear(bool has_target, const int32_t *dtypes, int n_dtypes, const int64_t *x, int rank, int64_t n) {
+  if (int why = gate(has_target, dtypes, n_dtypes)) return why;
+  if (x == nullptr) return SVODK_GRAPH_SYMBOLIC;
+  if (rank < 1) return SVODK_GRAPH_SHAPE;
+  int64_t rows = 1;
+  for (int i = 0; i + 1 < rank; i++) rows *= x[i];
+  if (n % 8 != 0 || rows == 0 || n <= 0) return SVODK_GRAPH_SHAPE;
+  if (!svodk::linear_supports(n, x[rank - 1])) return SVODK_GRAPH_SHAPE;
+  return 0;
+}
+
+int svodk_plan_linear(int32_t has_target, const int32_t *dtypes, int32_t n_dtypes, const int64_t *x_dims, int32_t x_rank,
+                      int64_t n) {
+  return plan_linear(has_target != 0, dtypes, n_dtypes, x_dims, x_rank, n);
+}
+
+// linear (tk/src/ops/linear.rs:60-231).
+int svodk_linear(const svodk_tensor *x, const svodk_tensor *w, const svodk_linear_opts *opts, const svodk_tensor *out,
+                 void *hip_stream) {
+  const char *op = "linear";
+  if (!well_formed(x) || !well_formed(w) || !well_formed(out) || opts == nullptr)
+    return fail(SVODK_ERR_ARGUMENT, "%s: a null or malformed tensor descriptor", op);
+  // L66-68: x is [..., K], w is [N, K] of x's type.
+  if (x->rank < 1) return fail(SVODK_ERR_SHAPE, "%s: x has shape %s, expected [..., K]", op, fmt_shape(x).c_str());
+  const int64_t k = x->shape[x->rank - 1];
+  if (!(w->rank == 2 && w->shape[1] == k))
+    return fail(SVODK_ERR_SHAPE, "%s: w has shape %s, expected [N, %lld]", op, fmt_shape(w).c_str(), (long long)k);
+  if (w->dtype != x->dtype)
+    return fail(SVODK_ERR_DTYPE, "%s: w is %s, the input is %s", op, dtype_name(w->dtype), dtype_name(x->dtype));
+  // L69-73: a gated weight holds gate rows over up rows.
+  int64_t n = w->shape[0];
+  if (opts->gated) {
+    if (n % 2 != 0) return fail(SVODK_ERR_SHAPE, "%s: w has shape %s, expected [2N, %lld]", op, fmt_shape(w).c_str(), (long long)k);
+    n /= 2;
+  }
+  // L74-77: the bias is [rows of w].
+  if (opts->bias != nullptr) {
+    if (!well_formed(opts->bias)) return fail(SVODK_ERR_ARGUMENT, "%s: bias descriptor malformed", op);
+    if (!(opts->bias->rank == 1 && opts->bias->shape[0] == w->shape[0]))
+      return fail(SVODK_ERR_SHAPE, "%s: bias has shape %s, expected [%lld]", op, fmt_shape(opts->bias).c_str(),
+                  (long long)w->shape[0]);
+  }
+  // The output the reference op allocates itself (L203-206): [lead..., N] of x's type.
+  bool out_fits = out->rank == x->rank && out->shape[out->rank - 1] == n;
+  for (int i = 0; out_fits && i + 1 < x->rank; i++) out_fits = out->shape[i] == x->shape[i];
+  // L79-82: the residual has the output's shape.
+  if (opts->residual != nullptr) {
+    if (!well_formed(opts->residual)) return fail(SVODK_ERR_ARGUMENT, "%s: residual descriptor malformed", op);
+    bool fits = opts->residual->rank == x->rank && opts->residual->shape[x->rank - 1] == n;
+    for (int i = 0; fits && i + 1 < x->rank; i++) fits = opts->residual->shape[i] == x->shape[i];
+    if (!fits) return fail(SVODK_ERR_SHAPE, "%s: residual has shape %s, expected [lead..., %lld]", op,
+                           fmt_shape(opts->residual).c_str(), (long long)n);
+  }
+  // L83-93: a rope wants x [B, T, K] under a plain weight, whole even heads inside N, tables [1, T, 1, d/2].
+  const svodk_rotary *rope = opts->rope;
+  if (rope != nullptr) {
+    if (!(x->rank == 3 && !opts->gated))
+      return fail(SVODK_ERR_SHAPE, "%s: x has shape %s, expected [B, T, K] under a plain weight", op, fmt_shape(x).c_str());
+    const bool fits = rope->head_dim > 0 && rope->head_dim % 2 == 0 && rope->heads >= 0 &&
+                      (int64_t)rope->heads * rope->head_dim <= n;
+    if (!fits)
+      return fail(SVODK_ERR_SHAPE, "%s: w has shape %s, expected [>= %d\xc2\xb7%d, %lld] of even heads", op,
+                  fmt_shape(w).c_str(), rope->heads, rope->head_dim, (long long)k);
+    const svodk_tensor *tables[2] = {rope->cos, rope->sin};
+    const char *names[2] = {"cos", "sin"};
+    for (int i = 0; i < 2; i++) {
+      if (!well_formed(tables[i])) return fail(SVODK_ERR_ARGUMENT, "%s: %s descriptor malformed", op, names[i]);
+      const svodk_tensor *tb = tables[i];
+      if (!(tb->rank == 4 && tb->shape[0] == 1 && tb->shape[1] == x->shape[1] && tb->shape[2] == 1 &&
+            tb->shape[3] == rope->head_dim / 2))
+        return fail(SVODK_ERR_SHAPE, "%s: %s has shape %s, expected [1, %lld, 1, %d]", op, names[i], fmt_shape(tb).c_str(),
+                    (long long)x->shape[1], rope->head_dim / 2);
+    }
+  }
+  if (!out_fits)
+    return fail(SVODK_ERR_SHAPE, "%s: out has shape %s, expected [lead..., %lld]", op, fmt_shape(out).c_str(), (long long)n);
+  if (out->dtype != x->dtype)
+    return fail(SVODK_ERR_DTYPE, "%s: out is %s, the input is %s", op, dtype_name(out->dtype), dtype_name(x->dtype));
+  const int64_t cap = x->shape[0];
+  if (opts->batch_live > cap)
+    return fail(SVODK_ERR_SHAPE, "%s: live batch %d exceeds the capacity %lld", op, opts->batch_live, (long long)cap);
+
+  // L107-127: the plan over every operand's type.
+  int32_t dtypes[4];
+  int nd = 0;
+  dtypes[nd++] = x->dtype;
+  dtypes[nd++] = w->dtype;
+  if (opts->bias) dtypes[nd++] = opts->bias->dtype;
+  if (opts->residual) dtypes[nd++] = opts->residual->dtype;
+  const int why = plan_linear(current_device_has_kernels(), dtypes, nd, x->shape, x->rank, n);
+  if (why != 0) return ran_graph(op, why);
+  // The parts of the reference's GEMM family this library has no kernel for keep the graph; so does a
+  // turn beside an activation, a residual or a scale (L135-141: the graph rotates before them).
+  if (opts->act != SVODK_ACT_NONE || opts->gated || opts->residual != nullptr || opts->has_scale)
+    return ran_graph(op, SVODK_GRAPH_CONFIG);
+  if (rope != nullptr) {
+    // L142-143: tables off the stream dtype leave the turn to the graph.
+    if (rope->cos->dtype != x->dtype || rope->sin->dtype != x->dtype) return ran_graph(op, SVODK_GRAPH_DTYPE);
+    // L176-184: no tile turns heads of this size.
+    if (!svodk::linear_turns(rope->head_dim)) return ran_graph(op, SVODK_GRAPH_CONFIG);
+  }
+  int64_t lead = 1;
+  for (int i = 1; i + 1 < x->rank; i++) lead *= x->shape[i];
+  const int64_t live = x->rank > 1 ? (opts->batch_live > 0 ? opts->batch_live : cap) : 1;
+  const int64_t rows = x->rank > 1 ? live * lead : 1;
+  if (n > 0x7fffffff || (rope && x->shape[1] > 0x7fffffff)) return ran_graph(op, SVODK_GRAPH_SHAPE);
+
+  const size_t table_bytes = rope ? (size_t)numel(rope->cos) * 2 : 0;
+  Span spans[6] = {{"x", x->data, (size_t)numel(x) * 2, false},
+                   {"w", w->data, (size_t)numel(w) * 2, false},
+                   {"bias", opts->bias ? opts->bias->data : nullptr, opts->bias ? (size_t)numel(opts->bias) * 2 : 0, false},
+                   {"cos", rope ? rope->cos->data : nullptr, table_bytes, false},
+                   {"sin", rope ? rope->sin->data : nullptr, table_bytes, false},
+                   {"out", out->data, (size_t)numel(out) * 2, true}};
+  if (x->data == nullptr || w->data == nullptr || out->data == nullptr || (opts->bias && opts->bias->data == nullptr) ||
+      (rope && (rope->cos->data == nullptr || rope->sin->data == nullptr)))
+    return fail(SVODK_ERR_ARGUMENT, "%s: a null device pointer", op);
+  for (const Span &sp : spans)
+    if (sp.data != nullptr && ((uintptr_t)sp.data & 15u) != 0)
+      return fail(SVODK_ERR_ARGUMENT, "%s: %s is not 16-byte aligned", op, sp.name);
+  if (int rc = check_aliasing(op, spans, 6)) return rc;
+
+  svodk::LinearArgs a{};
+  a.x = x->data;
+  a.w = w->data;
+  a.bias = opts->bias ? opts->bias->data : nullptr;
+  a.cos = rope ? rope->cos->data : nullptr;
+  a.sin = rope ? rope->sin->data : nullptr;
+  a.y = out->data;
+  a.rows = rows;
+  a.n = (int32_t)n;
+  a.k = (int32_t)k;
+  a.seq = rope ? (int32_t)x->shape[1] : 1;
+  a.heads = rope ? rope->heads : 0;
+  a.head_dim = rope ? rope->head_dim : 0;
+  a.f16 = x->dtype == SVODK_F16;
+  ran(op, "gemm", rope ? "GemmCfg { bm: 256, bn: 256, bk: 32, stages: 4, warps: [4, 2], epilogue: { bias, rope } }"
+                       : "GemmCfg { bm: 256, bn: 256, bk: 32, stages: 4, warps: [4, 2], epilogue: { bias } }");
+  const hipError_t e = svodk::launch_linear(a, (hipStream_t)hip_stream);
+  if (e != hipSuccess) return fail(SVODK_ERR_LAUNCH, "%s: %s", op, hipGetErrorString(e));
+  return SVODK_KERNEL;
+}
+
 int svodk_plan_norm(int32_t has_target, const int32_t *dtypes, int32_t n_dtypes, const int64_t *x_dims, int32_t x_rank) {
   return plan_norm(has_target != 0, dtypes, n_dtypes, x_dims, x_rank);
 }

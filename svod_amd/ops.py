@@ -59,6 +59,17 @@ class _Qkv(ctypes.Structure):
     ]
 
 
+class _Rotary(ctypes.Structure):
+    _fields_ = [("cos", ctypes.POINTER(_Tensor)), ("sin", ctypes.POINTER(_Tensor)), ("heads", ctypes.c_int32),
+                ("head_dim", ctypes.c_int32)]
+
+
+class _Linear(ctypes.Structure):
+    _fields_ = [("bias", ctypes.POINTER(_Tensor)), ("act", ctypes.c_int32), ("gated", ctypes.c_int32),
+                ("residual", ctypes.POINTER(_Tensor)), ("has_scale", ctypes.c_int32), ("scale", ctypes.c_float),
+                ("rope", ctypes.POINTER(_Rotary)), ("batch_live", ctypes.c_int32)]
+
+
 _lib: Optional[ctypes.CDLL] = None
 
 # Fill the outputs and workspaces this module allocates with NaN bit patterns before the call, so that
@@ -115,6 +126,10 @@ def load_library(path: Optional[str] = None) -> ctypes.CDLL:
         fn.argtypes = [tp] * n_tensors_before_eps + [ctypes.c_double, ctypes.c_int32] + [tp] * n_outputs + [ctypes.c_void_p]
     lib.svodk_plan_norm.restype = ctypes.c_int
     lib.svodk_plan_norm.argtypes = [ctypes.c_int32, i32p, ctypes.c_int32, i64p, ctypes.c_int32]
+    lib.svodk_linear.restype = ctypes.c_int
+    lib.svodk_linear.argtypes = [tp, tp, ctypes.POINTER(_Linear), tp, ctypes.c_void_p]
+    lib.svodk_plan_linear.restype = ctypes.c_int
+    lib.svodk_plan_linear.argtypes = [ctypes.c_int32, i32p, ctypes.c_int32, i64p, ctypes.c_int32, ctypes.c_int64]
     lib.svodk_order_rows.restype = ctypes.c_int
     lib.svodk_order_rows.argtypes = [tp, tp, ctypes.c_void_p]
     lib.svodk_tune_streaming.restype = None
@@ -399,6 +414,72 @@ def heads(qkv: torch.Tensor, opts: Qkv, out: Optional[Tuple[torch.Tensor, torch.
                              ctypes.c_void_p(_stream(qkv)))
     _finish("heads", status)
     return out
+
+
+class Act(enum.IntEnum):
+    """``Act`` of tk/src/ops/mod.rs."""
+
+    NONE = 0
+    Gelu = 1
+    Silu = 2
+
+
+@dataclass
+class Rotary:
+    """``Rotary`` of tk/src/ops/linear.rs:47-58: tables ``[1, T, 1, head_dim/2]``."""
+
+    cos: torch.Tensor
+    sin: torch.Tensor
+    heads: int
+    head_dim: int
+
+
+@dataclass
+class Linear:
+    """``Linear`` of tk/src/ops/linear.rs:24-45 (without ``into``: the caller's ``out`` stands for it)."""
+
+    bias: Optional[torch.Tensor] = None
+    act: Act = Act.NONE
+    gated: bool = False
+    residual: Optional[torch.Tensor] = None
+    scale: Optional[float] = None
+    rope: Optional[Rotary] = None
+    batch_live: Optional[int] = None
+
+
+def linear(x: torch.Tensor, w: torch.Tensor, opts: Optional[Linear] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``x [lead..., K] · w [N, K]ᵀ (+ bias)`` → ``[lead..., N]``, a fused projection's first heads rotated in the
+    GEMM's store (tk/src/ops/linear.rs:60-63)."""
+    opts = opts or Linear()
+    lib = load_library()
+    if out is None:
+        n = w.shape[0] // 2 if opts.gated else w.shape[0]
+        out = _fresh((*x.shape[:-1], n), x.dtype, x.device)
+    keep: list = []
+    o = _Linear()
+    o.bias, o.residual = _ref(keep, opts.bias), _ref(keep, opts.residual)
+    o.act, o.gated = int(opts.act), int(opts.gated)
+    if opts.scale is not None:
+        o.has_scale, o.scale = 1, float(opts.scale)
+    if opts.rope is not None:
+        r = _Rotary()
+        r.cos, r.sin = _ref(keep, opts.rope.cos), _ref(keep, opts.rope.sin)
+        r.heads, r.head_dim = int(opts.rope.heads), int(opts.rope.head_dim)
+        keep.append(r)
+        o.rope = ctypes.pointer(r)
+    o.batch_live = opts.batch_live or 0
+    xd, wd, od = _desc(x), _desc(w), _desc(out)
+    status = lib.svodk_linear(ctypes.byref(xd), ctypes.byref(wd), ctypes.byref(o), ctypes.byref(od), ctypes.c_void_p(_stream(x)))
+    _finish("linear", status)
+    return out
+
+
+def plan_linear(has_target: bool, dtypes, x_dims, n: int) -> Optional[Fallback]:
+    """``shape::linear`` (tk/src/ops/shape.rs:120-139) as a pure function."""
+    lib = load_library()
+    dt = (ctypes.c_int32 * len(dtypes))(*[_DTYPES[d] for d in dtypes])
+    xd = None if x_dims is None else (ctypes.c_int64 * len(x_dims))(*x_dims)
+    return _plan(lib.svodk_plan_linear(int(has_target), dt, len(dtypes), xd, 0 if x_dims is None else len(x_dims), n))
 
 
 def _norm(name: str, x, residual, w, b, eps, batch_live, out):

@@ -570,3 +570,67 @@ def test_norm_closed_forms():
     assert max_abs(y2, oracle.norm_direct(oracle.LAYER, x, ones, eps=0.0)[0]) < 1e-12
     z = oracle.norm_direct(oracle.RMS, x, ones, eps=0.0)[0]
     assert np.abs((z * z).mean(-1) - 1.0).max() < 1e-12
+
+
+# ---- linear with the rope epilogue (tk/src/ops/linear.rs:303-347, tk/src/kernels/gemm.rs:604-716)
+def linear_case(b, t, k, h, hkv, d, seed=40):
+    """``rand`` of the reference's turned-linear test (tk/src/test/unit/ops.rs:301-309): x ~ 1.0, w ~ 0.3, a bias."""
+    g = Lcg(seed)
+    n = (h + 2 * hkv) * d
+    return g.bf16((b, t, k)), g.bf16((n, k), mul=0.3), g.bf16((n,)), n
+
+
+def bf16_tables(t, d, theta=10_000.0):
+    cos, sin = oracle.rope_table(theta, t, d)
+    return oracle.round_bf16(cos), oracle.round_bf16(sin)
+
+
+@pytest.mark.parametrize("b,t,h,hkv,d,bias", [(2, 37, 4, 2, 64, False), (1, 100, 12, 12, 64, True), (3, 16, 2, 1, 128, False)])
+def test_turned_linear_matches_numpy_float64(b, t, h, hkv, d, bias):
+    """An independent evaluation: a float64 matmul, and the turn as the complex product (y1 + i y2)(cos + i sin)
+    over a head's halves (the reference's own cases, tk/src/test/unit/ops.rs:296-299)."""
+    x, w, bv, n = linear_case(b, t, 128, h, hkv, d)
+    cos, sin = bf16_tables(t, d)
+    turned = h + hkv
+    got = oracle.linear_direct(x, w, bv if bias else None, (cos, sin, turned, d))
+    y = x.astype(np.float64) @ w.astype(np.float64).T + (bv.astype(np.float64) if bias else 0.0)
+    z = y[:, :, :turned * d].reshape(b, t, turned, d)
+    zc = (z[..., :d // 2] + 1j * z[..., d // 2:]) * (cos.astype(np.float64) + 1j * sin.astype(np.float64))[None, :, None, :]
+    want = y.copy()
+    want[:, :, :turned * d] = np.concatenate([zc.real, zc.imag], -1).reshape(b, t, turned * d)
+    assert max_abs(got, want) < 1e-12
+
+
+def test_turned_linear_closed_forms():
+    b, t, h, hkv, d = 2, 19, 2, 1, 64
+    x, w, bv, n = linear_case(b, t, 64, h, hkv, d, seed=43)
+    plain = oracle.linear_direct(x, w, bv)
+    assert max_abs(plain, x.astype(np.float64) @ w.astype(np.float64).T + bv) < 1e-12
+    # Zero angles (cos 1, sin 0) leave the product as it is.
+    still = oracle.linear_direct(x, w, bv, (np.ones((t, d // 2), np.float32), np.zeros((t, d // 2), np.float32), h + hkv, d))
+    assert np.array_equal(still, plain)
+    # A turn by unrounded tables keeps each pair's norm, and the columns past the turned heads are the plain product.
+    cos, sin = oracle.rope_table(10_000.0, t, d)
+    c64 = np.cos(np.arccos(np.clip(cos.astype(np.float64), -1, 1)))
+    s64 = np.sqrt(np.maximum(0.0, 1.0 - c64 * c64)) * np.sign(sin)
+    got = oracle.linear_direct(x, w, bv, (c64.astype(np.float32), s64.astype(np.float32), h + hkv, d))
+    turned = (h + hkv) * d
+    pairs = lambda y: (y[:, :, :turned].reshape(b, t, h + hkv, 2, d // 2) ** 2).sum(3)
+    assert np.abs(pairs(got) - pairs(plain)).max() < 1e-5 * np.abs(pairs(plain)).max()
+    assert np.array_equal(got[:, :, turned:], plain[:, :, turned:])
+    # A quarter turn swaps the halves: y1' = -y2, y2' = y1.
+    quarter = oracle.linear_direct(x, w, bv, (np.zeros((t, d // 2), np.float32), np.ones((t, d // 2), np.float32), h + hkv, d))
+    z, q = plain[:, :, :turned].reshape(b, t, h + hkv, 2, d // 2), quarter[:, :, :turned].reshape(b, t, h + hkv, 2, d // 2)
+    assert np.array_equal(q[:, :, :, 0], -z[:, :, :, 1]) and np.array_equal(q[:, :, :, 1], z[:, :, :, 0])
+
+
+@pytest.mark.parametrize("b,t,h,hkv,d,bias", [(2, 37, 4, 2, 64, False), (1, 100, 12, 12, 64, True), (3, 16, 2, 1, 128, False)])
+def test_the_kernels_linear_arithmetic_is_within_the_references_tolerance(b, t, h, hkv, d, bias):
+    """tk/src/test/unit/ops.rs:312: rel 2e-2 against the unrounded reference."""
+    x, w, bv, n = linear_case(b, t, 128, h, hkv, d)
+    cos, sin = bf16_tables(t, d)
+    rope = (cos, sin, h + hkv, d)
+    got = oracle.linear_kernel(x, w, bv if bias else None, rope)
+    want = oracle.linear_direct(x, w, bv if bias else None, rope)
+    assert np.all(np.abs(got - want) <= 2e-2 * np.maximum(np.abs(want), 1.0))
+    assert np.array_equal(got, oracle.round_bf16(got))

@@ -10,7 +10,10 @@
  * allocates no device memory: the caller owns every buffer.
  *
  * All pointers in tensor descriptors are DEVICE pointers (dense, row-major,
- * in the layouts the reference op takes).  Launches are enqueued on the HIP
+ * in the layouts the reference op takes), 16-byte aligned for the 16-bit tensors
+ * and the workspace (the kernels move them in 128-bit pieces) and aligned to
+ * their element for integers and masks; an address off that answers
+ * SVODK_ERR_ARGUMENT.  Launches are enqueued on the HIP
  * stream given and return without synchronising.
  */
 #ifndef SVODK_H
@@ -133,9 +136,12 @@ typedef struct svodk_attn {
   void *workspace; /* device scratch for key splits, or NULL */
   int64_t workspace_bytes;
   /* [B] I32 or NULL, no counterpart in the reference's Attn: the order in which the launch takes
-   * the batch rows (place p works on row row_order[p]; a permutation of 0..B-1, out-of-range
-   * entries are clamped).  Results do not depend on it.  svodk_order_rows fills one from the key
-   * lengths; a model computes it once per batch and passes it to every layer's call. */
+   * the batch rows (place p works on row row_order[p]).  It must be a permutation of 0..B-1: its
+   * contents are device data that no host check reads, so an order that names a row twice computes
+   * that row twice and leaves the rows it skips UNWRITTEN (entries out of range are clamped into the
+   * batch, never followed out of the tensors).  With a permutation results do not depend on it.
+   * svodk_order_rows fills one from the key lengths (always a permutation); a model computes it once
+   * per batch and passes it to every layer's call. */
   const svodk_tensor *row_order;
 } svodk_attn;
 

@@ -1614,8 +1614,8 @@ hipError_t launch(const AttnArgs &a, hipStream_t stream) {
   const int smem = TL::kLds + (a.key_mask != nullptr ? kMaskLds : 0);
   const int64_t q_row = a.q_row_elems > 0 ? a.q_row_elems : (int64_t)a.heads * a.d;
   const int64_t kv_row = a.kv_row_elems > 0 ? a.kv_row_elems : (int64_t)a.kv_heads * a.d;
-  // The fills address a (batch, kv head)'s rows with 32-bit byte offsets.
-  if ((int64_t)a.tk * kv_row * 2 > 0x7fffffffLL || q_row > 0x7fffffffLL) return hipErrorInvalidValue;
+  // A fill addresses the rows of one key block with 32-bit byte offsets from the block's 64-bit base.
+  if (kv_row * 2 * kBkv > 0x7fffffffLL || q_row > 0x7fffffffLL) return hipErrorInvalidValue;
   auto kernel = flash_fwd_kernel<D, NW, CAUSAL, SPLIT, RANGED, BIASED, CACHED, GROUPED, F16>;
   // The LDS ring is above the default limit of a launch: one attribute call per instantiation
   // and device, from whichever thread gets there first (a second call is harmless).
@@ -1858,7 +1858,7 @@ hipError_t launch_attention(const AttnArgs &a, hipStream_t stream) {
 // memory), then the scalars batch, t, tk, heads, kv_heads, scale_bits.  Launch: workgroups
 // [ceil(batch * kv_heads, 8) * (heads / kv_heads) * ceil(t / 128), 1, 1] of [256, 1, 1] threads.
 // The host side's checks are the caller's: heads a multiple of kv_heads, heads < 65536, dimensions
-// positive, tk * kv_heads * D * 2 < 2^31.
+// positive, 64 rows of k or v within 2^31 bytes (kv_heads * D < 2^24).
 // ---------------------------------------------------------------------------------------------
 #if defined(__HIP_DEVICE_COMPILE__)
 // floor(2^32 / d) for div_by, or one less where d divides 2^32 (the estimate stays within one).

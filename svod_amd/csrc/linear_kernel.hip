@@ -177,25 +177,36 @@ __device__ __forceinline__ void linear_body(uint8_t *smem, const uint16_t *__res
 #pragma unroll
     for (int cb = 0; cb < 4; cb++) acc[rb][cb] = zero;
 
+  // Fragments of (stage slot, k-step): four of W (this wave's column blocks), two of X (its row blocks).
+  auto fragments = [&](int slot, int ks, u32x4 (&af)[4], u32x4 (&bf)[2]) {
+    const uint8_t *st = smem + slot * kStageBytes;
+#pragma unroll
+    for (int cb = 0; cb < 4; cb++) af[cb] = *reinterpret_cast<const u32x4 *>(st + a_read[cb] + chunk_at[ks]);
+#pragma unroll
+    for (int rb = 0; rb < 2; rb++) bf[rb] = *reinterpret_cast<const u32x4 *>(st + b_read[rb] + chunk_at[ks]);
+  };
+  auto multiply = [&](const u32x4 (&af)[4], const u32x4 (&bf)[2]) {
+#pragma unroll
+    for (int cb = 0; cb < 4; cb++)
+#pragma unroll
+      for (int rb = 0; rb < 2; rb++) acc[rb][cb] = mma<F16>(af[cb], bf[rb], acc[rb][cb]);
+  };
+  // The loop runs one stage behind its barrier: iteration s first makes sure stage s + 1 has landed for
+  // every wave (and that every wave is done with stage s - 1, whose slot stage s + 3 then takes), so the
+  // first fragments of stage s + 1 can be asked for under the last products of stage s and no product
+  // waits on LDS behind a barrier.
+  u32x4 a0[4], b0[2], a1[4], b1[2];
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kFills * (kStages - 2)) : "memory");  // stage 0 is in
+  __syncthreads();
+  fragments(0, 0, a0, b0);
   for (int s = 0; s < nk; s++) {
-    // This wave's fills of stage s have landed (two younger stages may still fly); after the barrier so
-    // have every wave's, and every wave is done reading stage s - 1, whose slot stage s + 3 takes.
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kFills * (kStages - 2)) : "memory");
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kFills * (kStages - 3)) : "memory");  // stage s + 1 is in
     __syncthreads();
     fill(s + kStages - 1);
-    const uint8_t *st = smem + (s % kStages) * kStageBytes;
-#pragma unroll
-    for (int ks = 0; ks < 2; ks++) {
-      u32x4 af[4], bf[2];
-#pragma unroll
-      for (int cb = 0; cb < 4; cb++) af[cb] = *reinterpret_cast<const u32x4 *>(st + a_read[cb] + chunk_at[ks]);
-#pragma unroll
-      for (int rb = 0; rb < 2; rb++) bf[rb] = *reinterpret_cast<const u32x4 *>(st + b_read[rb] + chunk_at[ks]);
-#pragma unroll
-      for (int cb = 0; cb < 4; cb++)
-#pragma unroll
-        for (int rb = 0; rb < 2; rb++) acc[rb][cb] = mma<F16>(af[cb], bf[rb], acc[rb][cb]);
-    }
+    fragments(s % kStages, 1, a1, b1);
+    multiply(a0, b0);
+    fragments((s + 1) % kStages, 0, a0, b0);
+    multiply(a1, b1);
   }
   // The empty fills still in flight write LDS: they land before the workgroup's LDS is given away.
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");

@@ -112,6 +112,21 @@ bool same_shape(const svodk_tensor *a, const svodk_tensor *b) {
 
 bool is_int(int32_t d) { return d == SVODK_I32 || d == SVODK_I64; }
 
+// What the kernels assume of a device address: 16-bit tensors are read and written in 128-bit pieces
+// (and filled into LDS 16 bytes a lane), integers and masks at their element's size.
+size_t alignment_of(const svodk_tensor *t) {
+  return (t->dtype == SVODK_BF16 || t->dtype == SVODK_F16) ? 16 : dtype_bytes(t->dtype);
+}
+
+// The first of `tensors` (nulls skipped) whose address is off its alignment, or -1.
+int misaligned(const svodk_tensor *const *tensors, int n) {
+  for (int i = 0; i < n; i++) {
+    const svodk_tensor *t = tensors[i];
+    if (t != nullptr && t->data != nullptr && ((uintptr_t)t->data & (alignment_of(t) - 1)) != 0) return i;
+  }
+  return -1;
+}
+
 // launch::aliasing (tk/src/launch.rs:227-246): no parameter the kernel writes
 // shares memory with another.  Here a parameter is a byte range.
 struct Span {
@@ -441,11 +456,11 @@ static int attend(const svodk_tensor *q, const svodk_tensor *k, const svodk_tens
   if (t > 0x7fffffff || tk > 0x7fffffff || heads > 0xffff || cap > 0x7fffffff)
     return ran_graph(op, SVODK_GRAPH_SHAPE);
   {
-    // The kernel addresses a (batch, KV head)'s rows with 32-bit byte offsets and counts its
-    // workgroups in 31 bits: shapes past either keep the graph.
+    // A fill addresses the 64 rows of one key block with 32-bit byte offsets from the block's own base
+    // (which is 64-bit), and the launch counts its workgroups in 31 bits: shapes past either keep the graph.
     const int64_t row_elems = packed ? (heads + 2 * kv_heads) * d : k->shape[2] * d;
     const int64_t tiles = (t + 127) / 128 * heads * cap;
-    if (tk * row_elems * 2 > 0x7fffffffLL || row_elems > 0x3fffffff || tiles * 64 > 0x7ffffff0LL)
+    if (row_elems * 2 * 64 > 0x7fffffffLL || tiles * 64 > 0x7ffffff0LL)
       return ran_graph(op, SVODK_GRAPH_SHAPE);
   }
 
@@ -464,6 +479,24 @@ static int attend(const svodk_tensor *q, const svodk_tensor *k, const svodk_tens
       (lens && lens->data == nullptr) || (bools && bools->data == nullptr) ||
       (opts->seg_start && opts->seg_start->data == nullptr) || (opts->bias && opts->bias->data == nullptr))
     return fail(SVODK_ERR_ARGUMENT, "%s: a null device pointer", op);
+  {
+    // 128-bit loads, stores and LDS fills on the 16-bit tensors; a bias row is read element-wise where
+    // it is not 8-byte aligned, so its base needs its element's alignment only.
+    const svodk_tensor *checked[10] = {q, k, v, out, lens, bools, opts->seg_start,
+                                       cache ? cache->row_map : nullptr, cache ? cache->k_app : nullptr,
+                                       cache ? cache->v_app : nullptr};
+    const char *names[10] = {"q", "k", "v", "out", "key lens", "key mask", "seg start", "row map", "appended k", "appended v"};
+    const int bad = misaligned(checked, 10);
+    if (bad >= 0)
+      return fail(SVODK_ERR_ARGUMENT, "%s: %s is not %zu-byte aligned", op, names[bad], alignment_of(checked[bad]));
+    if (opts->bias != nullptr && ((uintptr_t)opts->bias->data & 1u) != 0)
+      return fail(SVODK_ERR_ARGUMENT, "%s: bias is not 2-byte aligned", op);
+    if (cache && cache->app_lens && cache->app_lens->data &&
+        ((uintptr_t)cache->app_lens->data & (dtype_bytes(cache->app_lens->dtype) - 1)) != 0)
+      return fail(SVODK_ERR_ARGUMENT, "%s: appended lens is not aligned to its element", op);
+    if (opts->workspace != nullptr && ((uintptr_t)opts->workspace & 15u) != 0)
+      return fail(SVODK_ERR_ARGUMENT, "%s: the workspace is not 16-byte aligned", op);
+  }
   if (int rc = check_aliasing(op, spans, 6)) return rc;
   if (opts->seg_start != nullptr) {
     const svodk_tensor *seg = opts->seg_start;
@@ -794,6 +827,11 @@ int svodk_heads(const svodk_tensor *qkv, const svodk_qkv *opts, const svodk_tens
       (opts->q_norm && opts->q_norm->data == nullptr) || (opts->k_norm && opts->k_norm->data == nullptr) ||
       (opts->cos && (opts->cos->data == nullptr || opts->sin->data == nullptr)))
     return fail(SVODK_ERR_ARGUMENT, "%s: a null device pointer", op);
+  {
+    const svodk_tensor *checked[8] = {qkv, opts->q_norm, opts->k_norm, opts->cos, opts->sin, q, k, v};
+    const int bad = misaligned(checked, 8);
+    if (bad >= 0) return fail(SVODK_ERR_ARGUMENT, "%s: %s is not 16-byte aligned", op, spans[bad].name);
+  }
   if (int rc = check_aliasing(op, spans, 8)) return rc;
 
   svodk::HeadsArgs a{};
@@ -880,6 +918,11 @@ static int norm(bool layer, const svodk_tensor *x, const svodk_tensor *residual,
   if (x->data == nullptr || w->data == nullptr || out->data == nullptr || (b && b->data == nullptr) ||
       (residual && residual->data == nullptr) || (sum && sum->data == nullptr))
     return fail(SVODK_ERR_ARGUMENT, "%s: a null device pointer", op);
+  {
+    const svodk_tensor *checked[6] = {x, residual, w, b, out, sum};
+    const int bad = misaligned(checked, 6);
+    if (bad >= 0) return fail(SVODK_ERR_ARGUMENT, "%s: %s is not 16-byte aligned", op, spans[bad].name);
+  }
   if (int rc = check_aliasing(op, spans, 6)) return rc;
 
   svodk::NormArgs a{};

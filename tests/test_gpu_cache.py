@@ -169,3 +169,22 @@ def test_a_non_finite_unread_element_never_reaches_the_output(device, splits):
     dirty = call(k2, v2)
     assert np.isfinite(to_np(dirty)).all()
     assert np.array_equal(bits(dirty), bits(clean))
+
+
+def test_a_cache_whose_rows_span_more_than_two_gib(device):
+    """A decoder step over a cache row of 64 KiB a token (512 heads of 64 over every layer) and 40 000 tokens: one
+    (lane, head)'s keys span 2.6 GB, past what 32-bit byte offsets reach; the fills count from each key block's own
+    64-bit base.  Two lanes over two rows, the layer's four heads near the end of the row, key lengths in the far part."""
+    rows, tk, all_heads, h, d, start = 2, 40_000, 512, 4, 64, 500
+    g = torch.Generator(device=device).manual_seed(3)
+    k = torch.randn((rows, tk, all_heads, d), generator=g, device=device, dtype=torch.bfloat16)
+    v = torch.randn((rows, tk, all_heads, d), generator=g, device=device, dtype=torch.bfloat16)
+    q = torch.randn((rows, 1, h, d), generator=g, device=device, dtype=torch.bfloat16)
+    lens = np.array([tk, 33_333])
+    got = svod_amd.attention(q, k, v, Attn(keys=KeyMask.lens(torch.tensor(lens, dtype=torch.int32, device=device)),
+                                           cache=Cache(head_start=start, kv_heads=h)))
+    torch.cuda.synchronize()
+    assert svod_amd.chosen().startswith('Kernel { op: "attention"'), svod_amd.chosen()
+    ks, vs = (to_np(x[:, :, start:start + h].contiguous()) for x in (k, v))
+    want = oracle.attention_direct(oracle.AttnProblem(to_np(q), ks, vs, key_lens=lens))
+    assert max_abs(to_np(got), want) < 2e-2

@@ -67,3 +67,44 @@ def test_a_row_order_is_validated(device):
     out = svod_amd.attention(q, k, k, Attn(row_order=wild))
     torch.cuda.synchronize()
     assert out.shape == q.shape
+
+
+def test_an_order_that_is_no_permutation_leaves_the_rows_it_skips_unwritten(device):
+    """The order's contents are device data no host check reads: the rows an order names are computed as ever, the
+    rows it leaves out stay as the caller's buffer had them (here the harness's NaN fill), and nothing else happens."""
+    g = Lcg(6)
+    q, k, v = (bf16_tensor(x, device) for x in (g.bf16((4, 70, 2, 64)), g.bf16((4, 90, 2, 64)), g.bf16((4, 90, 2, 64))))
+    whole = svod_amd.attention(q, k, v, Attn())
+    twice = torch.tensor([2, 0, 2, 0], dtype=torch.int32, device=device)  # rows 1 and 3 are never named
+    got = svod_amd.attention(q, k, v, Attn(row_order=twice))
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(got[[0, 2]]), bits(whole[[0, 2]]))
+    assert torch.isnan(got[[1, 3]].float()).all()
+
+
+def misaligned_like(t):
+    """The same values at an address one element past a 16-byte boundary (dense, but off the kernels' alignment)."""
+    flat = torch.empty(t.numel() + 8, dtype=t.dtype, device=t.device)
+    view = flat[1:1 + t.numel()].view(t.shape)
+    view.copy_(t)
+    return view
+
+
+def test_addresses_off_the_kernels_alignment_are_refused(device):
+    g = Lcg(8)
+    q, k = bf16_tensor(g.bf16((2, 64, 2, 64)), device), bf16_tensor(g.bf16((2, 64, 2, 64)), device)
+    for args in ((misaligned_like(q), k, k), (q, misaligned_like(k), k), (q, k, misaligned_like(k))):
+        with pytest.raises(svod_amd.OpError) as e:
+            svod_amd.attention(*args, Attn())
+        assert e.value.kind == "Argument" and "aligned" in str(e.value)
+    with pytest.raises(svod_amd.OpError) as e:
+        svod_amd.attention(q, k, k, Attn(), out=misaligned_like(q))
+    assert e.value.kind == "Argument" and "out is not 16-byte aligned" in str(e.value)
+    x = bf16_tensor(g.bf16((2, 8, 512)), device)
+    w = bf16_tensor(g.bf16((512,)), device)
+    with pytest.raises(svod_amd.OpError) as e:
+        svod_amd.rms_norm(misaligned_like(x), w)
+    assert e.value.kind == "Argument" and "aligned" in str(e.value)
+    with pytest.raises(svod_amd.OpError) as e:
+        svod_amd.heads(misaligned_like(x), svod_amd.Qkv(4, 2, 64))
+    assert e.value.kind == "Argument" and "aligned" in str(e.value)

@@ -757,9 +757,8 @@ __device__ __forceinline__ void flash_fwd_body(
     const int32_t *__restrict__ row_order, int32_t t, uint32_t tk_lens64, const uint16_t *__restrict__ q,
     const uint16_t *__restrict__ k, const uint16_t *__restrict__ v, uint16_t *__restrict__ o,
     const void *__restrict__ key_mask, int32_t mask_bytes, float scale, const Splits &sp, int32_t q_row_elems,
-    int32_t kv_row_elems, const Ranges &rg, uint32_t group_rcp) {
+    int32_t kv_row_elems, const Ranges &rg) {
   // Two of the arguments are packed: heads | group << 16, and tk | (key_lens is 64-bit) << 31.
-  // `unit_size` is the span of the launch's order (see below).
   const Geometry geo = {unit_size, unit_rcp, nqt_u, nqt_rcp, kvh_u, kvh_rcp, heads_group >> 16, units};
   const int heads = (int)(heads_group & 0xffffu);
   const int tk = (int)(tk_lens64 & 0x7fffffffu);
@@ -775,32 +774,14 @@ __device__ __forceinline__ void flash_fwd_body(
   // are dealt to the XCDs round-robin too and a unit's workgroups all land on one XCD: they
   // meet in one L2 instead of being spread over all eight.  (The reference's grid is query
   // tile fastest, then head, then batch, attention.rs:512,523; the order within a unit is that.)
-  //
-  // The order of an XCD's workgroups is the order its CUs take them in.  Without a causal mask the
-  // tiles of a unit cost the same and run side by side (span = group * nqt workgroups a unit).  Under
-  // a causal mask a tile's cost falls with its place in the order (longest first, L524-528), and a launch
-  // that ran unit after unit would end on whichever unit came last, long tiles included: there the order
-  // is tile-major, every unit's longest tile, then every unit's next (span = the XCD's units * group
-  // workgroups a place), so that the launch ends on short tiles everywhere.
   const uint32_t wg = __builtin_amdgcn_workgroup_id_x();
   SVODK_TL_STAMPS;
   SVODK_TL(0);
   const uint32_t local = wg / kXcds;
-  uint32_t round, head_in_group;
-  int order;
-  if (CAUSAL) {
-    const uint32_t place = div_by(local, geo.unit_size, geo.unit_rcp);
-    if (place >= geo.nqt) return;
-    const uint32_t rest = local - place * geo.unit_size;
-    round = div_by(rest, geo.group, group_rcp);
-    head_in_group = rest - round * geo.group;
-    order = (int)place;
-  } else {
-    round = div_by(local, geo.unit_size, geo.unit_rcp);
-    const uint32_t within = local - round * geo.unit_size;
-    head_in_group = div_by(within, geo.nqt, geo.nqt_rcp);
-    order = (int)(within - head_in_group * geo.nqt);
-  }
+  const uint32_t round = div_by(local, geo.unit_size, geo.unit_rcp);
+  const uint32_t within = local - round * geo.unit_size;
+  const uint32_t head_in_group = div_by(within, geo.nqt, geo.nqt_rcp);
+  const int order = (int)(within - head_in_group * geo.nqt);
   const uint32_t unit = round * kXcds + wg % kXcds;
   if (unit >= geo.units) return;
   const int b_place = (int)div_by(unit, geo.kv_heads, geo.kvh_rcp);
@@ -1229,7 +1210,7 @@ __global__ __launch_bounds__(NW * 64, (D <= 64 && !BIASED) ? 3 : (D <= 128 ? 2 :
     uint32_t units, uint32_t heads_group, const void *__restrict__ key_lens, const int32_t *__restrict__ row_order,
     int32_t t, uint32_t tk_lens64, const uint16_t *__restrict__ q, const uint16_t *__restrict__ k,
     const uint16_t *__restrict__ v, uint16_t *__restrict__ o, const void *__restrict__ key_mask, int32_t mask_bytes,
-    float scale, Splits sp, int32_t q_row_elems, int32_t kv_row_elems, Ranges rg, uint32_t group_rcp) {
+    float scale, Splits sp, int32_t q_row_elems, int32_t kv_row_elems, Ranges rg) {
 #if defined(__HIP_DEVICE_COMPILE__)
   // The first 14 dwords of the arguments (up to tk_lens64) arrive in registers with the wave
   // (kernarg preload, scalars and pointers only): they are what the workgroup's coordinates,
@@ -1237,7 +1218,7 @@ __global__ __launch_bounds__(NW * 64, (D <= 64 && !BIASED) ? 3 : (D <= 128 ? 2 :
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
   flash_fwd_body<D, NW, CAUSAL, SPLIT, RANGED, BIASED, CACHED, GROUPED, F16>(
       smem, unit_size, unit_rcp, nqt_u, nqt_rcp, kvh_u, kvh_rcp, units, heads_group, key_lens, row_order, t, tk_lens64,
-      q, k, v, o, key_mask, mask_bytes, scale, sp, q_row_elems, kv_row_elems, rg, group_rcp);
+      q, k, v, o, key_mask, mask_bytes, scale, sp, q_row_elems, kv_row_elems, rg);
 #endif
 }
 
@@ -1657,9 +1638,6 @@ hipError_t launch(const AttnArgs &a, hipStream_t stream) {
   }
   const uint32_t heads_group = (uint32_t)a.heads | geo.group << 16;
   const uint32_t tk_lens64 = (uint32_t)a.tk | (a.lens_i64 ? 0x80000000u : 0u);
-  // The span of the kernel's workgroup order: a unit's workgroups, or under a causal mask the
-  // workgroups of one place in the tile order (an XCD's units times the group).
-  const uint32_t span = CAUSAL ? (uint32_t)((units + kXcds - 1) / kXcds) * geo.group : geo.unit_size;
   Splits sp;
   sp.count = (uint32_t)splits;
   sp.rcp = rcp(sp.count);
@@ -1688,11 +1666,11 @@ hipError_t launch(const AttnArgs &a, hipStream_t stream) {
   rg.app_rows = a.app_rows;
   rg.app_lens = a.app_lens;
   rg.app_lens_i64 = a.app_lens_i64;
-  hipLaunchKernelGGL(kernel, dim3((uint32_t)grid), dim3(NW * 64), smem, stream, span, rcp(span), geo.nqt,
+  hipLaunchKernelGGL(kernel, dim3((uint32_t)grid), dim3(NW * 64), smem, stream, geo.unit_size, geo.unit_rcp, geo.nqt,
                      geo.nqt_rcp, geo.kv_heads, geo.kvh_rcp, geo.units, heads_group, a.key_lens,
                      (const int32_t *)a.row_order, a.t, tk_lens64, (const uint16_t *)a.q, (const uint16_t *)a.k,
                      (const uint16_t *)a.v, (uint16_t *)a.o, a.key_mask, a.mask_bytes, a.scale, sp, (int32_t)q_row,
-                     (int32_t)kv_row, rg, rcp(geo.group));
+                     (int32_t)kv_row, rg);
   return hipGetLastError();
 }
 
@@ -1874,7 +1852,7 @@ __device__ __forceinline__ void attention_entry(uint8_t *smem, const uint16_t *q
   const uint32_t group = (uint32_t)heads / (uint32_t)kv_heads;
   const uint32_t nqt = ((uint32_t)t + NW * kWaveRows - 1) / (NW * kWaveRows);
   const uint32_t units = (uint32_t)kv_heads * (uint32_t)batch;
-  const uint32_t span = CAUSAL ? (units + kXcds - 1) / kXcds * group : group * nqt;  // see flash_fwd_body
+  const uint32_t span = group * nqt;  // a unit's workgroups
   const Splits sp = {1u, 0xffffffffu, nullptr, nullptr, nullptr, (uint32_t)batch};
   Ranges rg = {};
   rg.win_left = -1;
@@ -1882,7 +1860,7 @@ __device__ __forceinline__ void attention_entry(uint8_t *smem, const uint16_t *q
   flash_fwd_body<D, NW, CAUSAL, false, false, false, false, false, F16>(
       smem, span, rcp_for(span), nqt, rcp_for(nqt), (uint32_t)kv_heads, rcp_for((uint32_t)kv_heads), units,
       (uint32_t)heads | group << 16, key_lens, nullptr, t, (uint32_t)tk, q, k, v, o, key_mask, 1,
-      __builtin_bit_cast(float, scale_bits), sp, heads * D, kv_heads * D, rg, rcp_for(group));
+      __builtin_bit_cast(float, scale_bits), sp, heads * D, kv_heads * D, rg);
 }
 #endif
 
@@ -1924,7 +1902,7 @@ __device__ __forceinline__ void attention_entry_full(uint8_t *smem, SVODK_FULL_P
   const uint32_t count = SPLIT ? (uint32_t)(splits > 0 ? splits : 1) : 1u;
   const uint32_t nqt = (GROUPED ? 1u : ((uint32_t)t + NW * kWaveRows - 1) / (NW * kWaveRows)) * count;
   const uint32_t units = (uint32_t)kv_heads * (uint32_t)batch;
-  const uint32_t span = CAUSAL ? (units + kXcds - 1) / kXcds * group : (GROUPED ? 1u : group) * nqt;  // see flash_fwd_body
+  const uint32_t span = (GROUPED ? 1u : group) * nqt;
   const Splits sp = {count, rcp_for(count), o_part, m_part, l_part, (uint32_t)batch};
   Ranges rg = {};
   rg.win_left = RANGED ? win_left : -1;
@@ -1950,7 +1928,7 @@ __device__ __forceinline__ void attention_entry_full(uint8_t *smem, SVODK_FULL_P
       smem, span, rcp_for(span), nqt, rcp_for(nqt), (uint32_t)kv_heads, rcp_for((uint32_t)kv_heads), units,
       (uint32_t)heads | group << 16, key_lens, nullptr, t, (uint32_t)tk | (lens_i64 ? 0x80000000u : 0u), q, k, v, o,
       key_mask, mask_bytes, __builtin_bit_cast(float, scale_bits), sp, q_row_elems > 0 ? q_row_elems : heads * D,
-      kv_row_elems > 0 ? kv_row_elems : kv_heads * D, rg, rcp_for(group));
+      kv_row_elems > 0 ? kv_row_elems : kv_heads * D, rg);
 }
 #endif
 

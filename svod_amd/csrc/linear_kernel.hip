@@ -11,7 +11,8 @@
 // owns 64 rows x 128 columns as 2 x 4 accumulators of v_mfma_f32_32x32x16.  The product runs transposed,
 // C^T = W . X^T, so that a lane owns one output ROW and, per accumulator register quad, four CONSECUTIVE
 // columns: the store is 8-byte runs, the rotation's partner column (32 or 64 columns along) is the same
-// lane's register of another accumulator, and the tables are read as 8-byte runs of the lane's row.
+// lane's register of another accumulator, and the tables (staged through LDS once the ring is done with)
+// are read as 8-byte runs of the lane's row.
 // X and W tiles of 32 k-columns stream through a four-stage LDS ring (32 KiB a stage), filled global -> LDS
 // by buffer_load_dwordx4 ... lds three stages ahead; rows are 64 bytes, their four 16-byte chunks
 // XOR-swizzled by (row / 4) % 4 through the lanes' source addresses so that a ds_read_b128 of 16 rows at one
@@ -46,6 +47,7 @@ constexpr int kWaves = 8;               // 4 along the rows x 2 along the column
 constexpr int kBm = 256, kBn = 256;     // the workgroup's output tile
 constexpr int kBk = 32;                 // k-columns a stage
 constexpr int kStages = 4;
+constexpr int kGroup = 8;               // column tiles an XCD's resident workgroups spread over
 constexpr int kRowBytes = kBk * 2;      // a tile row in LDS
 constexpr int kTileBytes = kBm * kRowBytes;           // one operand's tile: 16 KiB
 constexpr int kStageBytes = 2 * kTileBytes;           // W tile, then X tile
@@ -105,17 +107,37 @@ __device__ __forceinline__ void linear_body(uint8_t *smem, const uint16_t *__res
                                             const uint16_t *__restrict__ bias, const uint16_t *__restrict__ cos_t,
                                             const uint16_t *__restrict__ sin_t, uint16_t *__restrict__ y, int64_t rows,
                                             int32_t n, int32_t k, int32_t seq, int32_t heads, uint32_t tiles_n,
-                                            uint32_t tiles, uint32_t per_xcd) {
+                                            uint32_t tiles, uint32_t per_xcd, uint32_t band) {
   const int tid = __builtin_amdgcn_workitem_id_x();
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int g = lane >> 5, ln = lane & 31;
-  // Workgroups are dealt to the 8 XCDs in turn, so XCD x takes a run of consecutive tiles, column tile
-  // fastest: its workgroups share x's row tile and walk w through one L2.
+  // Workgroups are dealt to the 8 XCDs in turn, each XCD with an L2 of its own.  With rows enough
+  // (`band` > 0) XCD x owns a band of `band` row tiles and walks it in groups of up to kGroup column
+  // tiles, row tile by row tile within a group: the workgroups resident together then share few w tiles
+  // (read once per XCD) and few x tiles (read once per group), instead of streaming all of w past every
+  // row tile.  With few rows XCD x takes a run of consecutive tiles, column tile fastest.
   const uint32_t wg = __builtin_amdgcn_workgroup_id_x();
-  const uint32_t tile = (wg % kXcds) * per_xcd + wg / kXcds;
-  if (wg / kXcds >= per_xcd || tile >= tiles) return;
-  const uint32_t tm = tile / tiles_n, tn = tile - tm * tiles_n;
+  const uint32_t xcd = wg % kXcds, local = wg / kXcds;
+  uint32_t tm, tn;
+  if (band > 0) {
+    const uint32_t full = band * kGroup;            // workgroups of a full-width group
+    const uint32_t ng = local / full;               // the group
+    const uint32_t first = ng * kGroup;             // its first column tile
+    if (first >= tiles_n) return;
+    const uint32_t width = min((uint32_t)kGroup, tiles_n - first);
+    const uint32_t r = local - ng * full;
+    const uint32_t tm_local = r / width;
+    if (tm_local >= band) return;
+    tm = xcd * band + tm_local;
+    tn = first + (r - tm_local * width);
+    if ((uint64_t)tm * tiles_n + tn >= tiles) return;  // past the last row tile
+  } else {
+    const uint32_t tile = xcd * per_xcd + local;
+    if (local >= per_xcd || tile >= tiles) return;
+    tm = tile / tiles_n;
+    tn = tile - tm * tiles_n;
+  }
   const int64_t m0 = (int64_t)tm * kBm;
   const int32_t n0 = (int32_t)tn * kBn;
   const int64_t row_bytes = (int64_t)k * 2;
@@ -231,41 +253,59 @@ __device__ __forceinline__ void linear_body(uint8_t *smem, const uint16_t *__res
     }
   }
   const int turned = HD > 0 ? heads * HD : 0;
-  if (HD > 0 && n0 + wave_n * 128 < turned) {
-    // The head size is 64 or 128: a head's halves are whole 32-column blocks of this wave's 128 columns,
-    // the partner of block cb is block cb +- nb, and a head never straddles two waves.
+  if (HD > 0 && n0 < turned) {  // the same for the whole workgroup
+    // The head size is 64 or 128: a head's halves are whole 32-column blocks of a wave's 128 columns, the
+    // partner of block cb is block cb +- nb, and a head never straddles two waves.
     constexpr int head_dim = HD > 0 ? HD : 64;
     constexpr int half = head_dim >> 1, nb = half >> 5;
+    // The tile's 256 rows of the tables go through LDS (the ring is done with): loaded 16 bytes a lane
+    // along the rows, read back 8 bytes a lane down them.  A lane owns a ROW of the output, so reading
+    // the tables straight from memory would touch 32 lines an instruction.  Rows of 2 * half + 8 bytes
+    // keep the reads off each other's banks.
+    constexpr int kPitch = half * 2 + 8, kChunks = half * 2 / 16;
+    uint8_t *cos_lds = smem, *sin_lds = smem + kBm * kPitch;
+    __syncthreads();  // every wave's last fragments are read and its last fills have landed
+    const uint32_t pos0 = (uint32_t)(m0 % seq);
+    for (int c = tid; c < kBm * kChunks; c += kWaves * 64) {
+      const int r = c / kChunks, ch = c % kChunks;
+      const uint32_t pos = (pos0 + (uint32_t)r) % (uint32_t)seq;  // gemm.rs:685: the table row of the token's position
+      const u32x4 vc = *reinterpret_cast<const u32x4 *>(cos_t + (int64_t)pos * half + ch * 8);
+      const u32x4 vs = *reinterpret_cast<const u32x4 *>(sin_t + (int64_t)pos * half + ch * 8);
+      u32x2 *cd = reinterpret_cast<u32x2 *>(cos_lds + r * kPitch + ch * 16);
+      u32x2 *sd = reinterpret_cast<u32x2 *>(sin_lds + r * kPitch + ch * 16);
+      cd[0] = u32x2{vc[0], vc[1]};
+      cd[1] = u32x2{vc[2], vc[3]};
+      sd[0] = u32x2{vs[0], vs[1]};
+      sd[1] = u32x2{vs[2], vs[3]};
+    }
+    __syncthreads();
+    if (n0 + wave_n * 128 < turned) {
 #pragma unroll
-    for (int rb = 0; rb < 2; rb++) {
-      const int64_t row = m0 + wave_m * 64 + rb * 32 + ln;
-      const int64_t pos = row % seq;  // gemm.rs:685: the table row of the token's position
-      const uint16_t *cos_row = cos_t + pos * half, *sin_row = sin_t + pos * half;
+      for (int rb = 0; rb < 2; rb++) {
+        const int r = wave_m * 64 + rb * 32 + ln;
+        const uint16_t *cos_row = reinterpret_cast<const uint16_t *>(cos_lds + r * kPitch);
+        const uint16_t *sin_row = reinterpret_cast<const uint16_t *>(sin_lds + r * kPitch);
 #pragma unroll
-      for (int cb = 0; cb < 4; cb++) {
-        constexpr int kBlocks = 4;
-        const int in_head = (cb * 32) & (head_dim - 1);  // the block's first column within its head
-        if (in_head >= half) continue;                   // second halves are turned with their first
-        if (n0 + wave_n * 128 + cb * 32 >= turned) continue;
-        const int pb = (cb + nb) % kBlocks;  // the partner block (a head's halves lie in one wave)
+        for (int cb = 0; cb < 4; cb++) {
+          constexpr int kBlocks = 4;
+          const int in_head = (cb * 32) & (head_dim - 1);  // the block's first column within its head
+          if (in_head >= half) continue;                   // second halves are turned with their first
+          if (n0 + wave_n * 128 + cb * 32 >= turned) continue;
+          const int pb = (cb + nb) % kBlocks;  // the partner block (a head's halves lie in one wave)
 #pragma unroll
-        for (int q = 0; q < 4; q++) {
-          const int at = in_head + 8 * q + 4 * g;  // index into the table row, < half
-          float c4[4], s4[4];
-          if (row < rows) {
+          for (int q = 0; q < 4; q++) {
+            const int at = in_head + 8 * q + 4 * g;  // index into the table row, < half
+            float c4[4], s4[4];
             load4<F16>(cos_row + at, c4);
             load4<F16>(sin_row + at, s4);
-          } else {
 #pragma unroll
-            for (int e = 0; e < 4; e++) c4[e] = 1.0f, s4[e] = 0.0f;
-          }
-#pragma unroll
-          for (int e = 0; e < 4; e++) {
-            const float y1 = acc[rb][cb][4 * q + e], y2 = acc[rb][pb][4 * q + e];
-            // gemm.rs:702-705: x cos, then the partner's product joined by one fused multiply-add.
-            const float y1c = y1 * c4[e], y2c = y2 * c4[e];
-            acc[rb][cb][4 * q + e] = __builtin_fmaf(y2, -s4[e], y1c);
-            acc[rb][pb][4 * q + e] = __builtin_fmaf(y1, s4[e], y2c);
+            for (int e = 0; e < 4; e++) {
+              const float y1 = acc[rb][cb][4 * q + e], y2 = acc[rb][pb][4 * q + e];
+              // gemm.rs:702-705: x cos, then the partner's product joined by one fused multiply-add.
+              const float y1c = y1 * c4[e], y2c = y2 * c4[e];
+              acc[rb][cb][4 * q + e] = __builtin_fmaf(y2, -s4[e], y1c);
+              acc[rb][pb][4 * q + e] = __builtin_fmaf(y1, s4[e], y2c);
+            }
           }
         }
       }
@@ -298,10 +338,11 @@ __global__ __launch_bounds__(kWaves * 64, 1) void linear_kernel(const uint16_t *
                                                                 const uint16_t *__restrict__ cos_t,
                                                                 const uint16_t *__restrict__ sin_t, uint16_t *__restrict__ y,
                                                                 int64_t rows, int32_t n, int32_t k, int32_t seq, int32_t heads,
-                                                                uint32_t tiles_n, uint32_t tiles, uint32_t per_xcd) {
+                                                                uint32_t tiles_n, uint32_t tiles, uint32_t per_xcd,
+                                                                uint32_t band) {
 #if defined(__HIP_DEVICE_COMPILE__)
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
-  linear_body<F16, HD>(smem, x, w, bias, cos_t, sin_t, y, rows, n, k, seq, heads, tiles_n, tiles, per_xcd);
+  linear_body<F16, HD>(smem, x, w, bias, cos_t, sin_t, y, rows, n, k, seq, heads, tiles_n, tiles, per_xcd, band);
 #endif
 }
 
@@ -310,7 +351,9 @@ hipError_t launch(const LinearArgs &a, hipStream_t stream) {
   const int64_t tiles_m = (a.rows + kBm - 1) / kBm, tiles_n = (a.n + kBn - 1) / kBn;
   const int64_t tiles = tiles_m * tiles_n;
   if (tiles == 0) return hipSuccess;
-  const int64_t per_xcd = (tiles + kXcds - 1) / kXcds;
+  // Bands of row tiles per XCD where every XCD gets at least two row tiles; else runs of tiles.
+  const int64_t band = tiles_m >= 2 * kXcds ? (tiles_m + kXcds - 1) / kXcds : 0;
+  const int64_t per_xcd = band > 0 ? band * tiles_n : (tiles + kXcds - 1) / kXcds;
   if (per_xcd * kXcds > 0x7fffffffLL) return hipErrorInvalidConfiguration;
   auto kernel = linear_kernel<F16, HD>;
   static std::atomic<uint64_t> configured{0};  // a bit per device ordinal, devices past 63 always ask
@@ -326,7 +369,7 @@ hipError_t launch(const LinearArgs &a, hipStream_t stream) {
   hipLaunchKernelGGL(kernel, dim3((uint32_t)(per_xcd * kXcds)), dim3(kWaves * 64), kLds, stream, (const uint16_t *)a.x,
                      (const uint16_t *)a.w, (const uint16_t *)a.bias, (const uint16_t *)a.cos, (const uint16_t *)a.sin,
                      (uint16_t *)a.y, a.rows, a.n, a.k, a.seq, a.heads, (uint32_t)tiles_n, (uint32_t)tiles,
-                     (uint32_t)per_xcd);
+                     (uint32_t)per_xcd, (uint32_t)band);
   return hipGetLastError();
 }
 

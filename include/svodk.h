@@ -306,8 +306,19 @@ int svodk_plan_norm(int32_t has_target, const int32_t *dtypes, int32_t n_dtypes,
  * workgroups that each walk a run of query tiles, the next tile's keys loading under the
  * current tile's last steps.  n > 0 = stream, n workgroups per XCD (96 fills an MI355X);
  * n <= 0 (the default) = a workgroup per tile.  Process-wide.  Results are bit-equal either way.
+ *
+ * A streaming launch hands out its tiles through one of SVODK_STREAMING_SETS sets of counters in
+ * device memory, taken in turn at enqueue time and put back to zero by the launch's last
+ * workgroup: at most SVODK_STREAMING_SETS streaming launches may be in flight at once on a device,
+ * and a launch that dies midway leaves its set dirty for the launch that meets it next.  A call on
+ * a stream that is being captured never streams (a graph's replays would all use the set the
+ * capture took, and overlapping replays would share it): it runs a workgroup per tile.
  */
+#define SVODK_STREAMING_SETS 256
 void svodk_tune_streaming(int32_t workgroups_per_xcd);
+/* The set the next streaming launch would take, and takes it (no device work): for tests of the
+ * assignment.  No counterpart in the reference. */
+uint32_t svodk_streaming_next_set(void);
 
 /*
  * ops::supported (tk/src/ops/mod.rs:164-166): 1 when the current HIP device is

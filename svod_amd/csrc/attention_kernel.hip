@@ -59,6 +59,7 @@ namespace svodk {
 // streaming launches so far: each takes the next set of shared counters.
 extern std::atomic<int> g_stream_slots;
 extern std::atomic<uint32_t> g_queue_turn;
+uint32_t next_queue_set();  // the counter set of the next streaming launch: the sets in turn
 #endif
 namespace {
 
@@ -1576,7 +1577,7 @@ hipError_t launch_stream(const AttnArgs &a, hipStream_t stream, int64_t slots, c
                      geo.nqt, geo.nqt_rcp, geo.kv_heads, geo.kvh_rcp, geo.units, heads_group, a.key_lens,
                      (const uint16_t *)a.q, a.t, tk_lens64, (const uint16_t *)a.k, (const uint16_t *)a.v,
                      (uint16_t *)a.o, a.scale, (int32_t)q_row, (int32_t)kv_row, (uint32_t)slots,
-                     g_queue_turn.fetch_add(1u, std::memory_order_relaxed) % kQueueSets, (const int32_t *)a.row_order);
+                     next_queue_set(), (const int32_t *)a.row_order);
   return hipGetLastError();
 }
 
@@ -1633,8 +1634,16 @@ hipError_t launch(const AttnArgs &a, hipStream_t stream) {
   // It is never chosen unasked: measured, it has not beaten a workgroup per tile.
   if constexpr (D == 64 && !SPLIT && !RANGED && !BIASED && !CACHED && !GROUPED) {
     const int knob = g_stream_slots.load(std::memory_order_relaxed);
-    if (knob > 0 && a.key_mask == nullptr)
-      return launch_stream<D, NW, CAUSAL, F16>(a, stream, knob, geo, q_row, kv_row);
+    if (knob > 0 && a.key_mask == nullptr) {
+      // A captured launch would keep its counter set for every replay, and replays that overlap
+      // (two graphs, one graph on two streams) would then share it: a capturing stream gets a
+      // workgroup per tile, which needs no counters.
+      hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+      e = hipStreamIsCapturing(stream, &capturing);
+      if (e != hipSuccess) return e;
+      if (capturing == hipStreamCaptureStatusNone)
+        return launch_stream<D, NW, CAUSAL, F16>(a, stream, knob, geo, q_row, kv_row);
+    }
   }
   const uint32_t heads_group = (uint32_t)a.heads | geo.group << 16;
   const uint32_t tk_lens64 = (uint32_t)a.tk | (a.lens_i64 ? 0x80000000u : 0u);
@@ -1769,6 +1778,7 @@ hipError_t launch_attention_d256(const AttnArgs &a, hipStream_t stream) { return
 #if SVODK_HAS_COMMON
 std::atomic<int> g_stream_slots{0};
 std::atomic<uint32_t> g_queue_turn{0};
+uint32_t next_queue_set() { return g_queue_turn.fetch_add(1u, std::memory_order_relaxed) % (uint32_t)kQueueSets; }
 
 hipError_t launch_order_rows(const void *keys, int32_t elem_bytes, int32_t n, int32_t tk, int32_t *order,
                              hipStream_t stream) {

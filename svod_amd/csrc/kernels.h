@@ -150,6 +150,8 @@ hipError_t launch_order_rows(const void *keys, int32_t elem_bytes, int32_t n, in
                              hipStream_t stream);
 // Tuning of the streaming form (workgroups that walk runs of query tiles): see svodk_tune_streaming.
 void attention_stream_slots(int32_t slots);
+// The set of shared counters the next streaming launch takes (and takes it): the sets in turn.
+uint32_t next_queue_set();
 // Text of the tile configuration launch_attention picks for `a` (for chosen()).
 const char *attention_config(const AttnArgs &a);
 

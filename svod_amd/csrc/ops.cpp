@@ -693,6 +693,7 @@ int svodk_attention_packed(const svodk_tensor *qkv, int32_t heads, int32_t kv_he
 }
 
 void svodk_tune_streaming(int32_t workgroups_per_xcd) { svodk::attention_stream_slots(workgroups_per_xcd); }
+uint32_t svodk_streaming_next_set(void) { return svodk::next_queue_set(); }
 
 // The batch rows by descending key count, for svodk_attn.row_order (no counterpart in the reference,
 // whose grid fixes what a block computes and leaves the order of blocks to the hardware).

@@ -132,6 +132,8 @@ def load_library(path: Optional[str] = None) -> ctypes.CDLL:
     lib.svodk_plan_linear.argtypes = [ctypes.c_int32, i32p, ctypes.c_int32, i64p, ctypes.c_int32, ctypes.c_int64]
     lib.svodk_order_rows.restype = ctypes.c_int
     lib.svodk_order_rows.argtypes = [tp, tp, ctypes.c_void_p]
+    lib.svodk_streaming_next_set.restype = ctypes.c_uint32
+    lib.svodk_streaming_next_set.argtypes = []
     lib.svodk_tune_streaming.restype = None
     lib.svodk_tune_streaming.argtypes = [ctypes.c_int32]
     lib.svodk_supported.restype = ctypes.c_int

@@ -266,3 +266,13 @@ def test_without_a_device_a_norm_names_the_graph():
         svod_amd.layer_norm(t([4, 512]), t([512]))
     assert e.value.why == Fallback.Target
     assert svod_amd.chosen() == 'Graph { op: "layer_norm", why: Target }'
+
+
+def test_streaming_launches_take_the_counter_sets_in_turn():
+    lib = svod_amd.load_library()
+    sets = int(re.search(r"#define SVODK_STREAMING_SETS (\d+)", open(os.path.join(ROOT, "include", "svodk.h")).read()).group(1))
+    taken = [lib.svodk_streaming_next_set() for _ in range(2 * sets + 1)]
+    assert all(0 <= s < sets for s in taken)
+    assert all((b - a) % sets == 1 for a, b in zip(taken, taken[1:]))  # one after another, round and round
+    assert len(set(taken[:sets])) == sets  # a set is met again only after every other one
+    assert taken[sets] == taken[0] and taken[2 * sets] == taken[0]

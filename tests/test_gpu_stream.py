@@ -127,3 +127,39 @@ def test_streaming_follows_a_row_order(device):
     streamed = svod_amd.attention(q, k, v, Attn(keys=KeyMask.lens(lens), row_order=order))
     torch.cuda.synchronize()
     assert np.array_equal(bits(streamed), plain)
+
+
+def test_a_captured_call_takes_no_counter_set(device):
+    """Under stream capture the knob is not followed: a graph's replays would share the one set of
+    tile counters the capture took.  The captured call runs a workgroup per tile, so it takes no
+    set, and every replay gives the eager result."""
+    lib = svod_amd.load_library()
+    sets = 256
+    q, k, v = (bf16_tensor(x, device) for x in case(4, 384, 384, 8, 2))
+    opts = Attn(causal=True)
+    svod_amd.tune_streaming(-1)
+    plain = svod_amd.attention(q, k, v, opts)
+    svod_amd.tune_streaming(3)
+    before = lib.svodk_streaming_next_set()
+    streamed = svod_amd.attention(q, k, v, opts)  # eager: streams, takes the next set
+    torch.cuda.synchronize()
+    assert (lib.svodk_streaming_next_set() - before) % sets == 2
+    out = torch.empty_like(plain)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        svod_amd.attention(q, k, v, opts, out=out)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    before = lib.svodk_streaming_next_set()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        svod_amd.attention(q, k, v, opts, out=out)
+    assert (lib.svodk_streaming_next_set() - before) % sets == 1  # only this probe took one
+    for _ in range(3):
+        out.fill_(3.0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(bits(out), bits(plain))
+    assert np.array_equal(bits(streamed), bits(plain))

@@ -783,7 +783,12 @@ __device__ __forceinline__ void flash_fwd_body(
   const uint32_t within = local - round * geo.unit_size;
   const uint32_t head_in_group = div_by(within, geo.nqt, geo.nqt_rcp);
   const int order = (int)(within - head_in_group * geo.nqt);
-  const uint32_t unit = round * kXcds + wg % kXcds;
+  // Which unit of a round an XCD takes turns with the round: with a power-of-two head count a
+  // fixed deal would hand an XCD the same heads in every batch row, i.e. always the same 128-byte
+  // residues of every K, V, Q and O row, and the XCD whose residues share a memory channel with
+  // other traffic then runs a tenth behind the rest (measured: whichever XCD read bytes 384..511
+  // of every KiB); turned, every XCD reads every residue and they finish together.
+  const uint32_t unit = round * kXcds + (wg + round) % kXcds;
   if (unit >= geo.units) return;
   const int b_place = (int)div_by(unit, geo.kv_heads, geo.kvh_rcp);
   const int kvh = (int)(unit - (uint32_t)b_place * geo.kv_heads);  // L548: query head h reads KV head h / (heads / kv_heads)

@@ -121,5 +121,6 @@ int main() {
   run<0, 1, true, 1>("registers only + softmax at the D=64 ratio", d, clk, rnd);
   run<2, 2, false>("fragment per 2 MFMAs, no VALU", d, clk, rnd);
   run<2, 2, true>("fragment per 2 MFMAs + softmax      [64-row wave]", d, clk, rnd);
+  run<2, 2, true, 1>("fragment per 2 MFMAs + softmax at the D=64 ratio", d, clk, rnd);
   return 0;
 }

@@ -1,6 +1,6 @@
 """Where and when the workgroups of one attention launch ran.
 
-    python -m svod_amd.probes.timeline [--build] [bge_m3|qwen3_attention|whisper|long] [--no-row-order]
+    python -m svod_amd.probes.timeline [--build] [bge_m3|qwen3_attention|whisper|long] [--no-row-order] [--raw=FILE.npy]
 
 Builds ``bin/libsvodk_timeline.so``, the library with ``-DSVODK_TIMELINE`` (thread 0 of every workgroup of
 ``flash_fwd_kernel`` stamps the 100 MHz clock at entry, first barrier, last computed step, last step and
@@ -82,6 +82,9 @@ def main(argv) -> None:
     point(None)
     t = buf.cpu().numpy().astype(np.uint64).reshape(-1, 8)
     t = t[t[:, 0] != 0]
+    raw = [a.split("=", 1)[1] for a in argv if a.startswith("--raw=")]
+    if raw:
+        np.save(raw[0], t)  # a row a workgroup, in launch order: the five stamps, the hardware id, blocks << 32
     t0 = np.int64(t[:, 0].min())
     start, first, loop_end, idle_end, end = ((t[:, c].astype(np.int64) - t0) * 0.01 for c in range(5))  # us
     hw, xcc = t[:, 5] & 0xffffffff, (t[:, 5] >> 32) & 0xf

@@ -59,7 +59,8 @@ def parse():
                          "none is served from the Infinity Cache")
     ap.add_argument("--no-graph", action="store_true", help="enqueue eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-row-order", action="store_true",
-                    help="bge_m3, bge_m3_bool: take the batch rows as they come instead of ordering them by length once per step")
+                    help="bge_m3, bge_m3_bool, qwen3_attention: take the batch rows as they come instead of ordering them by "
+                         "length once per step")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="rough budget of the CPU baseline sample")
     ap.add_argument("--no-others", action="store_true",
@@ -211,7 +212,13 @@ def build_workload(name, args, dev, row_order=True):
         keys = KeyMask.lens(w.key_lens) if w.key_lens is not None else KeyMask.none()
         ins = [(w.q, w.k, w.v)] + [(w.q.clone(), w.k.clone(), w.v.clone()) for _ in range(3)]
         outs = [torch.empty_like(w.q) for _ in range(4)]
-        opts = Attn(causal=w.causal, keys=keys, scale=w.scale)
+        # Ragged batches are ordered by length once per step, like the bge_m3 rows above (--no-row-order: as given).
+        order = None
+        if row_order and name == "qwen3_attention":
+            order = torch.empty(w.key_lens.shape, dtype=torch.int32, device=dev)
+            wl.extra_calls.append(lambda: svod_amd.order_rows(w.key_lens, out=order))
+            wl.text += ", batch rows ordered by length once per step"
+        opts = Attn(causal=w.causal, keys=keys, scale=w.scale, row_order=order)
         for i in range(args.calls):
             calls.append(lambda i=i: svod_amd.attention(*ins[i % 4], opts, out=outs[i % 4]))
         wl.flops_vis, wl.flops_nom, wl.bytes_min = w.visible_flops(), w.nominal_flops(), w.min_bytes()

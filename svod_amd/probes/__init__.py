@@ -7,6 +7,7 @@ a config (``tk/src/probe.rs``); here the results are evidence for the kernels' d
     python -m svod_amd.probes            build the probes into svod_amd/probes/bin/ and run them (needs a GPU)
     python -m svod_amd.probes --build    build only
     python -m svod_amd.probes.timeline qwen3_attention    (see timeline.py)
+    python -m svod_amd.probes.linear_parts                (see linear_parts.py)
 """
 from __future__ import annotations
 

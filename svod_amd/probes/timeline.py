@@ -7,7 +7,8 @@ Builds ``bin/libsvodk_timeline.so``, the library with ``-DSVODK_TIMELINE`` (thre
 stores landed, and notes its XCD, shader engine and CU), runs one call of a ``bench.py`` workload after
 warm-up and prints: the launch's span against the sum of the workgroups' own times, their phases, the
 time per key block, how many workgroups are resident over time, the gaps between one workgroup's end and
-the next one's start on a CU, and how each XCD deals workgroups to its shader engines.  The stamps cost
+the next one's start on a CU, each XCD's share of the time and its last end, and how each XCD deals
+workgroups to its shader engines.  The stamps cost
 time themselves (a launch takes about a quarter longer): proportions count, not microseconds.
 """
 from __future__ import annotations
@@ -121,6 +122,9 @@ def main(argv) -> None:
     print("gap between a workgroup's end and the next start on its CU:", pct(gaps), " max %.1f;" % gaps.max(),
           "gaps sum to %.0f %% of the slots' time, the ragged end to %.0f %%" %
           (100 * gaps.sum() / (slots * span), 100 * (slots * span - dur.sum() - gaps.sum()) / (slots * span)))
+    print("per XCD: the workgroups' own times sum to", [int(dur[xcc == x].sum()) for x in range(8)], "us; last end",
+          [round(float(end[xcc == x].max()), 1) for x in range(8)])
+    print("per XCD: entry -> first barrier, mean", [round(float((first - start)[xcc == x].mean()), 2) for x in range(8)])
     ends = np.array([end[key == k].max() for k in cus])
     print("a CU's last end: min %.1f  p50 %.1f  max %.1f" % (ends.min(), np.median(ends), ends.max()))
     order = np.argsort(t[:, 0], kind="stable")

@@ -34,6 +34,8 @@ TURNED = [
     ("d 128", (3, 16), (2, 1, 128), False, 128),
     ("an odd count of turned heads of 64", (2, 50), (2, 1, 64), True, 96),
     ("rows and columns across tiles", (2, 300), (4, 2, 128), True, 256),
+    ("a k loop of one stage", (2, 40), (2, 2, 64), True, 32),
+    ("a k loop of two stages, shorter than the ring", (1, 300), (2, 1, 128), False, 64),
 ]
 
 

@@ -46,7 +46,7 @@ static __device__ unsigned long long *g_timeline = nullptr;
 extern "C" int SVODK_TL_CAT(svodk_debug_timeline_h, SVODK_HEAD)(void *buf) {
   return (int)hipMemcpyToSymbol(HIP_SYMBOL(g_timeline), &buf, sizeof(buf));
 }
-#define SVODK_TL_STAMPS unsigned long long tl_stamp[5] = {0, 0, 0, 0, 0}
+#define SVODK_TL_STAMPS unsigned long long tl_stamp[6] = {0, 0, 0, 0, 0, 0}
 #define SVODK_TL(i) asm volatile("s_memrealtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(tl_stamp[i])::"memory")
 #else
 #define SVODK_TL_STAMPS
@@ -805,9 +805,16 @@ __device__ __forceinline__ void flash_fwd_body(
   // when): with an order from the caller, place p of the launch works on row row_order[p], so
   // that rows with more keys can go first and the launch ends on its short tiles.
   int b = b_place;
+  if (row_order != nullptr) b = row_order[b_place];
+  // Everything the first loads and fills take from the argument record (past the words that arrive in
+  // registers with the wave) is asked for HERE, while the row's number is on its way: left to the
+  // compiler those loads sit behind the wait for it, and a workgroup's start is three scalar memory
+  // round trips (the row, the arguments, the length) where two will do.
+  asm volatile("" : "+s"(b) : "s"(q), "s"(k), "s"(v), "s"(o), "s"(key_mask), "s"(mask_bytes), "s"(scale), "s"(q_row_elems),
+               "s"(kv_row_elems));
   if (row_order != nullptr) {
     const int nbatch = (int)div_by(geo.units, geo.kv_heads, geo.kvh_rcp);
-    b = min(max(row_order[b_place], 0), nbatch - 1);
+    b = min(max(b, 0), nbatch - 1);
   }
   // Grid x of the reference is order * splits + split (L523); geo.nqt counts those.
   int split = 0, tile = order, nqt = (int)geo.nqt;
@@ -839,7 +846,6 @@ __device__ __forceinline__ void flash_fwd_body(
   // the fused projection's row for operands read in place (tk/src/ops/attention.rs:104-122).
   const int64_t q_row_stride = q_row_elems;
   const int64_t o_row_stride = (int64_t)heads * D;
-  // ---- Q fragments: B operand of the score product, resident for the block.
   const int row = q_off + w.wave * kWaveRows + ln;  // this lane's row of the tile
   static_assert(!GROUPED || (!CAUSAL && !RANGED), "grouped tiles take no per-row masks");
   // This lane's query: row q_row of head q_head, when there is one.
@@ -850,15 +856,6 @@ __device__ __forceinline__ void flash_fwd_body(
     q_row = row - in_group * t;
     q_ok = in_group < (int)geo.group;
     q_head = kvh * (int)geo.group + min(in_group, (int)geo.group - 1);
-  }
-  {
-    const uint16_t *q_ptr = q + ((int64_t)b * t + q_row) * q_row_stride + (int64_t)q_head * D + w.g * 8;
-#pragma unroll
-    for (int ks = 0; ks < KS; ks++) {
-      u32x4 x = {0, 0, 0, 0};
-      if (q_ok) x = *reinterpret_cast<const u32x4 *>(q_ptr + ks * 16);
-      w.qf[ks] = x;
-    }
   }
 
   // L584-608: key blocks [first, end) hold every key some query of the tile sees.
@@ -974,6 +971,18 @@ __device__ __forceinline__ void flash_fwd_body(
   fill_k<D, NW>(w, 0, 0);
   fill_v<D, NW>(w, 0, 0);
   fill_k<D, NW>(w, 1, 1);
+  SVODK_TL(5);
+  // ---- Q fragments: B operand of the score product, resident for the block.  They are asked for after
+  // the fills (which have the longer way: the first barrier waits for both).
+  {
+    const uint16_t *q_ptr = q + ((int64_t)b * t + q_row) * q_row_stride + (int64_t)q_head * D + w.g * 8;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+      u32x4 x = {0, 0, 0, 0};
+      if (q_ok) x = *reinterpret_cast<const u32x4 *>(q_ptr + ks * 16);
+      w.qf[ks] = x;
+    }
+  }
   // A key mask row of up to kScannedBlocks blocks is scanned now, under the fills' flight: every
   // wave ballots each block's 64 keys into a word of its own LDS copy.  The scan also says where
   // the row's last visible key is (later blocks are skipped, like blocks past a length) and how
@@ -1212,7 +1221,7 @@ __device__ __forceinline__ void flash_fwd_body(
     for (int i = 0; i < 5; i++) at[i] = tl_stamp[i];
     at[5] = ((unsigned long long)xcc << 32) | hw;
     at[6] = ((unsigned long long)(unsigned)end << 32) | (unsigned)my_end;
-    at[7] = ((unsigned long long)(unsigned)b << 32) | (unsigned)(h << 8 | qt);
+    at[7] = tl_stamp[5];  // the first fills are out
   }
 #endif
 }

@@ -3,8 +3,8 @@
     python -m svod_amd.probes.timeline [--build] [bge_m3|qwen3_attention|whisper|long] [--no-row-order] [--raw=FILE.npy]
 
 Builds ``bin/libsvodk_timeline.so``, the library with ``-DSVODK_TIMELINE`` (thread 0 of every workgroup of
-``flash_fwd_kernel`` stamps the 100 MHz clock at entry, first barrier, last computed step, last step and
-stores landed, and notes its XCD, shader engine and CU), runs one call of a ``bench.py`` workload after
+``flash_fwd_kernel`` stamps the 100 MHz clock at entry, first fills issued, first barrier, last computed
+step, last step and stores landed, and notes its XCD, shader engine and CU), runs one call of a ``bench.py`` workload after
 warm-up and prints: the launch's span against the sum of the workgroups' own times, their phases, the
 time per key block, how many workgroups are resident over time, the gaps between one workgroup's end and
 the next one's start on a CU, each XCD's share of the time and its last end, and how each XCD deals
@@ -102,6 +102,8 @@ def main(argv) -> None:
     print(f"span {span:.1f} us; the workgroups' own times sum to {dur.sum():.0f} us = {dur.sum() / slots:.1f} us a slot "
           f"({100 * dur.sum() / slots / span:.0f} % of the span)")
     pct = lambda x: "mean %.2f  p50 %.2f  p90 %.2f" % (x.mean(), *np.percentile(x, [50, 90]))
+    fills_out = (t[:, 7].astype(np.int64) - t0) * 0.01
+    print("entry -> first fills out    ", pct(fills_out - start))
     print("entry -> first barrier      ", pct(first - start))
     print("first barrier -> last step  ", pct(idle_end - first), " per key block", pct((idle_end - first) / blocks))
     print("last step -> stores landed  ", pct(end - idle_end))

@@ -996,9 +996,27 @@ __device__ __forceinline__ void flash_fwd_body(
     bool open = true;
     int visible = 0, last_key = 0;  // keys the row shows, and the place after the last of them
     for (int base = 0; base < end; base += 8) {
+      // Eight blocks' elements in flight together: every lane loads (a key past the row's end, or a block
+      // past the tile's, loads the row's first element and drops it), so that no branch stands between the
+      // loads and a single wait brings them in.
       int words[8];
+      if (w.mask_bytes == 1) {
 #pragma unroll
-      for (int i = 0; i < 8; i++) words[i] = base + i < end ? mask_lane<D, NW>(w, base + i) : 0;
+        for (int i = 0; i < 8; i++) {
+          const int key = (base + i) * kBkv + w.lane;
+          const bool there = base + i < end && key < w.tk;
+          const int x = (int)((const uint8_t *)w.key_mask)[w.mask_row + (there ? key : 0)];
+          words[i] = there ? x : 0;
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+          const int key = (base + i) * kBkv + w.lane;
+          const bool there = base + i < end && key < w.tk;
+          const int x = ((const int *)w.key_mask)[w.mask_row + (there ? key : 0)];
+          words[i] = there ? x : 0;
+        }
+      }
 #pragma unroll
       for (int i = 0; i < 8; i++) {
         if (base + i >= end) break;

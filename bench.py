@@ -28,7 +28,8 @@ HBM_PEAK_GBS = 8000.0
 ROOT = os.path.dirname(os.path.abspath(__file__))
 # The workloads a default run times after the headline one, a few steps each, so that one run
 # carries every figure the targets are set on.
-OTHERS = ["qwen3_attention", "qwen3_prologue", "whisper", "long", "qwen3_projection"]
+OTHERS = ["bge_m3_bool", "qwen3_attention", "qwen3_prologue", "qwen3_add_rms_norm", "whisper", "long", "whisper_decode",
+          "qwen3_projection"]
 
 
 def hbm_traffic(workload):
@@ -41,6 +42,22 @@ def hbm_traffic(workload):
             return json.load(f).get("bytes_per_launch", {}).get(workload)
     except (OSError, ValueError):
         return None
+
+
+def device_clock_mhz():
+    """The device's peak engine clock in MHz, asked of the HIP runtime torch has loaded
+    (hipDeviceGetAttribute, hipDeviceAttributeClockRate), or a string that says why there is none."""
+    import ctypes
+
+    try:
+        hip = ctypes.CDLL("libamdhip64.so")
+        khz = ctypes.c_int(0)
+        rc = hip.hipDeviceGetAttribute(ctypes.byref(khz), ctypes.c_int(5), ctypes.c_int(0))  # 5: ClockRate, kHz
+        if rc != 0 or khz.value <= 0:
+            return "unavailable: hipDeviceGetAttribute(ClockRate) returned %d" % rc
+        return khz.value // 1000
+    except OSError as e:
+        return "unavailable: %s" % e
 
 
 def parse():
@@ -380,7 +397,9 @@ def main():
               "operands": "cold: the calls of a step rotate over operand sets larger than the 256 MB Infinity Cache "
                           "(us_per_call_warm: one set back to back, eager launches)",
               "device": props.name or props.gcnArchName, "compute_units": props.multi_processor_count,
-              "clock_mhz": props.clock_rate // 1000 if hasattr(props, "clock_rate") else None}
+              "clock_mhz": device_clock_mhz(),
+              "clock_note": "peak engine clock the runtime reports; the roofline peaks are MI355X's published ones "
+                            "(2.5 PFLOP/s dense bf16 at 2.4 GHz, 8 TB/s)"}
 
     # ---- CPU baseline: the oracle's restatement of the reference graph path, bounded sample.
     cpu = None
@@ -404,10 +423,14 @@ def main():
             ow = build_workload(other, args, dev)
             om = measure(ow, args.other_steps, 2, use_graph=not args.no_graph, spread=False, warm=False)
             r = roofline(other, ow, om["kernel_us"])
-            others.append({"workload": ow.text, "name": other, "calls_per_step": len(ow.calls), "steps": args.other_steps,
-                           "kernel": r["kernel"], "kernel_us": r["kernel_us"], "bound": r["bound"],
-                           "achieved": r["achieved"], "unit": r["unit"], "peak": r["peak"], "frac": r["frac"],
-                           "traffic": r["traffic"]})
+            entry = {"workload": ow.text, "name": other, "calls_per_step": len(ow.calls), "steps": args.other_steps,
+                     "kernel": r["kernel"], "kernel_us": r["kernel_us"], "bound": r["bound"],
+                     "achieved": r["achieved"], "unit": r["unit"], "peak": r["peak"], "frac": r["frac"],
+                     "traffic": r["traffic"]}
+            if other == "qwen3_prologue" and not args.no_cpu_baseline:
+                # ms/call against the host CPU for the prologue too: a short bounded sample of its graph path.
+                entry["cpu_baseline"] = cpu_baseline(ow.cpu_sample, min(args.cpu_seconds, 3.0), ow.bound)
+            others.append(entry)
             del ow
             torch.cuda.empty_cache()
 

@@ -141,7 +141,9 @@ typedef struct svodk_attn {
    * that row twice and leaves the rows it skips UNWRITTEN (entries out of range are clamped into the
    * batch, never followed out of the tensors).  With a permutation results do not depend on it.
    * svodk_order_rows fills one from the key lengths (always a permutation); a model computes it once
-   * per batch and passes it to every layer's call. */
+   * per batch and passes it to every layer's call.  Under a bound batch (0 < batch_live < B) the
+   * order is IGNORED and the rows run as they come: an order of all B rows would name rows past the
+   * live ones. */
   const svodk_tensor *row_order;
 } svodk_attn;
 
@@ -173,9 +175,11 @@ int svodk_attention(const svodk_tensor *q, const svodk_tensor *k, const svodk_te
  * svodk_attention; the one difference is where the partial states of a split call live: in a
  * static device array of the library, svodk_noalloc_scratch_bytes() (8 MiB) on each GPU the library
  * runs on, held until the process ends.  `opts->workspace` is ignored.  The call and everything
- * under it allocate nothing.  A call whose splits (named, or chosen for `splits` = 0 as if a workspace
- * had been lent) need more than the array holds answers SVODK_ERR_ARGUMENT and launches nothing;
- * svodk_attention_workspace says how much a call needs.  Every call on a GPU shares that GPU's
+ * under it allocate nothing.  With `splits` = 0 the count is chosen as if a workspace had been lent
+ * and then lowered to what the array holds (down to one split: the call runs unsplit, as
+ * svodk_attention runs it without a workspace).  A call whose NAMED splits need more than the array
+ * holds answers SVODK_ERR_ARGUMENT and launches nothing; svodk_attention_workspace says how much a
+ * call needs.  Every call on a GPU shares that GPU's
  * array: calls that overlap on one GPU (two streams, two threads) race on it and must be ordered
  * by the caller.  Nothing in the array has to start at zero (a split call writes every partial
  * state its merge reads).

@@ -35,24 +35,6 @@
 
 #include "kernels.h"
 
-// A timeline build (-DSVODK_TIMELINE, never the shipped library: svod_amd/probes/timeline.py makes and
-// reads one): thread 0 of every workgroup of flash_fwd_kernel leaves five stamps of the 100 MHz clock
-// (entry, first barrier, last computed step, last step, stores landed), where it ran and what it had to
-// do in the buffer svodk_debug_timeline_h<head size> names, eight 64-bit words a workgroup.
-#if defined(SVODK_TIMELINE) && defined(SVODK_HEAD) && !defined(SVODK_CODE_OBJECT)
-static __device__ unsigned long long *g_timeline = nullptr;
-#define SVODK_TL_CAT2(a, b) a##b
-#define SVODK_TL_CAT(a, b) SVODK_TL_CAT2(a, b)
-extern "C" int SVODK_TL_CAT(svodk_debug_timeline_h, SVODK_HEAD)(void *buf) {
-  return (int)hipMemcpyToSymbol(HIP_SYMBOL(g_timeline), &buf, sizeof(buf));
-}
-#define SVODK_TL_STAMPS unsigned long long tl_stamp[6] = {0, 0, 0, 0, 0, 0}
-#define SVODK_TL(i) asm volatile("s_memrealtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(tl_stamp[i])::"memory")
-#else
-#define SVODK_TL_STAMPS
-#define SVODK_TL(i)
-#endif
-
 namespace svodk {
 #if !defined(SVODK_CODE_OBJECT)
 // Workgroups per XCD of the streaming form (<= 0: a workgroup per query tile instead), and the
@@ -776,8 +758,6 @@ __device__ __forceinline__ void flash_fwd_body(
   // meet in one L2 instead of being spread over all eight.  (The reference's grid is query
   // tile fastest, then head, then batch, attention.rs:512,523; the order within a unit is that.)
   const uint32_t wg = __builtin_amdgcn_workgroup_id_x();
-  SVODK_TL_STAMPS;
-  SVODK_TL(0);
   const uint32_t local = wg / kXcds;
   const uint32_t round = div_by(local, geo.unit_size, geo.unit_rcp);
   const uint32_t within = local - round * geo.unit_size;
@@ -971,7 +951,6 @@ __device__ __forceinline__ void flash_fwd_body(
   fill_k<D, NW>(w, 0, 0);
   fill_v<D, NW>(w, 0, 0);
   fill_k<D, NW>(w, 1, 1);
-  SVODK_TL(5);
   // ---- Q fragments: B operand of the score product, resident for the block.  They are asked for after
   // the fills (which have the longer way: the first barrier waits for both).
   {
@@ -1077,7 +1056,6 @@ __device__ __forceinline__ void flash_fwd_body(
   // them lands inside the loop, where it would also wait out the fills in flight.
   __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
   __syncthreads();
-  SVODK_TL(1);
 
   // ---- the first block's scores, masked, and their row maximum.
   // A causal wave past its last visible key has nothing to add from a block: it only keeps
@@ -1134,9 +1112,7 @@ __device__ __forceinline__ void flash_fwd_body(
     hot_step<D, NW, 1>(w, smem, blk + 1, nv, sv, bm);
   }
   for (; blk < my_end; blk++) edge_step<D, NW, CAUSAL>(w, smem, blk, my_end, sv, bm);
-  SVODK_TL(2);
   for (; blk < end; blk++) idle_step<D, NW>(w, blk);
-  SVODK_TL(3);
 
   // ---- the appended rows (L739-755, L827-846): one more block of keys, from their own tensors,
   // which only the last split scores; the first `seen` of them are visible and no other mask
@@ -1229,19 +1205,6 @@ __device__ __forceinline__ void flash_fwd_body(
       }
     }
   }
-#if defined(SVODK_TIMELINE) && defined(SVODK_HEAD) && !defined(SVODK_CODE_OBJECT)
-  __builtin_amdgcn_s_waitcnt(0x0f70);  // the stores have landed
-  SVODK_TL(4);
-  if (g_timeline != nullptr && tid == 0) {
-    unsigned hw, xcc;
-    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)\n\ts_getreg_b32 %1, hwreg(HW_REG_XCC_ID)" : "=s"(hw), "=s"(xcc));
-    unsigned long long *at = g_timeline + (size_t)wg * 8;
-    for (int i = 0; i < 5; i++) at[i] = tl_stamp[i];
-    at[5] = ((unsigned long long)xcc << 32) | hw;
-    at[6] = ((unsigned long long)(unsigned)end << 32) | (unsigned)my_end;
-    at[7] = tl_stamp[5];  // the first fills are out
-  }
-#endif
 }
 #endif  // __HIP_DEVICE_COMPILE__
 

@@ -170,9 +170,6 @@ __device__ __forceinline__ void linear_body(uint8_t *smem, const uint16_t *__res
     for (int f = 0; f < kFills; f++) {
       i32x4 r = rsrc[f];
       if (s >= nk) r[2] = 0;
-#if defined(SVODK_LINEAR_WITHOUT_FILLS)  // a timing build (svod_amd/probes/linear_parts.py): wrong results
-      if (s >= kStages - 1) r[2] = 0;
-#endif
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
                    :
                    : "s"(lds_at[f] + slot), "v"(voff), "s"(r)
@@ -328,9 +325,6 @@ __device__ __forceinline__ void linear_body(uint8_t *smem, const uint16_t *__res
         u32x2 out;
         out[0] = pack2<F16>(acc[rb][cb][4 * q], acc[rb][cb][4 * q + 1]);
         out[1] = pack2<F16>(acc[rb][cb][4 * q + 2], acc[rb][cb][4 * q + 3]);
-#if defined(SVODK_LINEAR_WITHOUT_STORES)  // a timing build: the values are computed and (all but never) stored
-        if (out[0] != 0x7fc17fc1u || out[1] != 0x7fc27fc2u) continue;
-#endif
         *reinterpret_cast<u32x2 *>(y_row + col) = out;
       }
     }

@@ -602,13 +602,17 @@ static int attend(const svodk_tensor *q, const svodk_tensor *k, const svodk_tens
   a.splits = split_count(opts, a.batch, t, heads, kv_heads, tk);
   void *workspace = opts->workspace;
   if (a.splits > 1 && own_scratch) {
-    // The library's own array holds the partial states: a call that needs more than it has is
-    // refused, not shrunk (the caller asked for a call that allocates nothing, and gets that or an error).
-    const int64_t need = (int64_t)a.splits * a.batch * t * heads * (d + 2) * 4;
+    // The library's own array holds the partial states.  A split count the rule chose is lowered to
+    // what the array holds (down to one, as svodk_attention does without a workspace); a count the
+    // caller named is refused when it does not fit, not shrunk.
+    const int64_t per_split = (int64_t)a.batch * t * heads * (d + 2) * 4;
     int64_t have = 0;
     const hipError_t e = svodk::split_scratch(&workspace, &have);
     if (e != hipSuccess) return fail(SVODK_ERR_LAUNCH, "%s: the static scratch: %s", op, hipGetErrorString(e));
-    if (need > have)
+    if (opts->splits <= 0 && (int64_t)a.splits * per_split > have)
+      a.splits = (int32_t)std::max<int64_t>(1, per_split > 0 ? have / per_split : 1);
+    const int64_t need = (int64_t)a.splits * per_split;
+    if (a.splits > 1 && need > have)
       return fail(SVODK_ERR_ARGUMENT,
                   "%s: %d key splits of %lld rows need %lld bytes of partial states, the static scratch holds %lld", op,
                   a.splits, (long long)((int64_t)a.batch * t * heads), (long long)need, (long long)have);

@@ -91,7 +91,7 @@ def _fresh(shape, dtype, device) -> torch.Tensor:
 def load_library(path: Optional[str] = None) -> ctypes.CDLL:
     """The shared library, loaded once.  Missing library = hard error: there is
     no other implementation behind these ops.  ``path`` names another build of the same
-    library (the timeline build of ``svod_amd.probes.timeline``) and only counts on the first call."""
+    library and only counts on the first call."""
     global _lib
     if _lib is not None:
         return _lib

@@ -81,7 +81,40 @@ def sample_slices(w, picks):
                                          scale=w.scale)
 
 
-def check_workload(device, w, picks, bool_mask=False):
+def torch_attention_everywhere(w, o):
+    """Every element of `o` against matmul -> mask -> softmax -> matmul in f32 with plain torch ops on
+    the device (the routine the golden fixtures are made with, tests/golden/make_golden.py, here in f32
+    and one (batch row, head) chunk at a time so that the scores of an 8192-key row fit).  Returns the
+    worst absolute difference over the whole tensor."""
+    b, t, tk, h, hkv, d = w.dims
+    group = h // hkv
+    scale = w.scale if w.scale is not None else d ** -0.5
+    rows = torch.arange(t, device=o.device).unsqueeze(1)
+    cols = torch.arange(tk, device=o.device).unsqueeze(0)
+    heads_a_chunk = max(1, min(h, (1 << 28) // max(1, t * tk)))  # at most 1 GiB of f32 scores at a time
+    worst = 0.0
+    for bi in range(b):
+        keep = torch.ones((t, tk), dtype=torch.bool, device=o.device)
+        if w.key_lens is not None:
+            keep &= cols < int(w.key_lens[bi])
+        if w.causal:
+            keep &= cols <= rows
+        for h0 in range(0, h, heads_a_chunk):
+            hs = torch.arange(h0, min(h, h0 + heads_a_chunk), device=o.device)
+            q = w.q[bi, :, hs].float().transpose(0, 1)                 # [heads, T, D]
+            k = w.k[bi][:, hs // group].float().transpose(0, 1)        # [heads, Tk, D]
+            v = w.v[bi][:, hs // group].float().transpose(0, 1)
+            s = torch.matmul(q, k.transpose(1, 2)) * scale
+            s = s.masked_fill(~keep, float("-inf"))
+            p = torch.softmax(s, dim=-1)
+            p = torch.where(keep.any(dim=1, keepdim=True), p, torch.zeros_like(p))  # a row no key reaches: zeros
+            want = torch.matmul(p, v).transpose(0, 1)                  # [T, heads, D]
+            worst = max(worst, float((o[bi, :, hs].float() - want).abs().max()))
+            del s, p, want
+    return worst
+
+
+def check_workload(device, w, picks, bool_mask=False, everywhere=True):
     keys = KeyMask.none()
     if w.key_lens is not None:
         keys = KeyMask.bool(w.key_mask()) if bool_mask else KeyMask.lens(w.key_lens)
@@ -92,6 +125,9 @@ def check_workload(device, w, picks, bool_mask=False):
     for bi, hs, p in sample_slices(w, picks):
         got = to_np(o[bi:bi + 1, :, hs])
         assert_bf16_parity(f"{w.name} b{bi} h{hs}", got, oracle.attention_direct(p), oracle.attention_flash(p, 128, 64))
+    if everywhere:
+        worst = torch_attention_everywhere(w, o)
+        assert worst <= 2e-2, f"{w.name}: max-abs {worst} over the whole tensor"  # tk/src/test/unit/attention.rs:483
     return o
 
 
@@ -100,7 +136,7 @@ def test_config2_bge_m3_full_size(device):
     lens = w.key_lens.tolist()
     picks = [(int(np.argmin(lens)), 0), (int(np.argmax(lens)), 15), (7, 3)]
     o = check_workload(device, w, picks)
-    ob = check_workload(device, w, picks[:1], bool_mask=True)
+    ob = check_workload(device, w, picks[:1], bool_mask=True, everywhere=False)  # the same bits, asserted below
     assert torch.equal(o.view(torch.int16), ob.view(torch.int16)), "Lens and Bool masks give the same bits"
     # Size-independent property: keys past the length do not matter.  Poison them and rerun.
     k2, v2 = w.k.clone(), w.v.clone()
@@ -125,6 +161,19 @@ def test_config3_qwen3_prologue_and_attention_full_size(device):
         for got, wd, wp, what in zip((q, k, v), want, prog, "qkv"):
             g = to_np(got[bi:bi + 1, rows])
             assert max_abs(g, wd) <= 2e-2 and max_abs(g, wp) <= 1e-2, what
+    # Every element of q and k against the same arithmetic in f32 with plain torch ops on the device
+    # (tk/src/kernels/heads.rs:73-111), at the op-against-graph bar of tk/src/test/unit/mod.rs:526-536.
+    x = p.qkv.view(8, 2048, 32, 128).float()
+    cos, sin = p.cos.float(), p.sin.float()  # [1, T, 1, D/2]
+    for got, sl, wn, what in ((q, slice(0, 16), p.q_w, "q"), (k, slice(16, 24), p.k_w, "k")):
+        xs = x[:, :, sl]
+        y = xs * torch.rsqrt((xs * xs).mean(dim=-1, keepdim=True) + p.eps) * wn.float()
+        y1, y2 = y[..., :64], y[..., 64:]
+        want = torch.cat((y1 * cos - y2 * sin, y1 * sin + y2 * cos), dim=-1)
+        diff = (got.float() - want).abs()
+        assert bool((diff <= 2e-2 * want.abs().clamp(min=1.0)).all()), f"{what}: worst {float(diff.max())} over the whole tensor"
+        del xs, y, want, diff
+    del x
     # v is the input's v slots bit for bit, everywhere.
     vin = p.qkv.view(8, 2048, 32, 128)[:, :, 24:, :]
     assert torch.equal(v.view(torch.int16), vin.contiguous().view(torch.int16))

@@ -25,9 +25,14 @@ def both(device, dev_ops, opts):
     want = svod_amd.attention(q, k, v, opts)  # lends a workspace of its own
     chosen_want = svod_amd.chosen()
     out = torch.full_like(q, float("nan"))
-    before = torch.cuda.memory_allocated(device)
+    # Neither torch's allocator nor the device itself gives anything out under the call: the second
+    # figure is the device's free bytes (a hipMalloc inside the library would lower it).
+    torch.cuda.synchronize()
+    before, free_before = torch.cuda.memory_allocated(device), torch.cuda.mem_get_info(device)[0]
     got = svod_amd.attention_noalloc(q, k, v, opts, out)
+    torch.cuda.synchronize()
     assert torch.cuda.memory_allocated(device) == before
+    assert torch.cuda.mem_get_info(device)[0] == free_before
     assert svod_amd.chosen() == chosen_want
     torch.cuda.synchronize()
     return got, want
@@ -71,3 +76,45 @@ def test_a_call_past_the_scratch_is_refused(device):
     assert e.value.kind == "Argument" and "static scratch holds" in str(e.value)
     torch.cuda.synchronize()
     assert torch.isnan(out).all()  # nothing was launched
+
+
+def test_splits_of_the_rules_own_shrink_to_the_scratch(device):
+    # splits = None on a prefill whose rule asks for 2 splits of 17 MB each: past the 8 MiB array the
+    # count drops to one, as svodk_attention drops it without a workspace, and the call runs unsplit.
+    b, t, tk, h, d = 1, 2048, 2048, 16, 128
+    assert 2 * b * t * h * (d + 2) * 4 > svod_amd.noalloc_scratch_bytes()
+    _, (q, k, v) = operands(device, b, t, tk, h, h, d, seed=21)
+    out = torch.full_like(q, float("nan"))
+    got = svod_amd.attention_noalloc(q, k, v, Attn(), out)
+    assert svod_amd.chosen().startswith('Kernel { op: "attention", family: "flash_attention"'), svod_amd.chosen()
+    want = svod_amd.attention(q, k, v, Attn(splits=1))
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(got), bits(want))
+
+
+def test_a_captured_split_call_replays(device):
+    # The callers the entry point is for: a split call captured in a HIP graph (after one eager call on
+    # the device, which looks the array's address up) and replayed with eager work between the replays.
+    host, dev_ops = operands(device, 2, 1, 2048, 8, 2, 128, seed=29)
+    q, k, v = dev_ops
+    opts = Attn(splits=4)
+    eager = svod_amd.attention_noalloc(q, k, v, opts, torch.full_like(q, float("nan")))
+    torch.cuda.synchronize()
+    out = torch.full_like(q, float("nan"))
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        svod_amd.attention_noalloc(q, k, v, opts, out)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        svod_amd.attention_noalloc(q, k, v, opts, out)
+    for _ in range(3):
+        out.fill_(float("nan"))
+        # eager work on the same array between the replays: a smaller split call
+        svod_amd.attention_noalloc(q[:1], k[:1], v[:1], Attn(splits=2), torch.empty_like(q[:1]))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(bits(out), bits(eager))

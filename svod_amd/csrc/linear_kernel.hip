@@ -10,14 +10,18 @@
 // The mapping onto CDNA4 is this file's own.  A workgroup of 8 waves owns a 256 x 256 output tile; a wave
 // owns 64 rows x 128 columns as 2 x 4 accumulators of v_mfma_f32_32x32x16.  The product runs transposed,
 // C^T = W . X^T, so that a lane owns one output ROW and, per accumulator register quad, four CONSECUTIVE
-// columns: the store is 8-byte runs, the rotation's partner column (32 or 64 columns along) is the same
-// lane's register of another accumulator, and the tables (staged through LDS once the ring is done with)
-// are read as 8-byte runs of the lane's row.
-// X and W tiles of 32 k-columns stream through a four-stage LDS ring (32 KiB a stage), filled global -> LDS
-// by buffer_load_dwordx4 ... lds three stages ahead; rows are 64 bytes, their four 16-byte chunks
-// XOR-swizzled by (row / 4) % 4 through the lanes' source addresses so that a ds_read_b128 of 16 rows at one
-// logical chunk touches every bank once.  Rows past the operands' ends read as zeros through the buffer
-// descriptors' bounds.  One barrier a stage (16 MFMAs a wave).
+// columns: the rotation's partner column (32 or 64 columns along) is the same lane's register of another
+// accumulator, and the tables (staged through LDS once the ring is done with) are read as 8-byte runs of the
+// lane's row.  The finished tile goes through LDS once more, a wave's rows in a stretch of its own, and
+// leaves as whole 256-byte row segments, 16 bytes a lane.
+// X and W tiles of 64 k-columns stream through a two-stage LDS ring (64 KiB a stage), filled global -> LDS
+// by buffer_load_dwordx4 ... lds a stage ahead.  What bounds this kernel is the way from L2 into LDS: the
+// part moves about 18 TB/s along it when every fill takes whole 128-byte lines and about 12 TB/s when it
+// takes half lines (measured: the fills of this kernel alone, without its products).  Hence tiles this
+// large (1 GiB of fills at the projection shape where 256 x 128 tiles move 1.5 GiB) and rows of 128 bytes,
+// a whole line each; their eight 16-byte chunks are XOR-swizzled by (row / 2) % 8 through the lanes' source
+// addresses so that a ds_read_b128 of 16 rows at one logical chunk touches every bank once.  Rows past the
+// operands' ends read as zeros through the buffer descriptors' bounds.  One barrier a stage (32 MFMAs a wave).
 #include <hip/hip_runtime.h>
 
 #include <atomic>
@@ -45,14 +49,17 @@ typedef __attribute__((ext_vector_type(4))) int i32x4;
 constexpr int kXcds = 8;
 constexpr int kWaves = 8;               // 4 along the rows x 2 along the columns
 constexpr int kBm = 256, kBn = 256;     // the workgroup's output tile
-constexpr int kBk = 32;                 // k-columns a stage
-constexpr int kStages = 4;
+constexpr int kBk = 64;                 // k-columns a stage: a row of a tile is one 128-byte line
+constexpr int kSteps = kBk / 16;        // k-steps of the matrix instruction a stage
+constexpr int kStages = 2;
 constexpr int kGroup = 8;               // column tiles an XCD's resident workgroups spread over
 constexpr int kRowBytes = kBk * 2;      // a tile row in LDS
-constexpr int kTileBytes = kBm * kRowBytes;           // one operand's tile: 16 KiB
+constexpr int kTileBytes = kBm * kRowBytes;           // one operand's tile: 32 KiB
 constexpr int kStageBytes = 2 * kTileBytes;           // W tile, then X tile
 constexpr int kLds = kStages * kStageBytes;           // 128 KiB
-constexpr int kFills = 2 * (kTileBytes / 1024) / kWaves;  // wave instructions of 1 KiB per wave and stage: 4
+constexpr int kFills = kStageBytes / 1024 / kWaves;   // wave instructions of 1 KiB per wave and stage: 8
+constexpr int kOutPitch = 128 * 2 + 16;               // a wave's row of the finished tile in LDS
+static_assert(kWaves * 32 * kOutPitch <= kLds, "half of the finished tile fits where the ring was");
 
 template <bool F16>
 __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
@@ -142,25 +149,29 @@ __device__ __forceinline__ void linear_body(uint8_t *smem, const uint16_t *__res
   const int32_t n0 = (int32_t)tn * kBn;
   const int64_t row_bytes = (int64_t)k * 2;
 
-  // ---- this wave's fills of a stage: 16 rows x 4 chunk places an instruction, rows 16 * wave and
-  // 128 + 16 * wave of the W tile and of the X tile.  The swizzle's period is 16 rows, so one lane
-  // offset serves all four; the descriptors' bases differ.
-  const int frow = lane >> 2, place = lane & 3;
-  const int src = frow * (int)row_bytes + ((place ^ ((frow >> 2) & 3)) << 4);
+  // ---- this wave's fills of a stage: 8 rows x 8 chunk places an instruction; a stage is 64 of them, the
+  // W tile's 32 and then the X tile's 32, and wave v takes instructions v, v + 8, ...  Those are 64 rows
+  // apart, a multiple of the swizzle's period of 16, so one lane offset serves all eight; the descriptors'
+  // bases differ.
+  const int frow = lane >> 3, place = lane & 7;
+  const int src = frow * (int)row_bytes + ((place ^ ((4 * (wave & 1) + (frow >> 1)) & 7)) << 4);
   i32x4 rsrc[kFills];
   int lds_at[kFills];
 #pragma unroll
   for (int f = 0; f < kFills; f++) {
+    const int j = wave + kWaves * f;  // the instruction of the stage
     const bool is_x = f >= kFills / 2;
-    const int block_row = 16 * wave + 128 * (f & 1);
+    const int block_row = 8 * (is_x ? j - kTileBytes / 1024 : j);
     const int64_t first = (is_x ? m0 : (int64_t)n0) + block_row;
     const int64_t limit = is_x ? rows : (int64_t)n;
     const uint16_t *base = is_x ? x : w;
     rsrc[f] = make_rsrc((const uint8_t *)base + first * row_bytes, (limit - first) * row_bytes);
-    lds_at[f] = (int)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)(smem) + (is_x ? kTileBytes : 0) +
-                block_row * kRowBytes;
+    lds_at[f] = (int)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)(smem) + j * 1024;
   }
-  const int nk = k / kBk;
+  // k is a multiple of 32: a last stage may hold two k-steps only (what its rows' second halves fetch is the
+  // next rows' data or, past the operand, zeros: never multiplied).
+  const int nk = (k + kBk - 1) / kBk;
+  const bool short_tail = (k % kBk) != 0;
   // Stage `s` of the k loop into its ring slot; past the last stage an empty descriptor (zeros land in a
   // slot nothing reads any more) keeps the count of fills in flight the same in every iteration.
   auto fill = [&](int s) {
@@ -176,8 +187,8 @@ __device__ __forceinline__ void linear_body(uint8_t *smem, const uint16_t *__res
                    : "memory");
     }
   };
-#pragma unroll
-  for (int s = 0; s < kStages - 1; s++) fill(s);
+  fill(0);
+  fill(1);
 
   // ---- operand reads: A = W rows (the output's columns), B = X rows (the output's rows); fragment
   // (block of 32 rows, k-step ks): row ln of the block, logical chunk 2 * ks + g.
@@ -187,10 +198,10 @@ __device__ __forceinline__ void linear_body(uint8_t *smem, const uint16_t *__res
   for (int cb = 0; cb < 4; cb++) a_read[cb] = (wave_n * 128 + cb * 32 + ln) * kRowBytes;
 #pragma unroll
   for (int rb = 0; rb < 2; rb++) b_read[rb] = kTileBytes + (wave_m * 64 + rb * 32 + ln) * kRowBytes;
-  const int swz = (ln >> 2) & 3;  // every block starts on a multiple of 16 rows
-  int chunk_at[2];
+  const int swz = (ln >> 1) & 7;  // every block starts on a multiple of 16 rows
+  int chunk_at[kSteps];
 #pragma unroll
-  for (int ks = 0; ks < 2; ks++) chunk_at[ks] = ((2 * ks + g) ^ swz) << 4;
+  for (int ks = 0; ks < kSteps; ks++) chunk_at[ks] = ((2 * ks + g) ^ swz) << 4;
 
   f32x16 acc[2][4];
   const f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
@@ -213,22 +224,28 @@ __device__ __forceinline__ void linear_body(uint8_t *smem, const uint16_t *__res
 #pragma unroll
       for (int rb = 0; rb < 2; rb++) acc[rb][cb] = mma<F16>(af[cb], bf[rb], acc[rb][cb]);
   };
-  // The loop runs one stage behind its barrier: iteration s first makes sure stage s + 1 has landed for
-  // every wave (and that every wave is done with stage s - 1, whose slot stage s + 3 then takes), so the
-  // first fragments of stage s + 1 can be asked for under the last products of stage s and no product
-  // waits on LDS behind a barrier.
+  // A stage is four k-steps.  Before its last one every wave makes sure its own fills of the next stage
+  // have landed and its reads of this stage are back, and meets the others: behind that barrier the next
+  // stage is whole and this stage's slot is free, so the fills of the stage after next go out and the next
+  // stage's first fragments are asked for under this stage's last products.
   u32x4 a0[4], b0[2], a1[4], b1[2];
-  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kFills * (kStages - 2)) : "memory");  // stage 0 is in
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kFills) : "memory");  // stage 0 is in
   __syncthreads();
   fragments(0, 0, a0, b0);
   for (int s = 0; s < nk; s++) {
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kFills * (kStages - 3)) : "memory");  // stage s + 1 is in
-    __syncthreads();
-    fill(s + kStages - 1);
-    fragments(s % kStages, 1, a1, b1);
+    const int slot = s & 1;
+    fragments(slot, 1, a1, b1);
     multiply(a0, b0);
-    fragments((s + 1) % kStages, 0, a0, b0);
+    fragments(slot, 2, a0, b0);
     multiply(a1, b1);
+    fragments(slot, 3, a1, b1);
+    const bool whole = !short_tail || s + 1 < nk;
+    if (whole) multiply(a0, b0);
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");  // stage s + 1 is in, stage s is read
+    __syncthreads();
+    fill(s + 2);
+    fragments(slot ^ 1, 0, a0, b0);
+    if (whole) multiply(a1, b1);
   }
   // The empty fills still in flight write LDS: they land before the workgroup's LDS is given away.
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -266,6 +283,7 @@ __device__ __forceinline__ void linear_body(uint8_t *smem, const uint16_t *__res
     uint8_t *cos_lds = smem, *sin_lds = smem + kBm * kPitch;
     __syncthreads();  // every wave's last fragments are read and its last fills have landed
     const uint32_t pos0 = (uint32_t)(m0 % seq);
+    static_assert(2 * kBm * kPitch <= kLds, "the tables fit where the ring was");
     for (int c = tid; c < kBm * kChunks; c += kWaves * 64) {
       const int r = c / kChunks, ch = c % kChunks;
       const uint32_t pos = (pos0 + (uint32_t)r) % (uint32_t)seq;  // gemm.rs:685: the table row of the token's position
@@ -311,22 +329,34 @@ __device__ __forceinline__ void linear_body(uint8_t *smem, const uint16_t *__res
       }
     }
   }
+  // ---- the store.  A lane owns rows, not runs of columns: written from the registers an instruction would
+  // touch 32 rows with 16 bytes each.  The rounded tile goes through LDS instead (every wave is done with the
+  // ring, and with the tables), 32 rows of a wave at a time in a stretch of its own, and leaves as whole row
+  // segments: an instruction stores 4 rows of 256 bytes, 16 bytes a lane.
+  __syncthreads();
+  uint8_t *stage = smem + wave * 32 * kOutPitch;
+  const int orow = lane >> 4, ochunk = lane & 15;
+  const int col = n0 + wave_n * 128 + ochunk * 8;  // n is a multiple of 8: a run of eight lies inside or outside
 #pragma unroll
   for (int rb = 0; rb < 2; rb++) {
-    const int64_t row = m0 + wave_m * 64 + rb * 32 + ln;
-    if (row >= rows) continue;
-    uint16_t *y_row = y + row * (int64_t)n;
+    uint8_t *srow = stage + ln * kOutPitch + 8 * g;
 #pragma unroll
     for (int cb = 0; cb < 4; cb++) {
 #pragma unroll
       for (int q = 0; q < 4; q++) {
-        const int col = col_base + 32 * cb + 8 * q;
-        if (col >= n) continue;  // n is a multiple of 8: a run of four lies inside or outside
         u32x2 out;
         out[0] = pack2<F16>(acc[rb][cb][4 * q], acc[rb][cb][4 * q + 1]);
         out[1] = pack2<F16>(acc[rb][cb][4 * q + 2], acc[rb][cb][4 * q + 3]);
-        *reinterpret_cast<u32x2 *>(y_row + col) = out;
+        *reinterpret_cast<u32x2 *>(srow + (32 * cb + 8 * q) * 2) = out;
       }
+    }
+#pragma unroll
+    for (int it = 0; it < 8; it++) {
+      const int r = it * 4 + orow;
+      const u32x4 out = *reinterpret_cast<const u32x4 *>(stage + r * kOutPitch + ochunk * 16);
+      const int64_t row = m0 + wave_m * 64 + rb * 32 + r;
+      // Streaming stores: the output is not read again here, and left out of L2 it does not push the operands out.
+      if (row < rows && col < n) __builtin_nontemporal_store(out, reinterpret_cast<u32x4 *>(y + row * (int64_t)n + col));
     }
   }
 }
@@ -375,7 +405,9 @@ hipError_t launch(const LinearArgs &a, hipStream_t stream) {
 
 }  // namespace
 
-bool linear_supports(int64_t n, int64_t k) { return n > 0 && n % 8 == 0 && k >= kBk && k % kBk == 0 && k <= 0x3fffffff; }
+// A fill's lanes address their rows with 32-bit byte offsets from the descriptor's base: 8 rows of 2 k bytes,
+// and the stage's place along them.
+bool linear_supports(int64_t n, int64_t k) { return n > 0 && n % 8 == 0 && k >= 32 && k % 32 == 0 && k <= (1 << 25); }
 
 bool linear_turns(int32_t head_dim) { return head_dim == 64 || head_dim == 128; }
 

@@ -97,9 +97,9 @@ typedef struct svodk_cache {
  * Windows, chunk masks, segment starts (I32 or I64, non-decreasing along T)
  * an additive bias (of the operands' type, rows unpadded; with appended rows
  * its last dim counts them, their columns last) and a cache have kernels.
- * Every combination the reference's own tests hold runs; a cache together with
- * a window, a chunk mask or segment starts, and more than 64 appended rows,
- * answer SVODK_GRAPH_CONFIG.
+ * Every combination runs, a cache under a window, a chunk mask or segment starts
+ * included (the ranges hide cached keys only; appended rows answer to app_lens alone);
+ * more than 64 appended rows answer SVODK_GRAPH_CONFIG.
  *
  * `splits` > 1 asks for key splits (tk/src/ops/attention.rs:76-79, 280-302): the
  * count is capped at the number of 64-key blocks of Tk (split_ranked, :405-410);

@@ -57,18 +57,19 @@ class _Ranges(ctypes.Structure):
                 ("bias", ctypes.POINTER(ctypes.c_float)), ("bias_per_batch", ctypes.c_int32),
                 ("bias_cols", ctypes.c_int32), ("appended", ctypes.c_int32),
                 ("k_app", ctypes.POINTER(ctypes.c_float)), ("v_app", ctypes.POINTER(ctypes.c_float)),
-                ("app_seen", ctypes.POINTER(ctypes.c_int32))]
+                ("app_seen", ctypes.POINTER(ctypes.c_int32)), ("app_from", ctypes.c_int32)]
 
 
 _rangesp = ctypes.POINTER(_Ranges)
 
 
-def _ranges(chunk, seg_start, bias=None, batch=None, appended=None):
+def _ranges(chunk, seg_start, bias=None, batch=None, appended=None, app_from=0):
     """(pointer or None, what must stay alive) for ``chunk = (size, left or None, right)``, ``seg_start [B,T]``,
     ``bias [B or 1, H, T, Tk (+ appended rows)]`` and ``appended = (k_app, v_app, seen or None)``."""
-    if chunk is None and seg_start is None and bias is None and appended is None:
+    if chunk is None and seg_start is None and bias is None and appended is None and not app_from:
         return None, None
     r = _Ranges()
+    r.app_from = int(app_from)
     seg = None
     if appended is not None:
         k_app, v_app, seen = appended
@@ -253,6 +254,7 @@ class AttnProblem:
     bf16: bool = True
     cache: Optional[Cache] = None
     appended: Optional[tuple] = None  # (k_app, v_app, seen or None) beside gathered k and v: what ``gathered`` leaves
+    app_from: int = 0  # the first appended column of keys that ``concatenated`` has joined (0: none): the direct softmax only
 
     def dims(self):
         b, t, h, d = self.q.shape
@@ -286,7 +288,7 @@ class AttnProblem:
         seen = np.full(b, n) if seen is None else seen
         mask = np.concatenate([np.arange(tk)[None, :] < lens[:, None], np.arange(n)[None, :] < seen[:, None]], axis=1)
         return dataclasses.replace(p, k=np.concatenate([p.k, k_app], axis=1), v=np.concatenate([p.v, v_app], axis=1),
-                                   key_lens=None, key_mask=mask, appended=None)
+                                   key_lens=None, key_mask=mask, appended=None, app_from=tk)
 
     def scale_f32(self) -> float:
         d = self.q.shape[-1]
@@ -303,7 +305,7 @@ class AttnProblem:
         keys = tk + (0 if self.appended is None else self.appended[0].shape[1])
         if self.bias is not None and tuple(self.bias.shape[1:]) != (h, t, keys):
             raise ValueError(f"bias has shape {self.bias.shape}, expected [{b} | 1, {h}, {t}, {keys}]")
-        ranges, alive = _ranges(self.chunk, self.seg_start, self.bias, b, self.appended)
+        ranges, alive = _ranges(self.chunk, self.seg_start, self.bias, b, self.appended, self.app_from)
         keep = (lens, mask, alive)
         args = [b, t, tk, h, hkv, d, int(self.causal), wl, wr, ctypes.c_float(self.scale_f32()),
                 _ptr(lens, _i32p), _ptr(mask, _i32p), tk, ranges]
@@ -324,7 +326,9 @@ def attention_direct(p: AttnProblem, threads: int = 8) -> np.ndarray:
 
 def attention_graph(p: AttnProblem, threads: int = 8) -> np.ndarray:
     """The op's graph fallback (tk/src/ops/attention.rs:496-584); float32 [B,T,H,D]."""
-    p = p.concatenated()
+    # The graph joins the appended rows to the cached keys and masks the lot (L507-531, L573-583): unlike the
+    # kernel's step for them, its causal, window, chunk and segment masks reach the appended columns too.
+    p = dataclasses.replace(p.concatenated(), app_from=0)
     q, k, v = _f32(p.q), _f32(p.k), _f32(p.v)
     out = np.empty(q.shape, dtype=np.float32)
     args, _keep = p._common()

@@ -221,6 +221,10 @@ typedef struct {
   int32_t appended;         /* rows a batch lane, 0 = none */
   const float *k_app, *v_app; /* [batch, appended, kv_heads, d] */
   const int32_t *app_seen;  /* [batch] visible appended rows, or NULL: all of them */
+  /* The direct softmax only, over keys that already hold the appended rows behind the cached ones: the
+   * first appended column (0 = none).  Columns from there on answer to the key mask alone
+   * (tk/src/test/unit/attention.rs:138-141: `if j >= s.tk { return j - s.tk >= seen; }`). */
+  int32_t app_from;
 } svod_oracle_extras;
 
 typedef struct {
@@ -268,6 +272,8 @@ static inline int hidden_without_ranges(const attn_problem *p, int32_t b, int32_
   return 0;
 }
 static inline int hidden(const attn_problem *p, int32_t b, int32_t i, int32_t j) {
+  if (p->ranges && p->ranges->app_from > 0 && j >= p->ranges->app_from)
+    return p->key_mask && p->key_mask[(int64_t)b * p->mask_stride + j] == 0;
   return hidden_without_ranges(p, b, i, j) || hidden_by_ranges(p, b, i, j);
 }
 

@@ -54,9 +54,8 @@ _COMBINE = [("o_part", B), ("m_part", B), ("l_part", B), ("o", B), ("rows", S), 
 
 def full_forms():
     """(causal, split, ranged, biased, cached, grouped) of every instantiation the library's own
-    dispatch reaches: a cache excludes per-row ranges; grouped tiles take neither a causal mask
-    nor ranges."""
-    for ranged, biased, cached in ((0, 0, 0), (0, 1, 0), (1, 0, 0), (1, 1, 0), (0, 0, 1), (0, 1, 1)):
+    dispatch reaches: grouped tiles take neither a causal mask nor ranges."""
+    for ranged, biased, cached in ((0, 0, 0), (0, 1, 0), (1, 0, 0), (1, 1, 0), (0, 0, 1), (0, 1, 1), (1, 0, 1), (1, 1, 1)):
         for causal in (0, 1):
             for split in (0, 1):
                 yield causal, split, ranged, biased, cached, 0
@@ -71,6 +70,8 @@ def full_name(d: int, dtype: str, causal, split, ranged, biased, cached, grouped
 
 _HEADS = [("qkv", B), ("q_w", B), ("k_w", B), ("cos", B), ("sin", B), ("q", B), ("k", B), ("v", B),
           ("rows", S), ("t", S), ("heads", S), ("kv_heads", S), ("eps_bits", S), ("rope", S)]
+_LINEAR = [("x", B), ("w", B), ("bias", B), ("cos", B), ("sin", B), ("y", B),
+           ("rows", S), ("n", S), ("k", S), ("seq", S), ("heads", S)]
 _TAIL = [("rows", S), ("d", S), ("eps_bits", S)]
 _ROWS = {"rms_norm": [("x", B), ("w", B), ("out", B)] + _TAIL,
          "add_rms_norm": [("x", B), ("residual", B), ("w", B), ("out", B), ("sum", B)] + _TAIL,
@@ -111,11 +112,19 @@ def entries() -> Dict[str, dict]:
                 "file": "svodk_combine.co", "source": "combine_kernel.hip", "params": _COMBINE, "local": [256, 1, 1],
                 "workgroups": f"(rows * {d // 4} + 255) // 256", "op": "combine_splits", "dtype": dtype, "head_dim": d,
                 "cfg": "NormCfg { br: 4 }"}
-        for d in (64, 128):
+        for d in (16, 32, 64, 128, 256):
             out[f"svodk_heads_d{d}_{dtype}"] = {
                 "file": "svodk_heads.co", "source": "heads_kernel.hip", "params": _HEADS, "local": [256, 1, 1],
                 "workgroups": f"(rows * (heads + 2 * kv_heads) * {d // 16} + 255) // 256",
                 "op": "heads", "dtype": dtype, "head_dim": d, "cfg": "NormCfg { lanes_per_head: d/16, block: 256 }"}
+        for turn in (0, 64, 128):  # the projection GEMM, plain or with the first `heads` heads of `turn` columns turned
+            out[f"svodk_linear_{'rope%d_' % turn if turn else ''}{dtype}"] = {
+                "file": "svodk_linear.co", "source": "linear_kernel.hip", "params": _LINEAR, "local": [512, 1, 1],
+                "workgroups": "(((rows + 255) // 256 + 7) // 8 * ((n + 255) // 256) if (rows + 255) // 256 >= 16 "
+                              "else ((rows + 255) // 256 * ((n + 255) // 256) + 7) // 8) * 8",
+                "op": "linear", "dtype": dtype, "rope_head_dim": turn,
+                "cfg": f"GemmCfg {{ bm: 256, bn: 256, bk: 64, stages: 2, waves: 8, core: mfma_f32_32x32x16_{dtype}"
+                       + (", epilogue: rope }" if turn else " }")}
         for kind, params in _ROWS.items():
             for dmax in (1024, 2048, 4096):
                 out[f"svodk_{kind}_d{dmax}_{dtype}"] = {

@@ -1209,7 +1209,7 @@ __device__ __forceinline__ void flash_fwd_body(
 #endif  // __HIP_DEVICE_COMPILE__
 
 template <int D, int NW, bool CAUSAL, bool SPLIT, bool RANGED, bool BIASED, bool CACHED, bool GROUPED, bool F16>
-__global__ __launch_bounds__(NW * 64, (D <= 64 && !BIASED) ? 3 : (D <= 128 ? 2 : 1)) void flash_fwd_kernel(
+__global__ __launch_bounds__(NW * 64, (D <= 64 && !BIASED && !(RANGED && CACHED)) ? 3 : (D <= 128 ? 2 : 1)) void flash_fwd_kernel(
     uint32_t unit_size, uint32_t unit_rcp, uint32_t nqt_u, uint32_t nqt_rcp, uint32_t kvh_u, uint32_t kvh_rcp,
     uint32_t units, uint32_t heads_group, const void *__restrict__ key_lens, const int32_t *__restrict__ row_order,
     int32_t t, uint32_t tk_lens64, const uint16_t *__restrict__ q, const uint16_t *__restrict__ k,
@@ -1707,7 +1707,9 @@ hipError_t launch_t(const AttnArgs &a, hipStream_t stream) {
   const bool ranged = a.win_left >= 0 || a.chunk_size > 0 || a.seg_start != nullptr;
   const bool biased = a.bias != nullptr;
   if (a.cached) {
-    if (ranged) return hipErrorInvalidValue;  // not instantiated: the op layer keeps the graph
+    // A cache under per-row ranges (Attn allows every combination, tk/src/ops/attention.rs:60-86): the ranges
+    // hide cached keys only, the appended rows answer to their own count (tk/src/test/unit/attention.rs:138-141).
+    if (ranged) return biased ? launch_s<D, true, true, true, F16>(a, stream) : launch_s<D, true, false, true, F16>(a, stream);
     return biased ? launch_s<D, false, true, true, F16>(a, stream) : launch_s<D, false, false, true, F16>(a, stream);
   }
   if (biased) return ranged ? launch_s<D, true, true, false, F16>(a, stream) : launch_s<D, false, true, false, F16>(a, stream);
@@ -1946,13 +1948,13 @@ __device__ __forceinline__ void attention_entry_full(uint8_t *smem, SVODK_FULL_P
 #endif
 
 #define SVODK_FULL_ENTRY(D, T, F16, C, S, R, B, K, G)                                                                 \
-  extern "C" __global__ __launch_bounds__(256, ((D) <= 64 && !(B)) ? 3 : ((D) <= 128 ? 2 : 1)) void                   \
+  extern "C" __global__ __launch_bounds__(256, ((D) <= 64 && !(B) && !((R) && (K))) ? 3 : ((D) <= 128 ? 2 : 1)) void  \
       svodk_attention_full_d##D##_##T##_c##C##s##S##r##R##b##B##k##K##g##G(SVODK_FULL_PARAMS) {                       \
     __shared__ __attribute__((aligned(1024))) uint8_t smem[Tile<D>::kLds + 4 * kScannedBlocks * 8];                   \
     attention_entry_full<D, C, S, R, B, K, G, F16>(smem, SVODK_FULL_ARGS);                                            \
   }
-// The instantiations the library's own dispatch reaches: a cache excludes per-row ranges; grouped
-// tiles take neither a causal mask nor ranges.
+// The instantiations the library's own dispatch reaches: grouped tiles take neither a causal mask nor
+// ranges.
 #define SVODK_FULL_SPLITS(D, T, F16, C, R, B, K, G) \
   SVODK_FULL_ENTRY(D, T, F16, C, 0, R, B, K, G) SVODK_FULL_ENTRY(D, T, F16, C, 1, R, B, K, G)
 #define SVODK_FULL_TILES(D, T, F16, R, B, K)                                                  \
@@ -1962,7 +1964,8 @@ __device__ __forceinline__ void attention_entry_full(uint8_t *smem, SVODK_FULL_P
   SVODK_FULL_TILES(D, T, F16, 0, 1, 0) SVODK_FULL_SPLITS(D, T, F16, 0, 0, 1, 0, 1)           \
   SVODK_FULL_TILES(D, T, F16, 1, 0, 0) SVODK_FULL_TILES(D, T, F16, 1, 1, 0)                   \
   SVODK_FULL_TILES(D, T, F16, 0, 0, 1) SVODK_FULL_SPLITS(D, T, F16, 0, 0, 0, 1, 1)           \
-  SVODK_FULL_TILES(D, T, F16, 0, 1, 1) SVODK_FULL_SPLITS(D, T, F16, 0, 0, 1, 1, 1)
+  SVODK_FULL_TILES(D, T, F16, 0, 1, 1) SVODK_FULL_SPLITS(D, T, F16, 0, 0, 1, 1, 1)           \
+  SVODK_FULL_TILES(D, T, F16, 1, 0, 1) SVODK_FULL_TILES(D, T, F16, 1, 1, 1)
 
 #if defined(SVODK_HEAD)  // one head size's whole family a file
 #if SVODK_HEAD == 32

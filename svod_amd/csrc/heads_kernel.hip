@@ -250,10 +250,16 @@ __device__ __forceinline__ void heads_entry(const uint16_t *qkv, const uint16_t 
     heads_entry<D, F16>(qkv, q_w, k_w, cos_t, sin_t, q, k, v, rows, t, heads, kv_heads, eps_bits, rope);              \
   }
 
+SVODK_HEADS_ENTRY(svodk_heads_d16_bf16, 16, false)
+SVODK_HEADS_ENTRY(svodk_heads_d32_bf16, 32, false)
 SVODK_HEADS_ENTRY(svodk_heads_d64_bf16, 64, false)
 SVODK_HEADS_ENTRY(svodk_heads_d128_bf16, 128, false)
+SVODK_HEADS_ENTRY(svodk_heads_d256_bf16, 256, false)
+SVODK_HEADS_ENTRY(svodk_heads_d16_f16, 16, true)
+SVODK_HEADS_ENTRY(svodk_heads_d32_f16, 32, true)
 SVODK_HEADS_ENTRY(svodk_heads_d64_f16, 64, true)
 SVODK_HEADS_ENTRY(svodk_heads_d128_f16, 128, true)
+SVODK_HEADS_ENTRY(svodk_heads_d256_f16, 256, true)
 #undef SVODK_HEADS_ENTRY
 
 }  // namespace

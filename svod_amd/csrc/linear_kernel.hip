@@ -362,6 +362,7 @@ __device__ __forceinline__ void linear_body(uint8_t *smem, const uint16_t *__res
 }
 #endif  // __HIP_DEVICE_COMPILE__
 
+#if !defined(SVODK_CODE_OBJECT)  // the library's kernel and its launch: not part of a code object build
 template <bool F16, int HD>
 __global__ __launch_bounds__(kWaves * 64, 1) void linear_kernel(const uint16_t *__restrict__ x, const uint16_t *__restrict__ w,
                                                                 const uint16_t *__restrict__ bias,
@@ -404,7 +405,50 @@ hipError_t launch(const LinearArgs &a, hipStream_t stream) {
 }
 
 }  // namespace
+#else  // SVODK_CODE_OBJECT
+// The same program as kernels for a loader that takes a code object and a flat argument record
+// (device/src/amd/program.rs:403-414, 655-675; device/src/hcq.rs:1262-1285): buffers first, then 4-byte
+// scalars, nothing hidden, static LDS, no launch geometry from the dispatch packet.
+// Parameters follow the reference GEMM's order (tk/src/kernels/gemm.rs:604-645: the operands, the bias, the
+// rotary tables, the output): x, w, bias (address 0: none), cos, sin (unread by the kernels that do not turn),
+// y, then rows (batch * seq), n, k, seq, heads (the first heads * head size columns are turned).
+// Launch: ceil(rows / 256) * ceil(n / 256) workgroups, rounded up to a multiple of 8, of 512 threads
+// (`workgroups` in the manifest); rows < 2^31, n a multiple of 8, k a multiple of 32 are the caller's checks.
+template <bool F16, int HD>
+__device__ __forceinline__ void linear_entry(uint8_t *smem, const uint16_t *x, const uint16_t *w, const uint16_t *bias,
+                                             const uint16_t *cos_t, const uint16_t *sin_t, uint16_t *y, int32_t rows,
+                                             int32_t n, int32_t k, int32_t seq, int32_t heads) {
+  if (rows <= 0 || n <= 0 || k <= 0) return;
+  const uint32_t tiles_m = ((uint32_t)rows + kBm - 1) / kBm, tiles_n = ((uint32_t)n + kBn - 1) / kBn;
+  const uint32_t tiles = tiles_m * tiles_n;
+  // The library's launch geometry (see launch below in the library build): bands of row tiles per XCD
+  // where every XCD gets at least two, else runs of tiles.
+  const uint32_t band = tiles_m >= 2 * kXcds ? (tiles_m + kXcds - 1) / kXcds : 0;
+  const uint32_t per_xcd = band > 0 ? band * tiles_n : (tiles + kXcds - 1) / kXcds;
+  linear_body<F16, HD>(smem, x, w, bias, cos_t, sin_t, y, (int64_t)rows, n, k, seq > 0 ? seq : 1, heads, tiles_n, tiles,
+                       per_xcd, band);
+}
 
+#define SVODK_LINEAR_ENTRY(NAME, F16, HD)                                                                             \
+  extern "C" __global__ __launch_bounds__(kWaves * 64, 1) void NAME(                                                  \
+      const uint16_t *__restrict__ x, const uint16_t *__restrict__ w, const uint16_t *__restrict__ bias,              \
+      const uint16_t *__restrict__ cos_t, const uint16_t *__restrict__ sin_t, uint16_t *__restrict__ y, int32_t rows, \
+      int32_t n, int32_t k, int32_t seq, int32_t heads) {                                                             \
+    __shared__ __attribute__((aligned(1024))) uint8_t smem[kLds];                                                     \
+    linear_entry<F16, HD>(smem, x, w, bias, cos_t, sin_t, y, rows, n, k, seq, heads);                                 \
+  }
+SVODK_LINEAR_ENTRY(svodk_linear_bf16, false, 0)
+SVODK_LINEAR_ENTRY(svodk_linear_rope64_bf16, false, 64)
+SVODK_LINEAR_ENTRY(svodk_linear_rope128_bf16, false, 128)
+SVODK_LINEAR_ENTRY(svodk_linear_f16, true, 0)
+SVODK_LINEAR_ENTRY(svodk_linear_rope64_f16, true, 64)
+SVODK_LINEAR_ENTRY(svodk_linear_rope128_f16, true, 128)
+#undef SVODK_LINEAR_ENTRY
+}  // namespace
+}  // namespace svodk
+#endif  // SVODK_CODE_OBJECT
+
+#if !defined(SVODK_CODE_OBJECT)
 // A fill's lanes address their rows with 32-bit byte offsets from the descriptor's base: 8 rows of 2 k bytes,
 // and the stage's place along them.
 bool linear_supports(int64_t n, int64_t k) { return n > 0 && n % 8 == 0 && k >= 32 && k % 32 == 0 && k <= (1 << 25); }
@@ -421,3 +465,4 @@ hipError_t launch_linear(const LinearArgs &a, hipStream_t stream) {
 }
 
 }  // namespace svodk
+#endif  // !SVODK_CODE_OBJECT

@@ -439,11 +439,8 @@ static int attend(const svodk_tensor *q, const svodk_tensor *k, const svodk_tens
   if (why != 0) return ran_graph(op, why);
   // Options the reference's kernel holds and this library's does not: no
   // config here holds them (the reference's own use of Fallback::Config, L210-214).
-  // L209-214: no config holds more appended rows than a key block; and this library has no
-  // kernel for a cache under per-row key ranges.
+  // L209-214: no config holds more appended rows than a key block.
   if (appended > 64) return ran_graph(op, SVODK_GRAPH_CONFIG);
-  if (cache != nullptr && (opts->has_window || opts->has_chunk || opts->seg_start != nullptr))
-    return ran_graph(op, SVODK_GRAPH_CONFIG);
   if (opts->has_window && (opts->window_left < 0 || opts->window_right < 0))
     return fail(SVODK_ERR_ARGUMENT, "%s: a negative window reach", op);
   // Chunk { size, left, right } of tk/src/ops/attention.rs:39-50: usize fields, a size of at least 1.

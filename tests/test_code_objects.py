@@ -41,8 +41,9 @@ def test_the_record_is_packed_as_the_loader_packs_it():
 
 def test_every_kernel_meets_the_loaders_conditions(built):
     table = co.entries()
-    assert len(table) == 60 + 5 * 2 * 32 + 10  # the short records, every form of every head size and type, the merges
-    assert len(list(co.full_forms())) == 32
+    # the short records (attention 32, prologue 10, norms 24, projection 6), every form of every head size and type, the merges
+    assert len(table) == 72 + 5 * 2 * 40 + 10
+    assert len(list(co.full_forms())) == 40
     for name, e in table.items():
         kd = co.check(built[e["file"]], name, e["params"])
         assert kd.kernarg_size == co.packed_size(e["params"]), name
@@ -55,6 +56,8 @@ def test_every_kernel_meets_the_loaders_conditions(built):
             mask_words = 4 * 256 * 8 if e.get("key_mask") else 0
             wide = 64 if e["head_dim"] == 48 else e["head_dim"]  # a head of 48 takes the 64-wide tile
             assert kd.group_segment_fixed_size == 2 * 2 * 64 * wide * 2 + mask_words, name
+        elif e["op"] == "linear":
+            assert kd.group_segment_fixed_size == 2 * 2 * 256 * 64 * 2, name  # two stages of a W and an X tile of 64 k-columns
         else:
             assert kd.group_segment_fixed_size == 0, name
 

@@ -133,11 +133,56 @@ def test_what_the_cache_has_no_kernel_for_keeps_the_graph(device):
     ints = lambda a: torch.tensor(a, dtype=torch.int32, device=device)
     g = Lcg(3)
     many = (dev(g.bf16((B, 65, h, d))), dev(g.bf16((B, 65, h, d))))
-    for opts in (Attn(keys=KeyMask.lens(ints(lens)), cache=Cache(h, h, ints(row_map), appended=many)),
-                 Attn(keys=KeyMask.lens(ints(lens)), cache=Cache(h, h, ints(row_map)), window=(10, 0))):
+    for opts in (Attn(keys=KeyMask.lens(ints(lens)), cache=Cache(h, h, ints(row_map), appended=many)),):
         with pytest.raises(svod_amd.GraphFallback) as e:
             svod_amd.attention(dev(q), dev(k), dev(v), opts)
         assert e.value.why == svod_amd.Fallback.Config
+
+
+# A cache under per-row key ranges: Attn allows every combination (tk/src/ops/attention.rs:60-86); the ranges
+# hide cached keys only and the appended rows answer to their own count (tk/src/test/unit/attention.rs:138-141).
+# (name, [t, d, h, tk], masks, appended, counted, biased, splits)
+RANGED = [
+    ("a causal window over a cache", [96, 64, 4, 200], dict(causal=True, window=(40, 0)), 0, False, False, None),
+    ("a window, eight appended rows", [8, 64, 4, 300], dict(window=(100, 150)), 8, True, False, None),
+    ("chunks of 16 behind a streaming chunk of queries, d 128", [16, 128, 4, 333], dict(chunk=(16, 4, 0)), 16, True, False, None),
+    ("segment starts, biased", [40, 64, 4, 128], dict(seg=20), 3, False, True, None),
+    ("every mask at once, d 48", [64, 48, 4, 128], dict(causal=True, window=(50, 0), chunk=(32, 3, 0), seg=40), 8, True, False, None),
+    ("a window with named splits runs the splits", [4, 64, 4, 640], dict(window=(600, 600)), 4, True, False, 2),
+]
+
+
+@pytest.mark.parametrize("name,dims,masks,appended,counted,biased,splits", RANGED, ids=[c[0] for c in RANGED])
+def test_a_cache_under_per_row_ranges(device, name, dims, masks, appended, counted, biased, splits):
+    t, d, h, tk = dims
+    q, k, v, k_app, v_app, bias, lens, row_map, seen = operands(t, d, h, tk, max(appended, 1))
+    lens = np.array([tk, 1, 37, tk - 1, 0])
+    masks = dict(masks)
+    seg = None
+    if "seg" in masks:
+        n = masks.pop("seg")
+        seg = np.tile(np.arange(t) - np.arange(t) % n, (B, 1))
+    if appended == 0:
+        bias = np.ascontiguousarray(bias[..., :tk])
+    ints = lambda a: torch.from_numpy(np.asarray(a)).to(torch.int32).to(device)
+    app = (bf16_tensor(k_app, device), bf16_tensor(v_app, device)) if appended else None
+    cache = Cache(head_start=h, kv_heads=h, row_map=ints(row_map), appended=app,
+                  app_lens=ints(seen) if counted and appended else None)
+    opts = Attn(causal=masks.get("causal", False), window=masks.get("window"), chunk=masks.get("chunk"),
+                seg_start=ints(seg) if seg is not None else None, keys=KeyMask.lens(ints(lens)), cache=cache,
+                splits=splits, bias=bf16_tensor(bias, device) if biased else None)
+    got = svod_amd.attention(bf16_tensor(q, device), bf16_tensor(k, device), bf16_tensor(v, device), opts)
+    torch.cuda.synchronize()
+    assert svod_amd.chosen().startswith('Kernel { op: "attention"'), svod_amd.chosen()
+    p = oracle.AttnProblem(q, k, v, causal=masks.get("causal", False), window=masks.get("window"), chunk=masks.get("chunk"),
+                           seg_start=seg, key_lens=lens, bias=bias if biased else None,
+                           cache=oracle.Cache(h, h, row_map, (k_app, v_app) if appended else None,
+                                              seen if counted and appended else None))
+    direct = oracle.attention_direct(p)
+    program = oracle.attention_flash(p, bq=128, bkv=64, splits=min(splits or 1, (tk + 63) // 64))
+    assert_bf16_parity(name, to_np(got), direct, program)
+    # Rows no key reaches (a lane without cached keys and without visible appended rows) are zeros.
+    assert np.isfinite(to_np(got)).all()
 
 
 @pytest.mark.parametrize("splits", [None, 4], ids=["whole", "a decoder step over four splits"])

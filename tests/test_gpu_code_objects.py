@@ -124,8 +124,10 @@ def test_key_mask_code_object_equals_the_library(device, runtime, d, causal, f16
 
 
 @pytest.mark.parametrize("d,f16,rope,norms", [(128, False, 1, True), (64, False, 2, True), (128, True, 1, False),
-                                              (64, True, 0, True)],
-                         ids=["d 128, shared table", "d 64, a table row per token", "f16 without norms", "f16 without rope"])
+                                              (64, True, 0, True), (16, False, 1, True), (32, True, 2, True),
+                                              (256, False, 1, True)],
+                         ids=["d 128, shared table", "d 64, a table row per token", "f16 without norms", "f16 without rope",
+                              "d 16", "d 32 f16, a table row per token", "d 256"])
 def test_prologue_code_object_equals_the_library(device, runtime, d, f16, rope, norms):
     b, t, h, hkv = 2, 37, 4, 2
     g = Lcg(7)
@@ -284,4 +286,29 @@ def test_full_kernel_reads_a_fused_projection_in_place(device, runtime):
                       kv_row_elems=row)
     rec["q"], rec["k"], rec["v"] = x.data_ptr(), x.data_ptr() + h * d * 2, x.data_ptr() + (h + hkv) * d * 2
     runtime.launch(co.full_name(d, "bf16", 1, 0, 0, 0, 0, 0), rec)
+    assert np.array_equal(bits(got), bits(want))
+
+
+@pytest.mark.parametrize("turn,f16,biased,shape", [(0, False, True, (3, 100, 96, 520)), (128, False, False, (2, 300, 256, 1024)),
+                                                  (64, True, True, (2, 70, 64, 384)), (128, False, True, (17, 256, 1024, 512))],
+                         ids=["plain with a bias, ragged tile edges", "24 of 32 heads of 128 turned",
+                              "f16, heads of 64 turned, a bias", "17 row tiles: bands of row tiles per XCD"])
+def test_linear_code_object_equals_the_library(device, runtime, turn, f16, biased, shape):
+    """The projection GEMM with its rope epilogue from the code object's bytes (tk/src/kernels/gemm.rs:604-716)."""
+    from svod_amd import Linear, Rotary
+    b, t, k, n = shape
+    g = Lcg(13)
+    x = tensor(g.bf16((b, t, k)), device, f16)
+    w = tensor(g.bf16((n, k), mul=0.125), device, f16)
+    bias = tensor(g.bf16((n,)), device, f16) if biased else None
+    heads = (n // turn) * 3 // 4 if turn else 0
+    cos = sin = None
+    if turn:
+        cos, sin = (tensor(g.bf16((1, t, 1, turn // 2)), device, f16) for _ in range(2))
+    want = svod_amd.linear(x, w, Linear(bias=bias, rope=Rotary(cos, sin, heads, turn) if turn else None))
+    got = torch.full_like(want, 7.0)
+    name = "svodk_linear_" + (f"rope{turn}_" if turn else "") + ("f16" if f16 else "bf16")
+    runtime.launch(name, {"x": x.data_ptr(), "w": w.data_ptr(), "bias": bias.data_ptr() if biased else 0,
+                          "cos": cos.data_ptr() if turn else 0, "sin": sin.data_ptr() if turn else 0, "y": got.data_ptr(),
+                          "rows": b * t, "n": n, "k": k, "seq": t, "heads": heads})
     assert np.array_equal(bits(got), bits(want))

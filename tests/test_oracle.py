@@ -634,3 +634,30 @@ def test_the_kernels_linear_arithmetic_is_within_the_references_tolerance(b, t, 
     want = oracle.linear_direct(x, w, bv if bias else None, rope)
     assert np.all(np.abs(got - want) <= 2e-2 * np.maximum(np.abs(want), 1.0))
     assert np.array_equal(got, oracle.round_bf16(got))
+
+
+def test_appended_rows_answer_to_their_count_alone():
+    """tk/src/test/unit/attention.rs:138-141: `if j >= s.tk { return j - s.tk >= seen; }` comes before every other
+    arm of hidden(j), so a causal mask, a window, a chunk mask and segment starts hide cached keys only.  The
+    direct softmax against loops written from that rule, and the tile program against the direct softmax."""
+    rng = np.random.default_rng(3)
+    b, t, tk, h, d, n = 2, 6, 40, 2, 16, 3
+    rb = lambda *s: oracle.round_bf16(rng.standard_normal(s).astype(np.float32))
+    q, k, v, k_app, v_app = rb(b, t, h, d), rb(b, tk, h, d), rb(b, tk, h, d), rb(b, n, h, d), rb(b, n, h, d)
+    lens, seen = np.array([40, 7]), np.array([3, 1])
+    win = (4, 0)
+    p = oracle.AttnProblem(q, k, v, causal=True, window=win, key_lens=lens,
+                           cache=oracle.Cache(0, h, None, (k_app, v_app), seen))
+    want = np.zeros((b, t, h, d))
+    for bi in range(b):
+        for hi in range(h):
+            for i in range(t):
+                keys = [(k[bi, j, hi], v[bi, j, hi]) for j in range(tk)
+                        if j < lens[bi] and j <= i and j + win[0] >= i and j <= i + win[1]]
+                keys += [(k_app[bi, j, hi], v_app[bi, j, hi]) for j in range(seen[bi])]
+                s = np.array([float(np.dot(q[bi, i, hi].astype(np.float64), kk.astype(np.float64))) for kk, _ in keys]) / 4.0
+                w = np.exp(s - s.max())
+                want[bi, i, hi] = (w[:, None] * np.array([vv for _, vv in keys], dtype=np.float64)).sum(0) / w.sum()
+    got = oracle.attention_direct(p)
+    assert np.abs(got - want).max() < 1e-12
+    assert np.abs(oracle.attention_flash(p, 64, 64) - want).max() < 2e-2

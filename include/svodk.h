@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define SVODK_ABI_VERSION 5
+#define SVODK_ABI_VERSION 6
 
 /* Element types of a tensor descriptor. */
 typedef enum svodk_dtype {
@@ -255,11 +255,19 @@ typedef struct svodk_linear_opts {
   float scale;
   const svodk_rotary *rope; /* or NULL */
   int32_t batch_live;       /* as in svodk_attn */
+  /* Linear::into (tk/src/ops/linear.rs:40-42), the `out=` of a fused projection: with has_into the
+   * call's `out` is the wider tensor [lead..., C] and the result is stored into its channels
+   * into_at .. into_at + N; the other channels are left as they are.  into_at + N <= C
+   * (tk/src/ops/mod.rs:459-477).  The kernel stores 16 bytes a lane: a window whose start or whose
+   * row is not a multiple of 8 elements answers SVODK_GRAPH_CONFIG (the reference then runs the
+   * plain kernel and lets the graph store the window, :96-103). */
+  int32_t has_into;
+  int64_t into_at;
 } svodk_linear_opts;
 
 /*
  * ops::linear (tk/src/ops/linear.rs:60-231) for a fused projection: x [B, T, K] . w [N, K]^T
- * (+ bias) -> out [B, T, N], the rope applied in the GEMM's store (tk/src/kernels/gemm.rs:604-645,
+ * (+ bias) -> out [B, T, N] (or channels of a wider out, see has_into), the rope applied in the GEMM's store (tk/src/kernels/gemm.rs:604-645,
  * 666-716): a model without QK norms gets its rotated queries and keys and its plain values from the
  * projection itself and needs no svodk_heads pass (svodk_attention_packed then reads `out` in place).
  * f32 accumulators, one rounding at the store.  N a multiple of 8 (tk/src/ops/shape.rs:133-136);

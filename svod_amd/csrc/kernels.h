@@ -50,7 +50,8 @@ struct LinearArgs {
   const void *bias;  // [n] or null
   const void *cos;   // [seq, head_dim / 2] or null: no turn
   const void *sin;
-  void *y;           // [rows, n]
+  void *y;           // [rows, n], or the window's first element in a wider output
+  int64_t y_ld;      // elements from an output row to the next: n, or the wider output's channels
   int64_t rows;      // live batches * seq
   int32_t n, k;
   int32_t seq;       // row r is the token at position r % seq

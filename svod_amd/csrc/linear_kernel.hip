@@ -112,9 +112,9 @@ __device__ __forceinline__ void load4(const uint16_t *p, float (&out)[4]) {
 template <bool F16, int HD>
 __device__ __forceinline__ void linear_body(uint8_t *smem, const uint16_t *__restrict__ x, const uint16_t *__restrict__ w,
                                             const uint16_t *__restrict__ bias, const uint16_t *__restrict__ cos_t,
-                                            const uint16_t *__restrict__ sin_t, uint16_t *__restrict__ y, int64_t rows,
-                                            int32_t n, int32_t k, int32_t seq, int32_t heads, uint32_t tiles_n,
-                                            uint32_t tiles, uint32_t per_xcd, uint32_t band) {
+                                            const uint16_t *__restrict__ sin_t, uint16_t *__restrict__ y, int64_t y_ld,
+                                            int64_t rows, int32_t n, int32_t k, int32_t seq, int32_t heads,
+                                            uint32_t tiles_n, uint32_t tiles, uint32_t per_xcd, uint32_t band) {
   const int tid = __builtin_amdgcn_workitem_id_x();
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -356,7 +356,7 @@ __device__ __forceinline__ void linear_body(uint8_t *smem, const uint16_t *__res
       const u32x4 out = *reinterpret_cast<const u32x4 *>(stage + r * kOutPitch + ochunk * 16);
       const int64_t row = m0 + wave_m * 64 + rb * 32 + r;
       // Streaming stores: the output is not read again here, and left out of L2 it does not push the operands out.
-      if (row < rows && col < n) __builtin_nontemporal_store(out, reinterpret_cast<u32x4 *>(y + row * (int64_t)n + col));
+      if (row < rows && col < n) __builtin_nontemporal_store(out, reinterpret_cast<u32x4 *>(y + row * y_ld + col));
     }
   }
 }
@@ -368,12 +368,13 @@ __global__ __launch_bounds__(kWaves * 64, 1) void linear_kernel(const uint16_t *
                                                                 const uint16_t *__restrict__ bias,
                                                                 const uint16_t *__restrict__ cos_t,
                                                                 const uint16_t *__restrict__ sin_t, uint16_t *__restrict__ y,
-                                                                int64_t rows, int32_t n, int32_t k, int32_t seq, int32_t heads,
+                                                                int64_t y_ld, int64_t rows, int32_t n, int32_t k, int32_t seq,
+                                                                int32_t heads,
                                                                 uint32_t tiles_n, uint32_t tiles, uint32_t per_xcd,
                                                                 uint32_t band) {
 #if defined(__HIP_DEVICE_COMPILE__)
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
-  linear_body<F16, HD>(smem, x, w, bias, cos_t, sin_t, y, rows, n, k, seq, heads, tiles_n, tiles, per_xcd, band);
+  linear_body<F16, HD>(smem, x, w, bias, cos_t, sin_t, y, y_ld, rows, n, k, seq, heads, tiles_n, tiles, per_xcd, band);
 #endif
 }
 
@@ -399,7 +400,8 @@ hipError_t launch(const LinearArgs &a, hipStream_t stream) {
   }
   hipLaunchKernelGGL(kernel, dim3((uint32_t)(per_xcd * kXcds)), dim3(kWaves * 64), kLds, stream, (const uint16_t *)a.x,
                      (const uint16_t *)a.w, (const uint16_t *)a.bias, (const uint16_t *)a.cos, (const uint16_t *)a.sin,
-                     (uint16_t *)a.y, a.rows, a.n, a.k, a.seq, a.heads, (uint32_t)tiles_n, (uint32_t)tiles,
+                     (uint16_t *)a.y, a.y_ld > 0 ? a.y_ld : (int64_t)a.n, a.rows, a.n, a.k, a.seq, a.heads, (uint32_t)tiles_n,
+                     (uint32_t)tiles,
                      (uint32_t)per_xcd, (uint32_t)band);
   return hipGetLastError();
 }
@@ -425,8 +427,8 @@ __device__ __forceinline__ void linear_entry(uint8_t *smem, const uint16_t *x, c
   // where every XCD gets at least two, else runs of tiles.
   const uint32_t band = tiles_m >= 2 * kXcds ? (tiles_m + kXcds - 1) / kXcds : 0;
   const uint32_t per_xcd = band > 0 ? band * tiles_n : (tiles + kXcds - 1) / kXcds;
-  linear_body<F16, HD>(smem, x, w, bias, cos_t, sin_t, y, (int64_t)rows, n, k, seq > 0 ? seq : 1, heads, tiles_n, tiles,
-                       per_xcd, band);
+  linear_body<F16, HD>(smem, x, w, bias, cos_t, sin_t, y, (int64_t)n, (int64_t)rows, n, k, seq > 0 ? seq : 1, heads, tiles_n,
+                       tiles, per_xcd, band);
 }
 
 #define SVODK_LINEAR_ENTRY(NAME, F16, HD)                                                                             \

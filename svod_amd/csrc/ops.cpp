@@ -1017,7 +1017,11 @@ int svodk_linear(const svodk_tensor *x, const svodk_tensor *w, const svodk_linea
                   (long long)w->shape[0]);
   }
   // The output the reference op allocates itself (L203-206): [lead..., N] of x's type.
-  bool out_fits = out->rank == x->rank && out->shape[out->rank - 1] == n;
+  // With `into` (L40-42, tk/src/ops/mod.rs:459-477) it is the caller's wider tensor [lead..., C], channels
+  // into_at .. into_at + N of which take the result.
+  const int64_t out_ld = out->rank >= 1 ? out->shape[out->rank - 1] : 0;
+  bool out_fits = out->rank == x->rank &&
+                  (opts->has_into ? (opts->into_at >= 0 && opts->into_at + n <= out_ld) : out_ld == n);
   for (int i = 0; out_fits && i + 1 < x->rank; i++) out_fits = out->shape[i] == x->shape[i];
   // L79-82: the residual has the output's shape.
   if (opts->residual != nullptr) {
@@ -1048,6 +1052,9 @@ int svodk_linear(const svodk_tensor *x, const svodk_tensor *w, const svodk_linea
                     (long long)x->shape[1], rope->head_dim / 2);
     }
   }
+  if (!out_fits && opts->has_into)
+    return fail(SVODK_ERR_SHAPE, "%s: into has shape %s, expected [lead..., %lld] widened to hold channels %lld.. past the last axis",
+                op, fmt_shape(out).c_str(), (long long)n, (long long)opts->into_at);
   if (!out_fits)
     return fail(SVODK_ERR_SHAPE, "%s: out has shape %s, expected [lead..., %lld]", op, fmt_shape(out).c_str(), (long long)n);
   if (out->dtype != x->dtype)
@@ -1075,6 +1082,8 @@ int svodk_linear(const svodk_tensor *x, const svodk_tensor *w, const svodk_linea
     // L176-184: no tile turns heads of this size.
     if (!svodk::linear_turns(rope->head_dim)) return ran_graph(op, SVODK_GRAPH_CONFIG);
   }
+  // tk/src/ops/mod.rs:475-476: a window the kernel's 16-byte stores cannot land in is the graph's to store.
+  if (opts->has_into && (opts->into_at % 8 != 0 || out_ld % 8 != 0)) return ran_graph(op, SVODK_GRAPH_CONFIG);
   int64_t lead = 1;
   for (int i = 1; i + 1 < x->rank; i++) lead *= x->shape[i];
   const int64_t live = x->rank > 1 ? (opts->batch_live > 0 ? opts->batch_live : cap) : 1;
@@ -1102,7 +1111,8 @@ int svodk_linear(const svodk_tensor *x, const svodk_tensor *w, const svodk_linea
   a.bias = opts->bias ? opts->bias->data : nullptr;
   a.cos = rope ? rope->cos->data : nullptr;
   a.sin = rope ? rope->sin->data : nullptr;
-  a.y = out->data;
+  a.y = (uint16_t *)out->data + (opts->has_into ? opts->into_at : 0);
+  a.y_ld = opts->has_into ? out_ld : n;
   a.rows = rows;
   a.n = (int32_t)n;
   a.k = (int32_t)k;
@@ -1110,8 +1120,8 @@ int svodk_linear(const svodk_tensor *x, const svodk_tensor *w, const svodk_linea
   a.heads = rope ? rope->heads : 0;
   a.head_dim = rope ? rope->head_dim : 0;
   a.f16 = x->dtype == SVODK_F16;
-  ran(op, "gemm", rope ? "GemmCfg { bm: 256, bn: 256, bk: 32, stages: 4, warps: [4, 2], epilogue: { bias, rope } }"
-                       : "GemmCfg { bm: 256, bn: 256, bk: 32, stages: 4, warps: [4, 2], epilogue: { bias } }");
+  ran(op, "gemm", rope ? "GemmCfg { bm: 256, bn: 256, bk: 64, stages: 2, warps: [4, 2], epilogue: { bias, rope } }"
+                       : "GemmCfg { bm: 256, bn: 256, bk: 64, stages: 2, warps: [4, 2], epilogue: { bias } }");
   const hipError_t e = svodk::launch_linear(a, (hipStream_t)hip_stream);
   if (e != hipSuccess) return fail(SVODK_ERR_LAUNCH, "%s: %s", op, hipGetErrorString(e));
   return SVODK_KERNEL;

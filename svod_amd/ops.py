@@ -67,7 +67,8 @@ class _Rotary(ctypes.Structure):
 class _Linear(ctypes.Structure):
     _fields_ = [("bias", ctypes.POINTER(_Tensor)), ("act", ctypes.c_int32), ("gated", ctypes.c_int32),
                 ("residual", ctypes.POINTER(_Tensor)), ("has_scale", ctypes.c_int32), ("scale", ctypes.c_float),
-                ("rope", ctypes.POINTER(_Rotary)), ("batch_live", ctypes.c_int32)]
+                ("rope", ctypes.POINTER(_Rotary)), ("batch_live", ctypes.c_int32), ("has_into", ctypes.c_int32),
+                ("into_at", ctypes.c_int64)]
 
 
 _lib: Optional[ctypes.CDLL] = None
@@ -438,7 +439,8 @@ class Rotary:
 
 @dataclass
 class Linear:
-    """``Linear`` of tk/src/ops/linear.rs:24-45 (without ``into``: the caller's ``out`` stands for it)."""
+    """``Linear`` of tk/src/ops/linear.rs:24-45.  ``into = (tensor [lead..., C], at)`` stores the result into the
+    tensor's channels ``at .. at + N`` and returns the tensor."""
 
     bias: Optional[torch.Tensor] = None
     act: Act = Act.NONE
@@ -447,6 +449,7 @@ class Linear:
     scale: Optional[float] = None
     rope: Optional[Rotary] = None
     batch_live: Optional[int] = None
+    into: Optional[Tuple[torch.Tensor, int]] = None
 
 
 def linear(x: torch.Tensor, w: torch.Tensor, opts: Optional[Linear] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -454,11 +457,14 @@ def linear(x: torch.Tensor, w: torch.Tensor, opts: Optional[Linear] = None, out:
     GEMM's store (tk/src/ops/linear.rs:60-63)."""
     opts = opts or Linear()
     lib = load_library()
+    keep: list = []
+    o = _Linear()
+    if opts.into is not None:
+        out, at = opts.into
+        o.has_into, o.into_at = 1, int(at)
     if out is None:
         n = w.shape[0] // 2 if opts.gated else w.shape[0]
         out = _fresh((*x.shape[:-1], n), x.dtype, x.device)
-    keep: list = []
-    o = _Linear()
     o.bias, o.residual = _ref(keep, opts.bias), _ref(keep, opts.residual)
     o.act, o.gated = int(opts.act), int(opts.gated)
     if opts.scale is not None:

@@ -142,3 +142,26 @@ def test_the_turned_projection_feeds_attention_in_place(device):
     # The two differ by one more rounding of q and k (the prologue rotates rounded values): within the op's bar.
     assert max_abs(to_np(a), to_np(bref)) < 2e-2
     assert np.array_equal(bits(fused[:, :, (h + hkv) * d:]), bits(plain[:, :, (h + hkv) * d:]))  # values: as they are
+
+
+def test_into_stores_a_window_of_a_wider_output(device):
+    """Linear::into (tk/src/ops/linear.rs:40-42, tk/src/ops/mod.rs:459-477): the result lands in channels
+    at .. at + N of the caller's [lead..., C] tensor, bit-equal to the plain call's, the rest untouched; a window
+    the 16-byte stores cannot land in keeps the graph; one that does not fit is a shape error."""
+    lead, k, n, c, at = (2, 70), 96, 3 * 64, 512, 128
+    x, w, bv = case(lead, k, n)
+    (cos, sin), (cos_d, sin_d) = tables(lead[1], 64, device)
+    opts = dict(bias=bf16_tensor(bv, device), rope=Rotary(cos_d, sin_d, 2, 64))
+    want = svod_amd.linear(bf16_tensor(x, device), bf16_tensor(w, device), Linear(**opts))
+    wide = torch.full((*lead, c), 3.0, dtype=torch.bfloat16, device=device)
+    got = svod_amd.linear(bf16_tensor(x, device), bf16_tensor(w, device), Linear(into=(wide, at), **opts))
+    torch.cuda.synchronize()
+    assert got is wide and svod_amd.chosen().startswith('Kernel { op: "linear"')
+    assert np.array_equal(bits(wide[..., at:at + n].contiguous()), bits(want))
+    assert bool((wide[..., :at] == 3.0).all()) and bool((wide[..., at + n:] == 3.0).all())
+    with pytest.raises(GraphFallback) as e:
+        svod_amd.linear(bf16_tensor(x, device), bf16_tensor(w, device), Linear(into=(wide, 4), **opts))
+    assert e.value.why == Fallback.Config
+    with pytest.raises(svod_amd.OpError) as e:
+        svod_amd.linear(bf16_tensor(x, device), bf16_tensor(w, device), Linear(into=(wide, c - n + 8), **opts))
+    assert e.value.kind == "Shape"

@@ -1191,18 +1191,26 @@ __device__ __forceinline__ void flash_fwd_body(
   }
   // ---- out = o / (l == 0 ? 1 : l), bounded store (L892-898, L974-980).
   const float inv = 1.0f / (l_tot == 0.0f ? 1.0f : l_tot);
-  if (q_ok) {
-    uint16_t *o_ptr = o + ((int64_t)b * t + q_row) * o_row_stride + (int64_t)q_head * D + 4 * w.g;
+  // A lane holds four consecutive columns of its row per register quad and its partner in the other half-wave
+  // the next four: the halves trade quads (v_permlane32_swap), so that each lane stores eight columns, 128 bits
+  // at a time: the lower half the even runs of eight, the upper half the odd ones.
+  uint16_t *o_ptr = o + ((int64_t)b * t + q_row) * o_row_stride + (int64_t)q_head * D + 8 * w.g;
 #pragma unroll
-    for (int db = 0; db < DB; db++) {
+  for (int db = 0; db < DB; db++) {
 #pragma unroll
-      for (int c = 0; c < 4; c++) {
-        if (32 * db + 8 * c >= D) continue;  // the tile's columns past the head
-        u32x2 x;
-        x[0] = pack2<F16>(w.acc[db][4 * c] * inv, w.acc[db][4 * c + 1] * inv);
-        x[1] = pack2<F16>(w.acc[db][4 * c + 2] * inv, w.acc[db][4 * c + 3] * inv);
-        *reinterpret_cast<u32x2 *>(o_ptr + 32 * db + 8 * c) = x;
+    for (int c = 0; c < 4; c += 2) {
+      if (32 * db + 8 * c >= D) continue;  // the tile's columns past the head (a head of 48: its last 16)
+      uint32_t x[2], y[2];
+#pragma unroll
+      for (int e = 0; e < 2; e++) {
+        x[e] = pack2<F16>(w.acc[db][4 * c + 2 * e] * inv, w.acc[db][4 * c + 2 * e + 1] * inv);
+        y[e] = pack2<F16>(w.acc[db][4 * c + 4 + 2 * e] * inv, w.acc[db][4 * c + 5 + 2 * e] * inv);
       }
+      // swap(x, y): {lower: own x, upper: the partner's y}, {lower: the partner's x, upper: own y}.
+      const auto lo = __builtin_amdgcn_permlane32_swap(x[0], y[0], false, false);
+      const auto hi = __builtin_amdgcn_permlane32_swap(x[1], y[1], false, false);
+      const u32x4 out = {lo[0], hi[0], lo[1], hi[1]};
+      if (q_ok) *reinterpret_cast<u32x4 *>(o_ptr + 32 * db + 8 * c) = out;
     }
   }
 }

@@ -224,6 +224,25 @@ __device__ __forceinline__ void linear_body(uint8_t *smem, const uint16_t *__res
 #pragma unroll
       for (int rb = 0; rb < 2; rb++) acc[rb][cb] = mma<F16>(af[cb], bf[rb], acc[rb][cb]);
   };
+  // The rotary tables' rows of this tile (16 bytes a lane along the rows, kTables loads a table and lane)
+  // are asked for behind the barrier of the last stage but one: they arrive under the last stage's products
+  // and are in registers when the epilogue wants them in LDS.
+  constexpr int kHalf = (HD > 0 ? HD : 64) / 2, kTChunks = kHalf * 2 / 16, kTables = kBm * kTChunks / (kWaves * 64);
+  const bool turning = HD > 0 && n0 < heads * HD;  // the same for the whole workgroup
+  u32x4 tc[kTables], ts[kTables];
+  bool tables_in = false;
+  auto load_tables = [&]() {
+    const uint32_t pos0 = (uint32_t)(m0 % seq);
+#pragma unroll
+    for (int i = 0; i < kTables; i++) {
+      const int c = tid + i * kWaves * 64, r = c / kTChunks, ch = c % kTChunks;
+      const uint32_t pos = (pos0 + (uint32_t)r) % (uint32_t)seq;  // gemm.rs:685: the table row of the token's position
+      tc[i] = *reinterpret_cast<const u32x4 *>(cos_t + (int64_t)pos * kHalf + ch * 8);
+      ts[i] = *reinterpret_cast<const u32x4 *>(sin_t + (int64_t)pos * kHalf + ch * 8);
+    }
+    tables_in = true;
+  };
+
   // A stage is four k-steps.  Before its last one every wave makes sure its own fills of the next stage
   // have landed and its reads of this stage are back, and meets the others: behind that barrier the next
   // stage is whole and this stage's slot is free, so the fills of the stage after next go out and the next
@@ -244,9 +263,11 @@ __device__ __forceinline__ void linear_body(uint8_t *smem, const uint16_t *__res
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");  // stage s + 1 is in, stage s is read
     __syncthreads();
     fill(s + 2);
+    if (HD > 0 && turning && s == nk - 2) load_tables();
     fragments(slot ^ 1, 0, a0, b0);
     if (whole) multiply(a1, b1);
   }
+  if (HD > 0 && turning && !tables_in) load_tables();  // a k loop of one stage
   // The empty fills still in flight write LDS: they land before the workgroup's LDS is given away.
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
@@ -270,7 +291,7 @@ __device__ __forceinline__ void linear_body(uint8_t *smem, const uint16_t *__res
     }
   }
   const int turned = HD > 0 ? heads * HD : 0;
-  if (HD > 0 && n0 < turned) {  // the same for the whole workgroup
+  if (HD > 0 && turning) {
     // The head size is 64 or 128: a head's halves are whole 32-column blocks of a wave's 128 columns, the
     // partner of block cb is block cb +- nb, and a head never straddles two waves.
     constexpr int head_dim = HD > 0 ? HD : 64;
@@ -282,13 +303,12 @@ __device__ __forceinline__ void linear_body(uint8_t *smem, const uint16_t *__res
     constexpr int kPitch = half * 2 + 8, kChunks = half * 2 / 16;
     uint8_t *cos_lds = smem, *sin_lds = smem + kBm * kPitch;
     __syncthreads();  // every wave's last fragments are read and its last fills have landed
-    const uint32_t pos0 = (uint32_t)(m0 % seq);
     static_assert(2 * kBm * kPitch <= kLds, "the tables fit where the ring was");
-    for (int c = tid; c < kBm * kChunks; c += kWaves * 64) {
-      const int r = c / kChunks, ch = c % kChunks;
-      const uint32_t pos = (pos0 + (uint32_t)r) % (uint32_t)seq;  // gemm.rs:685: the table row of the token's position
-      const u32x4 vc = *reinterpret_cast<const u32x4 *>(cos_t + (int64_t)pos * half + ch * 8);
-      const u32x4 vs = *reinterpret_cast<const u32x4 *>(sin_t + (int64_t)pos * half + ch * 8);
+    static_assert(kChunks == kTChunks && half == kHalf, "the prefetch's chunks are the tables'");
+#pragma unroll
+    for (int i = 0; i < kTables; i++) {
+      const int c = tid + i * kWaves * 64, r = c / kChunks, ch = c % kChunks;
+      const u32x4 vc = tc[i], vs = ts[i];
       u32x2 *cd = reinterpret_cast<u32x2 *>(cos_lds + r * kPitch + ch * 16);
       u32x2 *sd = reinterpret_cast<u32x2 *>(sin_lds + r * kPitch + ch * 16);
       cd[0] = u32x2{vc[0], vc[1]};

@@ -168,15 +168,16 @@ __device__ __forceinline__ void linear_body(uint8_t *smem, const uint16_t *__res
     rsrc[f] = make_rsrc((const uint8_t *)base + first * row_bytes, (limit - first) * row_bytes);
     lds_at[f] = (int)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)(smem) + j * 1024;
   }
-  // k is a multiple of 32: a last stage may hold two k-steps only (what its rows' second halves fetch is the
-  // next rows' data or, past the operand, zeros: never multiplied).
+  // k is a multiple of 32: a last stage may hold two k-steps only.  The lanes that would fetch the second
+  // half of its rows (the next rows' data) then address past every descriptor's bound and land zeros.
   const int nk = (k + kBk - 1) / kBk;
   const bool short_tail = (k % kBk) != 0;
+  const bool second_half = ((place ^ ((4 * (wave & 1) + (frow >> 1)) & 7)) & 4) != 0;
   // Stage `s` of the k loop into its ring slot; past the last stage an empty descriptor (zeros land in a
   // slot nothing reads any more) keeps the count of fills in flight the same in every iteration.
   auto fill = [&](int s) {
     const int slot = (s % kStages) * kStageBytes;
-    const int voff = src + s * kRowBytes;
+    const int voff = (short_tail && s == nk - 1 && second_half) ? (int)0xfffffff0u : src + s * kRowBytes;
 #pragma unroll
     for (int f = 0; f < kFills; f++) {
       i32x4 r = rsrc[f];
@@ -210,19 +211,25 @@ __device__ __forceinline__ void linear_body(uint8_t *smem, const uint16_t *__res
 #pragma unroll
     for (int cb = 0; cb < 4; cb++) acc[rb][cb] = zero;
 
-  // Fragments of (stage slot, k-step): four of W (this wave's column blocks), two of X (its row blocks).
-  auto fragments = [&](int slot, int ks, u32x4 (&af)[4], u32x4 (&bf)[2]) {
+  // One k-step: eight products of the fragment set `set` (four of W: this wave's column blocks; two of X: its
+  // row blocks), and beside the first six of them the six fragment reads of k-step `nks` of stage slot `nslot`
+  // into the other set, so that a product's operands were asked for six to eight products earlier.  The fences
+  // keep the order: left to itself the scheduler gathers the reads in front of the products that want them.
+  u32x4 af[2][4], bf[2][2];
+  auto read_fragment = [&](int slot, int ks, int i, int set) {
     const uint8_t *st = smem + slot * kStageBytes;
-#pragma unroll
-    for (int cb = 0; cb < 4; cb++) af[cb] = *reinterpret_cast<const u32x4 *>(st + a_read[cb] + chunk_at[ks]);
-#pragma unroll
-    for (int rb = 0; rb < 2; rb++) bf[rb] = *reinterpret_cast<const u32x4 *>(st + b_read[rb] + chunk_at[ks]);
+    if (i < 2)
+      bf[set][i] = *reinterpret_cast<const u32x4 *>(st + b_read[i] + chunk_at[ks]);
+    else
+      af[set][i - 2] = *reinterpret_cast<const u32x4 *>(st + a_read[i - 2] + chunk_at[ks]);
   };
-  auto multiply = [&](const u32x4 (&af)[4], const u32x4 (&bf)[2]) {
+  auto step = [&](int set, int nslot, int nks, bool reads) {
 #pragma unroll
-    for (int cb = 0; cb < 4; cb++)
-#pragma unroll
-      for (int rb = 0; rb < 2; rb++) acc[rb][cb] = mma<F16>(af[cb], bf[rb], acc[rb][cb]);
+    for (int i = 0; i < 8; i++) {
+      acc[i & 1][i >> 1] = mma<F16>(af[set][i >> 1], bf[set][i & 1], acc[i & 1][i >> 1]);
+      if (reads && i < 6) read_fragment(nslot, nks, i, set ^ 1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
   };
   // The rotary tables' rows of this tile (16 bytes a lane along the rows, kTables loads a table and lane)
   // are asked for behind the barrier of the last stage but one: they arrive under the last stage's products
@@ -247,25 +254,20 @@ __device__ __forceinline__ void linear_body(uint8_t *smem, const uint16_t *__res
   // have landed and its reads of this stage are back, and meets the others: behind that barrier the next
   // stage is whole and this stage's slot is free, so the fills of the stage after next go out and the next
   // stage's first fragments are asked for under this stage's last products.
-  u32x4 a0[4], b0[2], a1[4], b1[2];
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kFills) : "memory");  // stage 0 is in
   __syncthreads();
-  fragments(0, 0, a0, b0);
+#pragma unroll
+  for (int i = 0; i < 6; i++) read_fragment(0, 0, i, 0);
   for (int s = 0; s < nk; s++) {
     const int slot = s & 1;
-    fragments(slot, 1, a1, b1);
-    multiply(a0, b0);
-    fragments(slot, 2, a0, b0);
-    multiply(a1, b1);
-    fragments(slot, 3, a1, b1);
-    const bool whole = !short_tail || s + 1 < nk;
-    if (whole) multiply(a0, b0);
+    step(0, slot, 1, true);
+    step(1, slot, 2, true);
+    step(0, slot, 3, true);
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");  // stage s + 1 is in, stage s is read
     __syncthreads();
     fill(s + 2);
     if (HD > 0 && turning && s == nk - 2) load_tables();
-    fragments(slot ^ 1, 0, a0, b0);
-    if (whole) multiply(a1, b1);
+    step(1, slot ^ 1, 0, true);
   }
   if (HD > 0 && turning && !tables_in) load_tables();  // a k loop of one stage
   // The empty fills still in flight write LDS: they land before the workgroup's LDS is given away.

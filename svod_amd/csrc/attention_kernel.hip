@@ -270,13 +270,14 @@ __device__ __forceinline__ void fill_tile(const Wave<D, NW, F16, FLAGS> &w, cons
   constexpr int NS = Tile<D>::sources(NW);
   static_assert((NS * NW * kRowsPer) % 16 == 0, "the swizzle repeats over a wave's fills");
   const int64_t off = (int64_t)blk * kBkv * row_bytes;
+  const i32x4 r = make_rsrc(base + off, bytes - off);
 #pragma unroll
   for (int i = 0; i < Wave<D, NW, F16, FLAGS>::CH; i++) {
-    const int64_t at = off + (int64_t)(NW * i * kRowsPer) * row_bytes;
-    const i32x4 r = make_rsrc(base + at, bytes - at);
+    int voff = src[i % NS] + (NW * i * kRowsPer) * row_bytes;
+    if constexpr (D == 48) voff = src[i % NS] == (int)0xfffffff0u ? src[i % NS] : voff;  // a chunk the row does not have
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
                  :
-                 : "s"(lds_at + (w.wave + NW * i) * 1024), "v"(src[i % NS]), "s"(r)
+                 : "s"(lds_at + (w.wave + NW * i) * 1024), "v"(voff), "s"(r)
                  : "memory");
   }
 }

@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define SVODK_ABI_VERSION 6
+#define SVODK_ABI_VERSION 7
 
 /* Element types of a tensor descriptor. */
 typedef enum svodk_dtype {
@@ -328,6 +328,16 @@ int svodk_plan_norm(int32_t has_target, const int32_t *dtypes, int32_t n_dtypes,
  */
 #define SVODK_STREAMING_SETS 256
 void svodk_tune_streaming(int32_t workgroups_per_xcd);
+/*
+ * No counterpart in the reference.  A decoder step (an attention call without causal or per-row masks or a bias
+ * whose KV heads each serve at most SVODK_DECODE_ROWS query rows, heads / kv_heads * T) streams K and V through
+ * registers past its rows instead of running 64-key tiles through LDS: such a call is bound by the bytes of K and V
+ * in flight, not by arithmetic.  `rows` = the most rows a KV head may serve for a call to go that way, 0 ..
+ * SVODK_DECODE_ROWS (the default); 0 = every call runs key tiles.  Process-wide.  Results of the two paths agree to
+ * the op's tolerance, not bit for bit: they sum in different orders.
+ */
+#define SVODK_DECODE_ROWS 4
+void svodk_tune_decode(int32_t rows);
 /* The set the next streaming launch would take, and takes it (no device work): for tests of the
  * assignment.  No counterpart in the reference. */
 uint32_t svodk_streaming_next_set(void);

@@ -24,6 +24,7 @@ from .ops import (  # noqa: F401
     attention_noalloc,
     attention_packed,
     noalloc_scratch_bytes,
+    tune_decode,
     tune_streaming,
     chosen,
     heads,

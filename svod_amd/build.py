@@ -16,7 +16,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libsvodk_gfx950.so")
 SOURCES = ["ops.cpp", "heads_kernel.hip", "attention_kernel.hip", "combine_kernel.hip", "rows_kernel.hip",
-           "linear_kernel.hip"]
+           "linear_kernel.hip", "decode_kernel.hip"]
 
 # Packed-FP32 VALU ops are switched off for device code; the host pass of hipcc
 # does not know the feature and says so, which is harmless.

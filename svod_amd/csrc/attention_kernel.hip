@@ -1813,6 +1813,9 @@ bool attention_groups(const AttnArgs &a) {
 void attention_stream_slots(int32_t slots) { g_stream_slots.store(slots, std::memory_order_relaxed); }
 
 const char *attention_config(const AttnArgs &a) {
+  if (attention_decodes(a))
+    return a.splits > 1 ? "FaCfg { rows: 4, lanes_per_key: d / 8, splits: n, core: v_dot2_f32, keys streamed through registers }"
+                        : "FaCfg { rows: 4, lanes_per_key: d / 8, splits: 1, core: v_dot2_f32, keys streamed through registers }";
   static const char *const kCfg[2][2] = {
       {"FaCfg { bq: 128, bkv: 64, stages: 2, splits: 1, forms: { raw_max, skip_rescale }, warp_rows: 32, core: "
        "mfma_f32_32x32x16_bf16 }",
@@ -1826,6 +1829,7 @@ const char *attention_config(const AttnArgs &a) {
 }
 
 hipError_t launch_attention(const AttnArgs &a, hipStream_t stream) {
+  if (attention_decodes(a)) return launch_decode(a, stream);  // a decoder step: no key tiles, a stream of K and V
   switch (a.d) {
     case 32: return launch_attention_d32(a, stream);
     case 48: return launch_attention_d48(a, stream);

@@ -138,6 +138,15 @@ bool attention_supports(int32_t d);
 // Whether launch_attention runs `a` on grouped tiles: the heads of a KV head's group side by side
 // in one query tile (a decoder step under GQA: no causal or per-row mask, group * t <= 128).
 bool attention_groups(const AttnArgs &a);
+// The decoder step's kernel (decode_kernel.hip): a call without causal or per-row masks or a bias whose (batch,
+// KV head) has at most kDecodeRows query rows (group * t) streams K and V past them in registers instead of
+// running key tiles through LDS.  launch_attention takes that path by itself; splits, caches, appended rows, key
+// lengths and key masks mean what they mean to the tile kernel.
+constexpr int kDecodeRows = 4;
+bool attention_decodes(const AttnArgs &a);
+// The most rows that path takes, 0..kDecodeRows (0: every call runs key tiles): see svodk_tune_decode.
+void attention_decode_rows(int32_t rows);
+hipError_t launch_decode(const AttnArgs &a, hipStream_t stream);
 // One head size's kernels each (launch_attention picks by AttnArgs::d).
 hipError_t launch_attention_d32(const AttnArgs &a, hipStream_t stream);
 hipError_t launch_attention_d48(const AttnArgs &a, hipStream_t stream);

@@ -694,6 +694,7 @@ int svodk_attention_packed(const svodk_tensor *qkv, int32_t heads, int32_t kv_he
 }
 
 void svodk_tune_streaming(int32_t workgroups_per_xcd) { svodk::attention_stream_slots(workgroups_per_xcd); }
+void svodk_tune_decode(int32_t rows) { svodk::attention_decode_rows(rows); }
 uint32_t svodk_streaming_next_set(void) { return svodk::next_queue_set(); }
 
 // The batch rows by descending key count, for svodk_attn.row_order (no counterpart in the reference,

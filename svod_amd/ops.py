@@ -137,6 +137,8 @@ def load_library(path: Optional[str] = None) -> ctypes.CDLL:
     lib.svodk_streaming_next_set.argtypes = []
     lib.svodk_tune_streaming.restype = None
     lib.svodk_tune_streaming.argtypes = [ctypes.c_int32]
+    lib.svodk_tune_decode.restype = None
+    lib.svodk_tune_decode.argtypes = [ctypes.c_int32]
     lib.svodk_supported.restype = ctypes.c_int
     lib.svodk_last_chosen.restype = ctypes.c_char_p
     lib.svodk_last_error.restype = ctypes.c_char_p
@@ -365,6 +367,13 @@ def tune_streaming(workgroups_per_xcd: int) -> None:
     run as n streaming workgroups per XCD, each walking a run of query tiles; n <= 0 (the default)
     = a workgroup per tile.  Process-wide; results are bit-equal either way."""
     load_library().svodk_tune_streaming(int(workgroups_per_xcd))
+
+
+def tune_decode(rows: int) -> None:
+    """The most query rows a KV head may serve (heads / kv_heads * T) for a call without causal or per-row masks
+    or a bias to run as a decoder step, K and V streamed through registers: 0..4, 4 by default; 0 = every call
+    runs key tiles.  Process-wide; the two paths agree to the op's tolerance, not bit for bit."""
+    load_library().svodk_tune_decode(int(rows))
 
 
 def attention_packed(qkv: torch.Tensor, heads: int, kv_heads: int, opts: Optional[Attn] = None,

@@ -12,6 +12,18 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with `-m gpu` on the GPU box)")
 
 
+@pytest.fixture
+def key_tiles():
+    """Every attention call runs key tiles: a decoder step of up to four rows a KV head has a kernel of its own
+    (tests/test_gpu_decode.py), and the modules that pin the tile kernel's program (its splits, its grouped tiles,
+    its cache reads) against the tile program's restatement keep their small cases on it."""
+    import svod_amd
+
+    svod_amd.tune_decode(0)
+    yield
+    svod_amd.tune_decode(4)
+
+
 @pytest.fixture(scope="session")
 def device():
     """cuda:0 on a box whose device has kernels; the GPU tests fail, not skip, when the

@@ -12,7 +12,7 @@ import svod_amd
 from svod_amd import Attn, Cache, KeyMask
 from util import Lcg, assert_bf16_parity, bf16_tensor, bits, max_abs, to_np
 
-pytestmark = pytest.mark.gpu
+pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("key_tiles")]
 
 B, ROWS, LAYERS = 5, 2, 3
 

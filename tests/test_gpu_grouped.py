@@ -11,7 +11,7 @@ import svod_amd
 from svod_amd import Attn, Cache, KeyMask
 from util import Lcg, bf16_tensor, bits, max_abs, to_np
 
-pytestmark = pytest.mark.gpu
+pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("key_tiles")]
 
 # (name, b, t, tk, h, hkv, d, splits, lens, biased)
 CASES = [

@@ -196,7 +196,7 @@ def build_workload(name, args, dev, row_order=True):
         wl.bytes_min = 2 * b * tk * h * d * 2 + 2 * b * h * d * 2  # the layer's K and V heads read once, q and o
         wl.text = ("Whisper-large-v3 decoder step, cross-attention bf16 B16 T1 H20 D64 over 1500 cached keys, "
                    "32 layer calls/step on one cache [16,1500,640,64] (splits chosen by the library)")
-        wl.kernel_name, wl.bound = "flash_fwd_kernel<64, split, cached> + combine_kernel<64>", "hbm"
+        wl.kernel_name, wl.bound = "decode_kernel<64, split> + combine_kernel<64>", "hbm"
     elif name == "qwen3_add_rms_norm":
         # The residual add + RMSNorm between Qwen3-Embedding's layers: hidden size 16 heads x 128 = 2048.
         g = torch.Generator(device=dev).manual_seed(0x5EED0030)

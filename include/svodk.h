@@ -333,10 +333,11 @@ void svodk_tune_streaming(int32_t workgroups_per_xcd);
  * whose KV heads each serve at most SVODK_DECODE_ROWS query rows, heads / kv_heads * T) streams K and V through
  * registers past its rows instead of running 64-key tiles through LDS: such a call is bound by the bytes of K and V
  * in flight, not by arithmetic.  `rows` = the most rows a KV head may serve for a call to go that way, 0 ..
- * SVODK_DECODE_ROWS (the default); 0 = every call runs key tiles.  Process-wide.  Results of the two paths agree to
- * the op's tolerance, not bit for bit: they sum in different orders.
+ * SVODK_DECODE_ROWS; 0 = every call runs key tiles; SVODK_DECODE_ROWS_DEFAULT until a call says otherwise.
+ * Process-wide.  Results of the two paths agree to the op's tolerance, not bit for bit: they sum in different orders.
  */
 #define SVODK_DECODE_ROWS 4
+#define SVODK_DECODE_ROWS_DEFAULT 2
 void svodk_tune_decode(int32_t rows);
 /* The set the next streaming launch would take, and takes it (no device work): for tests of the
  * assignment.  No counterpart in the reference. */

@@ -24,6 +24,7 @@ from .ops import (  # noqa: F401
     attention_noalloc,
     attention_packed,
     noalloc_scratch_bytes,
+    DECODE_ROWS_DEFAULT,
     tune_decode,
     tune_streaming,
     chosen,

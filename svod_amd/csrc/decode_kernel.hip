@@ -34,7 +34,7 @@ typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kNoKey = -1e30f;   // the running maximum before any key: finite, so that differences of it are
 constexpr int kMaxWaves = 8;       // waves a workgroup
-constexpr int kAhead = 4;          // key rows a lane has in flight beyond the ones it works on
+constexpr int kAhead = 2;          // key rows a lane has in flight beyond the ones it works on
 
 // What the kernel takes: AttnArgs without the fields a decoder step does not have.
 struct DecodeArgs {
@@ -362,13 +362,15 @@ hipError_t launch_d(const DecodeArgs &p, int rows, int waves, bool f16, hipStrea
   return f16 ? launch_r<D, 4, true>(p, waves, stream) : launch_r<D, 4, false>(p, waves, stream);
 }
 
-std::atomic<int> g_decode_rows{kDecodeRows};
+std::atomic<int> g_decode_rows{kDecodeRowsDefault};
 
 }  // namespace
 
 void attention_decode_rows(int32_t rows) {
   g_decode_rows.store(rows < 0 ? 0 : (rows > kDecodeRows ? kDecodeRows : rows), std::memory_order_relaxed);
 }
+
+int32_t attention_decode_limit() { return g_decode_rows.load(std::memory_order_relaxed); }
 
 bool attention_decodes(const AttnArgs &a) {
   const bool ranged = a.win_left >= 0 || a.chunk_size > 0 || a.seg_start != nullptr;
@@ -414,7 +416,7 @@ hipError_t launch_decode(const AttnArgs &a, hipStream_t stream) {
   const int rows = p.group * p.t;
   // Few workgroups take eight waves each, so that the launch still has its bytes in flight.
   const int64_t grid = (int64_t)p.batch * p.kv_heads * p.splits;
-  const int waves = grid >= 1024 ? 4 : kMaxWaves;
+  const int waves = grid >= 256 ? 4 : kMaxWaves;
   switch (a.d) {
     case 32: return launch_d<32>(p, rows, waves, a.f16 != 0, stream);
     case 48: return launch_d<48>(p, rows, waves, a.f16 != 0, stream);

@@ -142,10 +142,12 @@ bool attention_groups(const AttnArgs &a);
 // KV head) has at most kDecodeRows query rows (group * t) streams K and V past them in registers instead of
 // running key tiles through LDS.  launch_attention takes that path by itself; splits, caches, appended rows, key
 // lengths and key masks mean what they mean to the tile kernel.
-constexpr int kDecodeRows = 4;
+constexpr int kDecodeRows = 4;         // the most the kernel is built for
+constexpr int kDecodeRowsDefault = 2;  // the most it takes unasked: up to there it has beaten the tile kernel where measured
 bool attention_decodes(const AttnArgs &a);
 // The most rows that path takes, 0..kDecodeRows (0: every call runs key tiles): see svodk_tune_decode.
 void attention_decode_rows(int32_t rows);
+int32_t attention_decode_limit();
 hipError_t launch_decode(const AttnArgs &a, hipStream_t stream);
 // One head size's kernels each (launch_attention picks by AttnArgs::d).
 hipError_t launch_attention_d32(const AttnArgs &a, hipStream_t stream);

@@ -286,8 +286,20 @@ static int split_count(const svodk_attn *opts, int64_t batch, int64_t t, int64_t
   if (asked == 1) return 1;
   if (asked > 1) return (int)(asked < most ? asked : most);
   if (opts->has_window || opts->has_chunk || opts->seg_start != nullptr) return 1;
-  // A decoder step under GQA runs a KV head's whole group in one tile (svodk::attention_groups).
   const int64_t group = kv_heads > 0 ? heads / kv_heads : 1;
+  // A decoder step of a few rows a KV head streams its keys (svodk::attention_decodes): a workgroup a (batch, KV
+  // head, split), splits of at least four key blocks, as many as bring the launch to about a thousand workgroups
+  // (one row) or five hundred (more): enough of them resident for the bytes in flight, few enough that their
+  // streams do not thrash the memory's open pages.
+  if (!opts->causal && opts->bias == nullptr && group * t >= 1 && group * t <= svodk::attention_decode_limit()) {
+    const int64_t units = kv_heads * batch;
+    if (units <= 0) return 1;
+    const int64_t target = group * t == 1 ? 1024 : 512;
+    const int64_t wanted = (target + units / 2) / units, fits = most / 4;
+    const int64_t n = wanted < fits ? wanted : fits;
+    return (int)(n < 1 ? 1 : (n > 64 ? 64 : n));
+  }
+  // A decoder step under GQA runs a KV head's whole group in one tile (svodk::attention_groups).
   const bool grouped = group > 1 && !opts->causal && group * t <= 128;
   const int64_t workgroups = grouped ? kv_heads * batch : (t + 127) / 128 * heads * batch;
   if (workgroups <= 0) return 1;

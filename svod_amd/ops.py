@@ -369,10 +369,13 @@ def tune_streaming(workgroups_per_xcd: int) -> None:
     load_library().svodk_tune_streaming(int(workgroups_per_xcd))
 
 
+DECODE_ROWS_DEFAULT = 2  # SVODK_DECODE_ROWS_DEFAULT of include/svodk.h
+
+
 def tune_decode(rows: int) -> None:
     """The most query rows a KV head may serve (heads / kv_heads * T) for a call without causal or per-row masks
-    or a bias to run as a decoder step, K and V streamed through registers: 0..4, 4 by default; 0 = every call
-    runs key tiles.  Process-wide; the two paths agree to the op's tolerance, not bit for bit."""
+    or a bias to run as a decoder step, K and V streamed through registers: 0..4, DECODE_ROWS_DEFAULT unasked;
+    0 = every call runs key tiles.  Process-wide; the two paths agree to the op's tolerance, not bit for bit."""
     load_library().svodk_tune_decode(int(rows))
 
 

@@ -21,7 +21,7 @@ def key_tiles():
 
     svod_amd.tune_decode(0)
     yield
-    svod_amd.tune_decode(4)
+    svod_amd.tune_decode(svod_amd.DECODE_ROWS_DEFAULT)
 
 
 @pytest.fixture(scope="session")

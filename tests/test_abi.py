@@ -194,15 +194,17 @@ def test_the_split_workspace_is_the_partial_tensors():
 
 def test_with_no_count_named_few_query_tiles_over_many_keys_are_split():
     """tk/src/ops/attention.rs:76-79: `None` lets the tuner choose; here a rule does: enough splits for about
-    512 workgroups, each with at least 8 key blocks, capped at 64."""
+    512 workgroups, each with at least 8 key blocks, capped at 64; a decoder step of one or two rows a KV head
+    (its own kernel) takes splits of at least 4 key blocks for about 1024 workgroups (one row) or 512 (two)."""
     import ctypes
     lib = svod_amd.load_library()
     from svod_amd.ops import _attn_options, _desc
     a = _attn_options(Attn(), [])
     # (batch, t, heads, tk) -> splits
-    for (b, tq, h, tk), want in (((16, 1, 20, 1500), 2), ((1, 1, 32, 8192), 16), ((4, 16, 16, 2048), 4),
+    for (b, tq, h, tk), want in (((16, 1, 20, 1500), 3), ((1, 1, 32, 8192), 32), ((4, 16, 16, 2048), 4),
                                  ((1, 128, 16, 8192), 16), ((64, 1, 20, 1500), 1), ((32, 512, 16, 512), 1),
-                                 ((1, 1, 1, 1 << 20), 64), ((2, 8192, 16, 8192), 1), ((1, 1, 4, 500), 1)):
+                                 ((1, 1, 1, 1 << 20), 64), ((2, 8192, 16, 8192), 1), ((1, 1, 4, 500), 2),
+                                 ((8, 2, 8, 4096), 8), ((8, 3, 8, 4096), 8)):
         qd, kd = _desc(t([b, tq, h, 64])), _desc(t([b, tk, h, 64]))
         got = lib.svodk_attention_workspace(ctypes.byref(qd), ctypes.byref(kd), ctypes.byref(a))
         assert got == (0 if want == 1 else want * b * tq * h * (64 + 2) * 4), (b, tq, h, tk)

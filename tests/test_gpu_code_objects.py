@@ -15,7 +15,7 @@ from svod_amd import Attn, KeyMask, Qkv
 from svod_amd import code_object as co
 from util import Lcg, bf16_tensor, bits
 
-pytestmark = pytest.mark.gpu
+pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("key_tiles")]  # the code objects hold the tile kernels
 
 
 class Runtime:

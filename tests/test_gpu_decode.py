@@ -11,9 +11,18 @@ import svod_amd
 from svod_amd import Attn, Cache, KeyMask
 from util import Lcg, bf16_tensor, max_abs, mean_rel, to_np
 
-pytestmark = pytest.mark.gpu
-
 STREAMED = "keys streamed through registers"
+
+
+@pytest.fixture(autouse=True)
+def up_to_four_rows():
+    """Unasked the library sends one and two rows that way; the kernel is built for up to four."""
+    svod_amd.tune_decode(4)
+    yield
+    svod_amd.tune_decode(svod_amd.DECODE_ROWS_DEFAULT)
+
+
+pytestmark = pytest.mark.gpu
 
 
 def both_paths(call):
@@ -28,7 +37,7 @@ def both_paths(call):
         torch.cuda.synchronize()
         assert STREAMED not in svod_amd.chosen(), svod_amd.chosen()
     finally:
-        svod_amd.tune_decode(4)
+        svod_amd.tune_decode(4)  # this module's setting (up_to_four_rows)
     return got, tiles
 
 
@@ -168,3 +177,13 @@ def test_a_captured_decoder_step_replays(device):
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(out, eager)
+
+
+def test_unasked_two_rows_stream_and_three_do_not(device):
+    svod_amd.tune_decode(svod_amd.DECODE_ROWS_DEFAULT)
+    g = Lcg(4)
+    k, v = g.bf16((1, 100, 1, 64)), g.bf16((1, 100, 1, 64))
+    dev = lambda x: bf16_tensor(x, device)
+    for heads, streams in ((1, True), (2, True), (3, False)):
+        svod_amd.attention(dev(g.bf16((1, 1, heads, 64))), dev(k), dev(v), Attn(splits=1))
+        assert (STREAMED in svod_amd.chosen()) == streams, (heads, svod_amd.chosen())

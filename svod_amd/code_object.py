@@ -49,6 +49,11 @@ _FULL = ([(n, B) for n in ("q", "k", "v", "o", "key_lens", "key_mask", "seg_star
                            "kv_row_elems", "splits", "win_left", "win_right", "chunk_size", "chunk_left", "chunk_right",
                            "seg_i64", "bias_per_batch", "kv_head_start", "row_map_i64", "cache_rows", "app_rows",
                            "app_lens_i64")])
+_DECODE = ([(n, B) for n in ("q", "k", "v", "o", "key_lens", "key_mask", "row_map", "k_app", "v_app", "app_lens", "o_part",
+                              "m_part", "l_part")] +
+           [(n, S) for n in ("batch", "t", "tk", "heads", "kv_heads", "scale_bits", "lens_i64", "mask_bytes", "q_row_elems",
+                             "kv_row_elems", "splits", "cached", "kv_head_start", "row_map_i64", "cache_rows", "app_rows",
+                             "app_lens_i64")])
 _COMBINE = [("o_part", B), ("m_part", B), ("l_part", B), ("o", B), ("rows", S), ("splits", S)]
 
 
@@ -108,6 +113,14 @@ def entries() -> Dict[str, dict]:
                     "ranged": bool(r), "biased": bool(b), "cached": bool(k), "grouped": bool(g), "key_mask": True,
                     "cfg": f"FaCfg {{ bq: 128, bkv: 64, stages: 2, splits: {'n' if s else 1}, forms: {{ raw_max, "
                            f"skip_rescale }}, warp_rows: 32, core: mfma_f32_32x32x16_{dtype} }}"}
+            for rows in (1, 2, 4):  # the decoder step: at most `rows` query rows a KV head, keys streamed through registers
+                for s in (0, 1):
+                    out[f"svodk_decode_d{d}_r{rows}_{dtype}_s{s}"] = {
+                        "file": "svodk_decode.co", "source": "decode_kernel.hip", "params": _DECODE, "local": [256, 1, 1],
+                        "workgroups": "batch * kv_heads" + (" * splits" if s else ""), "op": "attention", "dtype": dtype,
+                        "head_dim": d, "causal": False, "split": bool(s), "rows_per_kv_head": rows, "key_mask": True,
+                        "cfg": f"FaCfg {{ rows: {rows}, lanes_per_key: {max(d, 64 if d == 48 else d) // 8}, splits: "
+                               f"{'n' if s else 1}, core: v_dot2_f32_{dtype}, keys streamed through registers }}"}
             out[f"svodk_combine_d{d}_{dtype}"] = {
                 "file": "svodk_combine.co", "source": "combine_kernel.hip", "params": _COMBINE, "local": [256, 1, 1],
                 "workgroups": f"(rows * {d // 4} + 255) // 256", "op": "combine_splits", "dtype": dtype, "head_dim": d,

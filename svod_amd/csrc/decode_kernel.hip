@@ -107,8 +107,9 @@ __device__ __forceinline__ void merge(State &a, const State &b) {
   for (int j = 0; j < 8; j++) a.acc[j] = a.acc[j] * wa + b.acc[j] * wb;
 }
 
+// The workgroup's program for `nw` waves, for the kernels below to inline.
 template <int D, int R, bool F16, bool SPLIT>
-__global__ __launch_bounds__(kMaxWaves * 64) void decode_kernel(const DecodeArgs p) {
+__device__ __forceinline__ void decode_body(const DecodeArgs &p, const int nw) {
 #if defined(__HIP_DEVICE_COMPILE__)
   constexpr int kWide = D == 48 ? 64 : D;
   constexpr int LPK = kWide / 8;   // lanes a key row
@@ -124,7 +125,6 @@ __global__ __launch_bounds__(kMaxWaves * 64) void decode_kernel(const DecodeArgs
   const int tid = (int)__builtin_amdgcn_workitem_id_x();
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int nw = (int)(__builtin_amdgcn_workgroup_size_x() >> 6);
   const int pos = lane % LPK;   // which 16 bytes of a row
   const int slot = lane / LPK;  // which row of a wave instruction
   const bool pos_ok = 8 * pos < D;
@@ -343,6 +343,14 @@ __global__ __launch_bounds__(kMaxWaves * 64) void decode_kernel(const DecodeArgs
 #endif  // __HIP_DEVICE_COMPILE__
 }
 
+#if !defined(SVODK_CODE_OBJECT)  // the library's kernel and its launch: not part of a code object build
+template <int D, int R, bool F16, bool SPLIT>
+__global__ __launch_bounds__(kMaxWaves * 64) void decode_kernel(const DecodeArgs p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  decode_body<D, R, F16, SPLIT>(p, (int)(__builtin_amdgcn_workgroup_size_x() >> 6));
+#endif
+}
+
 template <int D, int R, bool F16>
 hipError_t launch_r(const DecodeArgs &p, int waves, hipStream_t stream) {
   const int64_t grid = (int64_t)p.batch * p.kv_heads * p.splits;
@@ -428,3 +436,46 @@ hipError_t launch_decode(const AttnArgs &a, hipStream_t stream) {
 }
 
 }  // namespace svodk
+
+#else  // SVODK_CODE_OBJECT
+}  // namespace
+}  // namespace svodk
+// ---------------------------------------------------------------------------------------------
+// The same program as kernels a loader outside the HIP runtime can run (a flat argument record, static LDS, no
+// dispatch packet: the workgroup is 256 threads, which the kernel cannot ask and therefore fixes).  One kernel an
+// instantiation, svodk_decode_d<D>_r<rows>_<type>_s<split>, all with one record.  Buffers, an address of 0 for what
+// a call does not have: q, k, v, o, key_lens, key_mask, row_map, k_app, v_app, app_lens, then the partial states of
+// a split call o_part, m_part, l_part.  Scalars: batch, t, tk, heads, kv_heads, scale_bits, lens_i64, mask_bytes (1 or
+// 4), q_row_elems, kv_row_elems (0: heads * D and kv_heads * D), splits, cached, kv_head_start, row_map_i64,
+// cache_rows, app_rows, app_lens_i64.  Launch: batch * kv_heads * (s ? splits : 1) workgroups of 256 threads; r is
+// the least of 1, 2, 4 that holds heads / kv_heads * t.
+// ---------------------------------------------------------------------------------------------
+#define SVODK_DECODE_ENTRY(D, R, T, F16, S)                                                                           \
+  extern "C" __global__ __launch_bounds__(256) void svodk_decode_d##D##_r##R##_##T##_s##S(                            \
+      const uint16_t *__restrict__ q, const uint16_t *__restrict__ k, const uint16_t *__restrict__ v,                 \
+      uint16_t *__restrict__ o, const void *__restrict__ key_lens, const void *__restrict__ key_mask,                 \
+      const void *__restrict__ row_map, const uint16_t *__restrict__ k_app, const uint16_t *__restrict__ v_app,       \
+      const void *__restrict__ app_lens, float *__restrict__ o_part, float *__restrict__ m_part,                      \
+      float *__restrict__ l_part, int32_t batch, int32_t t, int32_t tk, int32_t heads, int32_t kv_heads,              \
+      int32_t scale_bits, int32_t lens_i64, int32_t mask_bytes, int32_t q_row_elems, int32_t kv_row_elems,            \
+      int32_t splits, int32_t cached, int32_t kv_head_start, int32_t row_map_i64, int32_t cache_rows,                 \
+      int32_t app_rows, int32_t app_lens_i64) {                                                                       \
+    if (batch <= 0 || t <= 0 || tk < 0 || kv_heads <= 0 || heads < kv_heads) return;                                  \
+    svodk::DecodeArgs p;                                                                                              \
+    p.q = q, p.k = k, p.v = v, p.o = o, p.key_lens = key_lens, p.key_mask = key_mask, p.row_map = row_map;            \
+    p.k_app = k_app, p.v_app = v_app, p.app_lens = app_lens, p.o_part = o_part, p.m_part = m_part, p.l_part = l_part; \
+    p.q_row_elems = q_row_elems > 0 ? q_row_elems : heads * D;                                                        \
+    p.kv_row_elems = kv_row_elems > 0 ? kv_row_elems : kv_heads * D;                                                  \
+    p.lens_i64 = lens_i64, p.mask_bytes = mask_bytes, p.row_map_i64 = row_map_i64, p.app_lens_i64 = app_lens_i64;     \
+    p.batch = batch, p.t = t, p.tk = tk, p.heads = heads, p.kv_heads = kv_heads, p.group = heads / kv_heads;          \
+    p.splits = (S) && splits > 1 ? splits : 1, p.cached = cached, p.kv_head_start = kv_head_start;                    \
+    p.cache_rows = cache_rows, p.app_rows = app_rows, p.scale = __builtin_bit_cast(float, scale_bits);                \
+    svodk::decode_body<D, R, F16, (S) != 0>(p, 4);                                                                    \
+  }
+#define SVODK_DECODE_ROWS_OF(D, T, F16, S) \
+  SVODK_DECODE_ENTRY(D, 1, T, F16, S) SVODK_DECODE_ENTRY(D, 2, T, F16, S) SVODK_DECODE_ENTRY(D, 4, T, F16, S)
+#define SVODK_DECODE_FAMILY(D)                                              \
+  SVODK_DECODE_ROWS_OF(D, bf16, false, 0) SVODK_DECODE_ROWS_OF(D, bf16, false, 1) \
+  SVODK_DECODE_ROWS_OF(D, f16, true, 0) SVODK_DECODE_ROWS_OF(D, f16, true, 1)
+SVODK_DECODE_FAMILY(32) SVODK_DECODE_FAMILY(48) SVODK_DECODE_FAMILY(64) SVODK_DECODE_FAMILY(128) SVODK_DECODE_FAMILY(256)
+#endif  // SVODK_CODE_OBJECT

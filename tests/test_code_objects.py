@@ -41,8 +41,9 @@ def test_the_record_is_packed_as_the_loader_packs_it():
 
 def test_every_kernel_meets_the_loaders_conditions(built):
     table = co.entries()
-    # the short records (attention 32, prologue 10, norms 24, projection 6), every form of every head size and type, the merges
-    assert len(table) == 72 + 5 * 2 * 40 + 10
+    # the short records (attention 32, prologue 10, norms 24, projection 6), every form of every head size and type, the
+    # merges, the decoder step (1, 2 or 4 rows a KV head, split or not)
+    assert len(table) == 72 + 5 * 2 * 40 + 10 + 5 * 2 * 3 * 2
     assert len(list(co.full_forms())) == 40
     for name, e in table.items():
         kd = co.check(built[e["file"]], name, e["params"])
@@ -50,7 +51,12 @@ def test_every_kernel_meets_the_loaders_conditions(built):
         assert kd.kernel_code_properties == co.KERNARG_SEGMENT_PTR, name  # the record's address and nothing else
         assert kd.user_sgprs == 2 and kd.kernarg_preload == 0, name
         assert kd.private_segment_fixed_size == 0, name
-        if e["op"] == "attention":
+        if "rows_per_kv_head" in e:
+            # The decoder step holds no keys in LDS: ten floats (m, l, eight columns) a row, a lane of a key row and a
+            # wave, for the merge of up to eight waves at the end.
+            wide = 64 if e["head_dim"] == 48 else e["head_dim"]
+            assert kd.group_segment_fixed_size == 8 * e["rows_per_kv_head"] * (wide // 8) * 10 * 4, name
+        elif e["op"] == "attention":
             # The K and V ring: two slots each of 64 keys (tk/src/kernels/attention.rs:187-190).
             # and behind it, with a key mask, a 64-bit word a key block for each of 4 waves (256 blocks scanned).
             mask_words = 4 * 256 * 8 if e.get("key_mask") else 0

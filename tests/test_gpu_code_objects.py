@@ -312,3 +312,39 @@ def test_linear_code_object_equals_the_library(device, runtime, turn, f16, biase
                           "cos": cos.data_ptr() if turn else 0, "sin": sin.data_ptr() if turn else 0, "y": got.data_ptr(),
                           "rows": b * t, "n": n, "k": k, "seq": t, "heads": heads})
     assert np.array_equal(bits(got), bits(want))
+
+
+@pytest.mark.parametrize("d,h,hkv,f16", [(64, 16, 8, False), (128, 8, 8, True)], ids=["d 64, two rows a KV head", "f16 d 128"])
+def test_decode_code_object_and_the_merge_equal_the_library(device, runtime, d, h, hkv, f16):
+    """A decoder step over a cache of three layers' heads with a row map, appended rows and their counts, two key
+    splits: the kernel that streams its keys through registers (as many workgroups as make the library launch four
+    waves each, which is what the code object's kernels are fixed at), then combine_splits."""
+    from svod_amd import Cache
+    b, t, tk, rows, layers, appended, splits = 16, 1, 700, 3, 3, 2, 2
+    g = Lcg(40)
+    q = tensor(g.bf16((b, t, h, d)), device, f16)
+    k, v = (tensor(g.bf16((rows, tk, layers * hkv, d)), device, f16) for _ in range(2))
+    k_app, v_app = (tensor(g.bf16((b, appended, hkv, d)), device, f16) for _ in range(2))
+    lens = torch.tensor([tk, 1, 37, tk - 1, 0, 64, 65, 300] * 2, dtype=torch.int32, device=device)
+    row_map = torch.tensor([0, 1, 2, 0, 1, 2, 1, 0] * 2, dtype=torch.int64, device=device)
+    seen = torch.tensor([2, 1, 2, 0, 1, 2, 2, 1] * 2, dtype=torch.int32, device=device)
+    svod_amd.tune_decode(svod_amd.DECODE_ROWS_DEFAULT)  # this module runs key tiles otherwise
+    want = svod_amd.attention(q, k, v, Attn(keys=KeyMask.lens(lens), splits=splits,
+                                            cache=Cache(hkv, hkv, row_map=row_map, appended=(k_app, v_app), app_lens=seen)))
+    assert "combine_splits" in svod_amd.chosen()
+    n = b * t * h
+    parts = (torch.full((splits, n, d), 7.0, device=device), torch.full((splits, n), 7.0, device=device),
+             torch.full((splits, n), 7.0, device=device))
+    kind = "f16" if f16 else "bf16"
+    runtime.launch(f"svodk_decode_d{d}_r{h // hkv * t}_{kind}_s1", {
+        "q": q.data_ptr(), "k": k.data_ptr(), "v": v.data_ptr(), "o": 0, "key_lens": lens.data_ptr(), "key_mask": 0,
+        "row_map": row_map.data_ptr(), "k_app": k_app.data_ptr(), "v_app": v_app.data_ptr(), "app_lens": seen.data_ptr(),
+        "o_part": parts[0].data_ptr(), "m_part": parts[1].data_ptr(), "l_part": parts[2].data_ptr(), "batch": b, "t": t,
+        "tk": tk, "heads": h, "kv_heads": hkv, "scale_bits": f32_bits(d ** -0.5), "lens_i64": 0, "mask_bytes": 0,
+        "q_row_elems": 0, "kv_row_elems": layers * hkv * d, "splits": splits, "cached": 1, "kv_head_start": hkv,
+        "row_map_i64": 1, "cache_rows": rows, "app_rows": appended, "app_lens_i64": 0})
+    got = torch.full_like(want, 7.0)
+    runtime.launch(f"svodk_combine_d{d}_{kind}", {"o_part": parts[0].data_ptr(), "m_part": parts[1].data_ptr(),
+                                                   "l_part": parts[2].data_ptr(), "o": got.data_ptr(), "rows": n,
+                                                   "splits": splits})
+    assert np.array_equal(bits(got), bits(want))

@@ -187,3 +187,30 @@ def test_unasked_two_rows_stream_and_three_do_not(device):
     for heads, streams in ((1, True), (2, True), (3, False)):
         svod_amd.attention(dev(g.bf16((1, 1, heads, 64))), dev(k), dev(v), Attn(splits=1))
         assert (STREAMED in svod_amd.chosen()) == streams, (heads, svod_amd.chosen())
+
+
+def test_the_fused_projection_read_in_place(device):
+    """attention_packed (tk/src/ops/attention.rs:104-122) on a decoder step: q, k and v are views of one row."""
+    b, t, h, hkv, d = 3, 1, 4, 2, 64
+    g = Lcg(6)
+    qkv = g.bf16((b, t, (h + 2 * hkv) * d))
+    qkv_d = bf16_tensor(qkv, device)
+    got = svod_amd.attention_packed(qkv_d, h, hkv, Attn(splits=1))
+    torch.cuda.synchronize()
+    assert STREAMED in svod_amd.chosen(), svod_amd.chosen()
+    q, k, v = (qkv[..., a * d:e * d].reshape(b, t, -1, d) for a, e in ((0, h), (h, h + hkv), (h + hkv, h + 2 * hkv)))
+    want = oracle.attention_direct(oracle.AttnProblem(np.ascontiguousarray(q), np.ascontiguousarray(k), np.ascontiguousarray(v)))
+    assert max_abs(to_np(got), want) < 2e-2
+
+
+def test_a_bound_batch_runs_its_live_rows_only(device):
+    b, live, t, tk, h, d = 4, 2, 1, 300, 4, 64
+    g = Lcg(13)
+    q, k, v = g.bf16((b, t, h, d)), g.bf16((b, tk, h, d)), g.bf16((b, tk, h, d))
+    out = torch.full((b, t, h, d), 7.0, dtype=torch.bfloat16, device=device)
+    svod_amd.attention(bf16_tensor(q, device), bf16_tensor(k, device), bf16_tensor(v, device), Attn(splits=1, batch_live=live), out=out)
+    torch.cuda.synchronize()
+    assert STREAMED in svod_amd.chosen()
+    want = oracle.attention_direct(oracle.AttnProblem(q[:live], k[:live], v[:live]))
+    assert max_abs(to_np(out[:live]), want) < 2e-2
+    assert (to_np(out[live:]) == 7.0).all()

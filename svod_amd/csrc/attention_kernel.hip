@@ -185,13 +185,22 @@ __device__ __forceinline__ Pair both_halves(float x) {
 // A raw buffer descriptor over `bytes` bytes at `base` (stride 0, 32-bit raw format): loads
 // past the end return zero, which is how rows at and past a batch's key length read (the
 // bounded views of tk/src/kernels/attention.rs:551-560).
+// Both arguments are the same in every lane (a descriptor lives in scalar registers).  The bound is `bytes`
+// clamped to [0, 2^32 - 1] on the scalar unit: written as comparisons of the 64-bit value the compiler does it on
+// the VALU (v_cmp_*_i64 on broadcast operands), six vector instructions a descriptor in a loop whose VALU port is
+// what bounds it.
 __device__ __forceinline__ i32x4 make_rsrc(const void *base, int64_t bytes) {
-  const int64_t clamped = bytes < 0 ? 0 : (bytes > 0xffffffffLL ? 0xffffffffLL : bytes);
   const uint64_t addr = (uint64_t)(uintptr_t)base;
+  const int lo = (int)(uint32_t)(uint64_t)bytes, hi = (int)(bytes >> 32);
+  int bound;
+  asm("s_cmp_lt_i32 %1, 0\n\ts_cselect_b32 %0, 0, %2\n\ts_cmp_gt_i32 %1, 0\n\ts_cselect_b32 %0, -1, %0"
+      : "=&s"(bound)
+      : "s"(hi), "s"(lo)
+      : "scc");
   i32x4 r;
   r[0] = (int)(uint32_t)addr;
   r[1] = (int)(uint32_t)((addr >> 32) & 0xffffu);
-  r[2] = (int)(uint32_t)clamped;
+  r[2] = bound;
   r[3] = 0x00020000;
   return r;
 }

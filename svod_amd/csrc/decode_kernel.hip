@@ -32,9 +32,9 @@ typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
 
 constexpr float kLog2e = 1.4426950408889634f;
-constexpr float kNoKey = -1e30f;   // the running maximum before any key: finite, so that differences of it are
+constexpr float kNoKey = -1e30f;   // the running maximum before any key: finite, so that its differences are numbers
 constexpr int kMaxWaves = 8;       // waves a workgroup
-constexpr int kAhead = 2;          // key rows a lane has in flight beyond the ones it works on
+constexpr int kAhead = 2;          // passes a lane works on at a time, with as many more in flight
 
 // What the kernel takes: AttnArgs without the fields a decoder step does not have.
 struct DecodeArgs {

@@ -953,16 +953,7 @@ __device__ __forceinline__ void flash_fwd_body(
       w.v_src[j] = TL::source(row, pc, w.kv_row_bytes, true, j * NW * kRowsPer);
     }
   }
-  // ---- K(0), V(0), K(1) go first: everything below runs in the shadow of their flight.
-  w.nxt_end = 0;  // one item a workgroup
-  w.end_even = end;
-  w.nxt_k = w.nxt_v = nullptr;
-  w.nxt_bytes = 0;
-  fill_k<D, NW>(w, 0, 0);
-  fill_v<D, NW>(w, 0, 0);
-  fill_k<D, NW>(w, 1, 1);
-  // ---- Q fragments: B operand of the score product, resident for the block.  They are asked for after
-  // the fills (which have the longer way: the first barrier waits for both).
+  // ---- Q fragments: B operand of the score product, resident for the block.
   {
     const uint16_t *q_ptr = q + ((int64_t)b * t + q_row) * q_row_stride + (int64_t)q_head * D + w.g * 8;
 #pragma unroll
@@ -972,24 +963,76 @@ __device__ __forceinline__ void flash_fwd_body(
       w.qf[ks] = x;
     }
   }
+  // ---- the first eight blocks' elements of a key mask row that is scanned up front (see below) are asked for
+  // now, a lane a key, straight into this wave's stretch of LDS: behind the Q loads and ahead of the fills in
+  // the memory counter's order, so that the scan can wait for them with the fills still in flight.
+  w.mask_words = (LDS_PTR(uint64_t))(smem + TL::kLds) + w.wave * kScannedBlocks;
+  const bool scan_early = key_mask != nullptr && end <= kScannedBlocks && end > 0;
+  if (scan_early) {
+    const uint8_t *row = (const uint8_t *)key_mask + w.mask_row * mask_bytes;
+    const i32x4 r = make_rsrc(row, (int64_t)w.tk * mask_bytes);  // keys past the row read as hidden
+    const int at = (int)(uintptr_t)(w.mask_words);
+    // Block i lies 64 elements further on: the instruction's own offset, which the LDS address takes as well as the
+    // memory address (block i's 256 bytes of LDS start at m0 + that offset).
+    const int voff = w.lane * mask_bytes;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      if (mask_bytes == 1)
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_ubyte %1, %2, 0 offen offset:%3 lds"
+                     :
+                     : "s"(at + i * 256 - i * kBkv), "v"(voff), "s"(r), "n"(i * kBkv)
+                     : "memory");
+      else
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, 0 offen offset:%3 lds"
+                     :
+                     : "s"(at + i * 256 - i * kBkv * 4), "v"(voff), "s"(r), "n"(i * kBkv * 4)
+                     : "memory");
+    }
+  }
+  // ---- K(0), V(0), K(1): everything below runs in the shadow of their flight.
+  w.nxt_end = 0;  // one item a workgroup
+  w.end_even = end;
+  w.nxt_k = w.nxt_v = nullptr;
+  w.nxt_bytes = 0;
+  const int fills_out = W::CH * (end > 1 ? 3 : end > 0 ? 2 : 0);
+  fill_k<D, NW>(w, 0, 0);
+  fill_v<D, NW>(w, 0, 0);
+  fill_k<D, NW>(w, 1, 1);
   // A key mask row of up to kScannedBlocks blocks is scanned now, under the fills' flight: every
   // wave ballots each block's 64 keys into a word of its own LDS copy.  The scan also says where
   // the row's last visible key is (later blocks are skipped, like blocks past a length) and how
   // many leading blocks hide nothing (those take the hot loop).  A longer row's words are read two
   // blocks ahead of their use instead.
   w.scanned = key_mask != nullptr && end <= kScannedBlocks;
-  w.mask_words = (LDS_PTR(uint64_t))(smem + TL::kLds) + w.wave * kScannedBlocks;
   int word0 = 0, lead_open = 0, seen_end = 0;
   w.mask_next = 0;
   if (w.scanned) {
     bool open = true;
     int visible = 0, last_key = 0;  // keys the row shows, and the place after the last of them
+    // A row of up to eight blocks keeps its words in scalar registers until it is known to need them: a padding
+    // mask (the usual case) turns into a length below and never reads them.
+    const bool few = end <= 8;
+    uint64_t kept[8];
     for (int base = 0; base < end; base += 8) {
       // Eight blocks' elements in flight together: every lane loads (a key past the row's end, or a block
       // past the tile's, loads the row's first element and drops it), so that no branch stands between the
       // loads and a single wait brings them in.
       int words[8];
-      if (w.mask_bytes == 1) {
+      if (base == 0 && scan_early) {
+        // Asked for ahead of the fills: everything issued before the fills is back when no more than the fills are out.
+        constexpr int kCh = W::CH;
+        if (fills_out == 3 * kCh)
+          asm volatile("s_waitcnt vmcnt(%0)" : : "n"(3 * kCh) : "memory");
+        else if (fills_out == 2 * kCh)
+          asm volatile("s_waitcnt vmcnt(%0)" : : "n"(2 * kCh) : "memory");
+        else
+          asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+        LDS_PTR(const int) raw = (LDS_PTR(const int))(w.mask_words);
+#pragma unroll
+        for (int i = 0; i < 8; i++) words[i] = raw[i * 64 + w.lane];
+        // The words go where the elements lay: every element is in a register before the first word is written.
+        asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");
+      } else if (w.mask_bytes == 1) {
 #pragma unroll
         for (int i = 0; i < 8; i++) {
           const int key = (base + i) * kBkv + w.lane;
@@ -1010,7 +1053,8 @@ __device__ __forceinline__ void flash_fwd_body(
       for (int i = 0; i < 8; i++) {
         if (base + i >= end) break;
         const uint64_t bits = __builtin_amdgcn_ballot_w64(words[i] != 0);
-        if (w.lane == 0) w.mask_words[base + i] = bits;
+        kept[i] = bits;
+        if (!few && w.lane == 0) w.mask_words[base + i] = bits;
         if (bits != 0) {
           seen_end = base + i + 1;
           last_key = (base + i) * kBkv + 64 - __builtin_clzll(bits);
@@ -1031,6 +1075,10 @@ __device__ __forceinline__ void flash_fwd_body(
       w.key_mask = nullptr;
       w.scanned = false;
       w.kv_bytes = len > 0 ? (int64_t)(len - 1) * w.kv_row_bytes + D * 2 : 0;
+    } else if (few && w.lane == 0) {
+#pragma unroll
+      for (int i = 0; i < 8; i++)
+        if (i < end) w.mask_words[i] = kept[i];
     }
   } else if (key_mask != nullptr) {
     word0 = mask_lane<D, NW>(w, 0);

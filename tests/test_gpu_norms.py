@@ -128,6 +128,32 @@ def test_many_rows_and_the_same_bits_whatever_the_row_count(device):
     assert close(to_np(many[1]), oracle.round_bf16(want), 1e-2)
 
 
+def test_the_stored_sum_rounds_as_the_reference_does_at_the_edges(device):
+    """tk/src/interp.rs:37-44 where a plausible narrowing differs: ties to even in both directions, the carry
+    into the exponent, the largest finite value's overflow to infinity, subnormals, signed zeros, infinities and
+    the bits of a NaN; every pair of bf16 values of a sweep as well (x + r in f32, narrowed once)."""
+    d = 256
+    x16 = np.array([0x3F80, 0x3F81, 0x3F80, 0x3FFF, 0x7F7F, 0x7F7F, 0xFF7F, 0x0001, 0x0001, 0x8001, 0x0000, 0x8000,
+                    0x7F80, 0x7F80, 0x7FC1, 0xFFA0, 0x0080, 0x4000], dtype=np.uint16)
+    r16 = np.array([0x3B80, 0x3B80, 0x3B00, 0x3B80, 0x7300, 0x7B00, 0xFB00, 0x0001, 0x8001, 0x8002, 0x8000, 0x8000,
+                    0xFF80, 0x3F80, 0x3F80, 0x0000, 0x8001, 0x3780], dtype=np.uint16)
+    g = np.random.default_rng(21)
+    sweep = g.integers(0, 1 << 16, size=(2, 64 * d - x16.size), dtype=np.uint16)
+    x = oracle.from_bf16_bits(np.concatenate([x16, sweep[0]])).reshape(64, d)
+    r = oracle.from_bf16_bits(np.concatenate([r16, sweep[1]])).reshape(64, d)
+    up = lambda a: torch.from_numpy((a.view(np.uint32) >> 16).astype(np.uint16).view(np.int16)).view(torch.bfloat16).to(device)
+    total, _ = svod_amd.add_rms_norm(up(x), up(r), bf16_tensor(np.ones(d, dtype=np.float32), device), 1e-6)
+    torch.cuda.synchronize()
+    with np.errstate(all="ignore"):
+        want = oracle.bf16_bits(x + r)
+        nan = np.isnan(x + r)
+    got = bits(total)
+    assert np.array_equal(got[~nan], want[~nan])
+    # A NaN keeps being one, quiet; which operand's payload the f32 add carries over is the adder's business.
+    assert ((got[nan] & 0x7FC0) == 0x7FC0).all()
+    assert nan.sum() > 100 and (~nan).sum() > 10000
+
+
 def test_a_width_without_a_kernel_keeps_the_graph(device):
     x = bf16_tensor(np.ones((4, 1000), dtype=np.float32), device)
     with pytest.raises(svod_amd.GraphFallback) as e:

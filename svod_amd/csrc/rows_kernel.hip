@@ -182,8 +182,8 @@ template <int SPANS, bool LAYER, bool RESIDUAL, bool BIAS, bool F16>
 hipError_t launch_rows(const NormArgs &a, hipStream_t stream) {
   // The same number of workgroups on every compute unit, at most what this instantiation's registers let a unit
   // hold (asked of the runtime once a device), every wave walking its share of the rows.  The units share the
-  // memory's bandwidth, so a launch costs about (rows a wave) x (workgroups a unit): the count that makes that
-  // least, the larger on a tie (more rows in flight).  A unit with a workgroup more than its neighbours, or a wave
+  // memory's bandwidth, so a launch costs about (rows a wave) x (workgroups a unit, or the count that keeps the
+  // memory busy if that is more): the count that makes that least, the larger on a tie (more rows in flight).  A unit with a workgroup more than its neighbours, or a wave
   // with a row more, is what the launch then waits for (683 workgroups for 16384 rows: 50.5 us; 512: 46.5).
   static std::atomic<int> geometry[64];  // (workgroups a unit) << 16 | units
   int device = 0;
@@ -205,9 +205,13 @@ hipError_t launch_rows(const NormArgs &a, hipStream_t stream) {
   if (all == 0) return hipSuccess;
   int64_t blocks = all;
   if (all > units) {
+    // Below about 64 KiB of loads in flight a unit the memory system is not kept busy and a row takes as long
+    // whatever the count: fewer workgroups than that buy nothing (a wave asks for a row ahead: a KiB a span and tensor).
+    constexpr int64_t kInFlight = 64 * 1024, kOfAWorkgroup = kRowsPerBlock * SPANS * (RESIDUAL ? 2 : 1) * 1024;
+    const int64_t enough = std::min(per_unit, (kInFlight + kOfAWorkgroup - 1) / kOfAWorkgroup);
     int64_t best = 0;
     for (int64_t m = per_unit; m >= 1; m--) {
-      const int64_t cost = (all + units * m - 1) / (units * m) * m;
+      const int64_t cost = (all + units * m - 1) / (units * m) * std::max(m, enough);
       if (best == 0 || cost < best) best = cost, blocks = units * m;
     }
   }

@@ -154,6 +154,33 @@ def test_the_stored_sum_rounds_as_the_reference_does_at_the_edges(device):
     assert nan.sum() > 100 and (~nan).sum() > 10000
 
 
+def test_a_form_first_met_under_stream_capture(device):
+    """The launch asks the runtime once per form what a compute unit holds; that question is allowed while a
+    stream is being captured, and the captured launch gives the eager call's bits on every replay."""
+    d = 3328  # a width and form no other test of this process runs: f16, LayerNorm, residual, bias
+    g = np.random.default_rng(3)
+    mk = lambda *shape: torch.from_numpy(g.standard_normal(shape).astype(np.float32)).to(torch.float16).to(device)
+    x, r, w, b = mk(301, d), mk(301, d), mk(d), mk(d)
+    total, y = torch.empty_like(x), torch.empty_like(x)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            svod_amd.add_layer_norm(x, r, w, b, 1e-5, out=(total, y))
+    torch.cuda.current_stream().wait_stream(side)
+    seen = []
+    for _ in range(3):
+        total.zero_(), y.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        seen.append((total.clone(), y.clone()))
+    eager = svod_amd.add_layer_norm(x, r, w, b, 1e-5)
+    torch.cuda.synchronize()
+    for t, o in seen:
+        assert torch.equal(t, eager[0]) and torch.equal(o, eager[1])
+
+
 def test_a_width_without_a_kernel_keeps_the_graph(device):
     x = bf16_tensor(np.ones((4, 1000), dtype=np.float32), device)
     with pytest.raises(svod_amd.GraphFallback) as e:

@@ -214,3 +214,71 @@ def test_a_bound_batch_runs_its_live_rows_only(device):
     want = oracle.attention_direct(oracle.AttnProblem(q[:live], k[:live], v[:live]))
     assert max_abs(to_np(out[:live]), want) < 2e-2
     assert (to_np(out[live:]) == 7.0).all()
+
+
+def test_random_calls_agree_with_the_tile_kernel(device):
+    """A seeded sweep over head sizes, row counts, GQA groups, key counts around the block edges, both types, split
+    counts, every key-mask form, caches with row maps, layers and appended rows, and scales of either sign: the
+    two kernels give the same outcome (a result or the same refusal) and results within the op's bar."""
+    import random
+    rng = random.Random(20)
+    torch.manual_seed(20)
+    compared = 0
+    for case in range(160):
+        d = rng.choice([32, 48, 64, 128, 256])
+        rows = rng.choice([1, 1, 2, 2, 3, 4])
+        group = rng.choice([g for g in (1, 2, 3, 4) if rows % g == 0])
+        t, hkv = rows // group, rng.choice([1, 2, 3, 5, 8])
+        h, b = hkv * group, rng.choice([1, 2, 3, 7, 16])
+        tk = rng.choice([1, 5, 63, 64, 65, 127, 128, 129, 300, 777, 1500, 4096])
+        dt = torch.float16 if rng.random() < 0.3 else torch.bfloat16
+        splits = rng.choice([None, None, 1, 2, 3, 5, 9])
+        kind = rng.choice(["none", "lens", "lens64", "mask", "maskint"])
+        cached = rng.random() < 0.4
+        layers = rng.choice([1, 3]) if cached else 1
+        crow = rng.choice([b, max(1, b // 2), b + 2]) if cached else b
+        mapped = cached and (crow != b or rng.random() < 0.5)
+        if cached and not mapped and crow != b:
+            crow = b
+        q = torch.randn(b, t, h, d, device=device).to(dt)
+        k = torch.randn(crow, tk, layers * hkv, d, device=device).to(dt)
+        v = torch.randn(crow, tk, layers * hkv, d, device=device).to(dt)
+        keys = KeyMask.none()
+        if kind in ("lens", "lens64"):
+            lens = [rng.choice([0, 1, tk, tk // 2, max(tk - 1, 0), rng.randint(0, tk)]) for _ in range(b)]
+            keys = KeyMask.lens(torch.tensor(lens, dtype=torch.int64 if kind == "lens64" else torch.int32, device=device))
+        elif kind in ("mask", "maskint"):
+            m = torch.rand(b, tk, device=device) < rng.choice([0.1, 0.5, 0.9])
+            if b > 1:
+                m[1] = False
+            keys = KeyMask.bool(m if kind == "mask" else m.to(torch.int32))
+        cache = None
+        if cached:
+            app = rng.choice([0, 1, 3, 8])
+            appended = (torch.randn(b, app, hkv, d, device=device).to(dt), torch.randn(b, app, hkv, d, device=device).to(dt)) if app else None
+            app_lens = (torch.tensor([rng.randint(0, app) for _ in range(b)], dtype=torch.int32, device=device)
+                        if app and rng.random() < 0.5 else None)
+            row_map = (torch.tensor([rng.randrange(crow) for _ in range(b)], dtype=rng.choice([torch.int32, torch.int64]), device=device)
+                       if mapped else None)
+            cache = Cache((layers - 1) * hkv, hkv, row_map, appended, app_lens)
+        opts = Attn(keys=keys, splits=splits, cache=cache, scale=rng.choice([None, None, 0.07, -0.1]))
+        name = f"case {case}: b{b} t{t} tk{tk} h{h}/{hkv} d{d} {dt} splits={splits} {kind} cached={cached} layers={layers} mapped={mapped}"
+        outcomes = []
+        for knob in (4, 0):
+            svod_amd.tune_decode(knob)
+            try:
+                ws = torch.empty(16 * b * t * h * (d + 2) * 4, dtype=torch.uint8, device=device)
+                outcomes.append(svod_amd.attention(q, k, v, opts, workspace=ws))
+            except (svod_amd.OpError, svod_amd.GraphFallback) as e:
+                outcomes.append(type(e).__name__ + ": " + str(e))
+        svod_amd.tune_decode(4)
+        torch.cuda.synchronize()
+        one, two = outcomes
+        if isinstance(one, str) or isinstance(two, str):
+            assert one == two, name
+            continue
+        compared += 1
+        assert torch.isfinite(one.float()).all(), name
+        if one.numel():
+            assert float((one.float() - two.float()).abs().max()) < 2e-2, name
+    assert compared > 120

@@ -108,3 +108,90 @@ def test_calls_that_draw_every_option_match_the_direct_softmax(device):
     for name, why in kept_graph:
         assert "Config" in why or "Shape" in why, (name, why)
     assert ran >= 130, (ran, kept_graph[:5])
+
+
+def test_projections_that_draw_every_option_match_the_reference(device):
+    """The GEMM with its epilogue over row, column and k counts on and off the 256 x 256 tile, the two-step last
+    stage, biases, turned heads of 64 and 128 and windows of a wider output (tk/src/ops/linear.rs:24-58), held to
+    the reference's bar against the unrounded f64 epilogue (tk/src/test/unit/ops.rs:312)."""
+    from svod_amd import Linear, Rotary
+    from util import Lcg, assert_rel_close, bf16_tensor, bits, mean_rel
+    rng = random.Random(43)
+    for case in range(60):
+        d = rng.choice([64, 128])
+        hq, hk = rng.choice([1, 2, 4, 6]), rng.choice([1, 2])
+        turned = rng.random() < 0.6
+        n = (hq + 2 * hk) * d if turned else 8 * rng.choice([1, 5, 32, 33, 63, 100])
+        batch, t = rng.choice([1, 2, 3]), rng.choice([1, 9, 37, 128, 255, 257, 300])
+        k = 32 * rng.choice([1, 2, 3, 4, 5, 8, 13])
+        g = Lcg(100 + case)
+        x, w, bv = g.bf16((batch, t, k)), g.bf16((n, k), mul=0.3), g.bf16((n,))
+        bias = rng.random() < 0.5
+        opts, rope = {}, None
+        if bias:
+            opts["bias"] = bf16_tensor(bv, device)
+        if turned:
+            cos, sin = oracle.rope_table(10_000.0, t, d)
+            cos, sin = oracle.round_bf16(cos), oracle.round_bf16(sin)
+            heads = rng.choice([hq + hk, hq, 1])
+            opts["rope"] = Rotary(bf16_tensor(cos.reshape(1, t, 1, d // 2), device), bf16_tensor(sin.reshape(1, t, 1, d // 2), device), heads, d)
+            rope = (cos, sin, heads, d)
+        name = f"case {case}: rows {batch}x{t} n {n} k {k} bias={bias} rope={None if rope is None else rope[2:]}"
+        wide = None
+        if rng.random() < 0.3:
+            at = 8 * rng.choice([0, 1, 16])
+            wide = torch.full((batch, t, n + at + 8 * rng.choice([0, 3])), 3.0, dtype=torch.bfloat16, device=device)
+            opts["into"] = (wide, at)
+        y = svod_amd.linear(bf16_tensor(x, device), bf16_tensor(w, device), Linear(**opts))
+        torch.cuda.synchronize()
+        assert svod_amd.chosen().startswith('Kernel { op: "linear", family: "gemm"'), (name, svod_amd.chosen())
+        if wide is not None:
+            assert y is wide, name
+            assert bool((wide[..., :at] == 3.0).all()) and bool((wide[..., at + n:] == 3.0).all()), name
+            y = wide[..., at:at + n].contiguous()
+        want = oracle.linear_direct(x, w, bv if bias else None, rope)
+        assert_rel_close(name, to_np(y), want, 2e-2)
+        assert mean_rel(to_np(y), oracle.round_bf16(want.astype(np.float32))) < 3e-4, name
+
+
+def test_prologues_that_draw_every_option_match_the_reference(device):
+    """The prologue over head counts, head sizes, row counts, either norm, rotary tables by position or by token,
+    both 16-bit types' worth of values (tk/src/ops/heads.rs:19-31) to the bars of tk/src/test/unit/heads.rs:124,159."""
+    from svod_amd import Qkv
+    from util import Lcg, bf16_tensor, bits
+    rng = random.Random(44)
+    for case in range(60):
+        d = rng.choice([16, 32, 64, 64, 128, 128, 256])
+        hk = rng.choice([1, 2, 3, 8])
+        hq = hk * rng.choice([1, 2, 4])
+        batch, t = rng.choice([1, 2, 3]), rng.choice([1, 5, 37, 64, 130, 257])
+        norms = (rng.random() < 0.6, rng.random() < 0.6)
+        rope = rng.choice([None, False, True])
+        g = Lcg(200 + case)
+        slots, half = hq + 2 * hk, d // 2
+        qkv = g.bf16((batch, t, slots * d), mul=3.0)
+        q_w = g.bf16((d,), mul=0.5, add=1.0) if norms[0] else None
+        k_w = g.bf16((d,), mul=0.5, add=1.0) if norms[1] else None
+        cos = sin = None
+        if rope is not None:
+            rows = batch * t if rope else t
+            e = np.arange(rows * half)
+            ang = (e // half).astype(np.float64) * 0.01 * (1.0 + (e % half).astype(np.float64))
+            shape = (batch if rope else 1, t, 1, half)
+            cos = oracle.round_bf16(np.cos(ang).astype(np.float32)).reshape(shape)
+            sin = oracle.round_bf16(np.sin(ang).astype(np.float32)).reshape(shape)
+        eps = rng.choice([1e-6, 1e-5])
+        up = lambda a: None if a is None else bf16_tensor(a, device)
+        name = f"case {case}: rows {batch}x{t} heads {hq}/{hk} d {d} norms {norms} rope {rope}"
+        got = svod_amd.heads(up(qkv), Qkv(hq, hk, d, up(q_w), up(k_w), eps, None if cos is None else (up(cos), up(sin))))
+        torch.cuda.synchronize()
+        assert svod_amd.chosen().startswith('Kernel { op: "heads", family: "heads"'), (name, svod_amd.chosen())
+        p = oracle.HeadsProblem(qkv, hq, hk, d, q_w, k_w, eps, cos, sin)
+        direct, program = oracle.heads_direct(p), oracle.heads_kernel(p)
+        for i, what in enumerate("qkv"):
+            out = to_np(got[i])
+            assert np.isfinite(out).all(), (name, what)
+            assert max_abs(out, direct[i]) <= 2e-2, (name, what)   # heads.rs:124
+            assert max_abs(out, program[i]) <= 1e-2, (name, what)  # heads.rs:159
+        want_v = bf16_tensor(qkv.reshape(batch, t, slots, d)[:, :, hq + hk:, :], "cpu")
+        assert np.array_equal(bits(got[2]), bits(want_v)), name

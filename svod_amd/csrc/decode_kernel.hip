@@ -99,6 +99,7 @@ struct State {
 };
 // `a` takes in `b` (the merge of two key splits, L948-1014).
 __device__ __forceinline__ void merge(State &a, const State &b) {
+#pragma clang fp contract(off)  // the products and sums as written, wherever this is inlined
   const float m = __builtin_fmaxf(a.m, b.m);
   const float wa = __builtin_amdgcn_exp2f(a.m - m), wb = __builtin_amdgcn_exp2f(b.m - m);
   a.m = m;
@@ -111,6 +112,9 @@ __device__ __forceinline__ void merge(State &a, const State &b) {
 template <int D, int R, bool F16, bool SPLIT>
 __device__ __forceinline__ void decode_body(const DecodeArgs &p, const int nw) {
 #if defined(__HIP_DEVICE_COMPILE__)
+  // No contraction beyond the fused multiply-adds written out below: the library's kernel (its wave count a launch
+  // argument) and a code object's (four waves, known to the compiler) are then the same arithmetic bit for bit.
+#pragma clang fp contract(off)
   constexpr int kWide = D == 48 ? 64 : D;
   constexpr int LPK = kWide / 8;   // lanes a key row
   constexpr int KPI = 64 / LPK;    // key rows a wave instruction
@@ -185,9 +189,13 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &p, const int nw) {
 
   // Keys [from, to) of rows `row_elems` apart at kb / vb (this lane's 16 bytes of the first row), `mask` their
   // visibility bytes or words (null: all visible).  A pass of the workgroup is nw * KPI rows; a lane works on U
-  // passes at a time and has the next U in flight meanwhile.
+  // passes at a time and has the next U in flight meanwhile.  The workgroup starts `turn` such chunks into the
+  // range and wraps: the softmax does not care where it starts, and the memory does.  Rows of a cache are very
+  // often a power of two apart, and so are the batch rows; workgroups that all walk from key 0 then ask the same
+  // few memory channels for their rows at the same time (a [64, 512, 128, 64] cache read one layer's 32 heads at a
+  // time: 3.8 TB/s from key 0, 5.2 with the starts spread; rows 20 or 80 KiB apart stream the same either way).
   auto stream = [&](const uint16_t *kb, const uint16_t *vb, int64_t row_elems, int from, int to, const void *mask,
-                    int mask_bytes) {
+                    int mask_bytes, uint32_t turn) {
     const int pass = nw * KPI;
     struct Rows {
       u32x4 k[U], v[U];
@@ -256,15 +264,23 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &p, const int nw) {
       }
     };
     // Two sets of rows take turns: one is worked on while the other is on its way.
-    int base = from + wave * KPI;  // the first row of this wave's pass: the same in all of its lanes
-    if (base >= to) return;
+    if (from + wave * KPI >= to) return;  // no chunk holds a row of this wave's
+    const int chunk = U * pass, chunks = (to - from + chunk - 1) / chunk;
+    const int first = (int)(turn % (uint32_t)chunks);
+    // This lane's first row of the i-th chunk the workgroup takes; past the last chunk, a row that is not there.
+    auto row_of = [&](int i) {
+      if (i >= chunks) return to;
+      int c = first + i;
+      if (c >= chunks) c -= chunks;
+      return from + c * chunk + wave * KPI + slot;
+    };
     Rows one, two;
-    load(one, base + slot);
-    for (; base < to; base += 2 * U * pass) {
-      load(two, base + U * pass + slot);
+    load(one, row_of(0));
+    for (int i = 0; i < chunks; i += 2) {
+      load(two, row_of(i + 1));
       work(one);
-      load(one, base + 2 * U * pass + slot);
-      if (base + U * pass < to) work(two);
+      load(one, row_of(i + 2));
+      if (i + 1 < chunks) work(two);
     }
   };
 
@@ -272,7 +288,10 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &p, const int nw) {
     const int64_t at = (kv_row * tk) * p.kv_row_elems + (int64_t)kv_col * D + 8 * pos;
     const void *mask = nullptr;
     if (p.key_mask != nullptr) mask = (const uint8_t *)p.key_mask + (int64_t)b * tk * p.mask_bytes;
-    stream(p.k + at, p.v + at, p.kv_row_elems, k0, k1, mask, p.mask_bytes);
+    // Turned by where the keys lie (the cache row, and the split's share of it), not by who asks: a batch lane
+    // mapped to another cache row reads it as that row's own lane would.  The heads of a row stay in step:
+    // their pieces of a key row lie side by side.
+    stream(p.k + at, p.v + at, p.kv_row_elems, k0, k1, mask, p.mask_bytes, (uint32_t)kv_row * 7u + (uint32_t)split * 3u);
   }
   // The appended rows (L739-755, L827-846): scored by the last split after the cached keys, the first
   // app_lens[b] of them visible, from tensors of their own.
@@ -283,7 +302,7 @@ __device__ __forceinline__ void decode_body(const DecodeArgs &p, const int nw) {
       seen = (int)(n < 0 ? 0 : (n < seen ? n : seen));
     }
     const int64_t at = ((int64_t)b * p.app_rows * p.kv_heads + kvh) * D + 8 * pos;
-    stream(p.k_app + at, p.v_app + at, (int64_t)p.kv_heads * D, 0, seen, nullptr, 1);
+    stream(p.k_app + at, p.v_app + at, (int64_t)p.kv_heads * D, 0, seen, nullptr, 1, 0u);
   }
 
   // The places of a wave that share output columns (lanes LPK apart) merge, then the waves.

@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define SVODK_ABI_VERSION 7
+#define SVODK_ABI_VERSION 8
 
 /* Element types of a tensor descriptor. */
 typedef enum svodk_dtype {
@@ -339,6 +339,14 @@ void svodk_tune_streaming(int32_t workgroups_per_xcd);
 #define SVODK_DECODE_ROWS 4
 #define SVODK_DECODE_ROWS_DEFAULT 2
 void svodk_tune_decode(int32_t rows);
+/*
+ * No counterpart in the reference, whose tuner picks a GEMM's tile by measurement (tk/src/tune.rs, GemmCfg of
+ * tk/src/ops/config/gemm.rs).  svodk_linear runs 256 x 256 output tiles by 8 waves, or 128 x 128 tiles by 4 waves
+ * where the larger tile would make fewer workgroups than half the device's compute units (a projection of few
+ * rows).  `tile` = 256 or 128 names the tile of every later call, 0 gives the choice back to the shape.
+ * Process-wide.  The two tiles give the same bits: a column's k-steps are summed in the same order.
+ */
+void svodk_tune_linear(int32_t tile);
 /* The set the next streaming launch would take, and takes it (no device work): for tests of the
  * assignment.  No counterpart in the reference. */
 uint32_t svodk_streaming_next_set(void);

@@ -26,6 +26,7 @@ from .ops import (  # noqa: F401
     noalloc_scratch_bytes,
     DECODE_ROWS_DEFAULT,
     tune_decode,
+    tune_linear,
     tune_streaming,
     chosen,
     heads,

@@ -57,11 +57,16 @@ struct LinearArgs {
   int32_t seq;       // row r is the token at position r % seq
   int32_t heads, head_dim;  // the first heads * head_dim columns are turned
   int32_t f16;
+  int32_t tile;      // the workgroup's output tile: 256 (8 waves) or 128 (4 waves), linear_tile_of's answer
 };
 hipError_t launch_linear(const LinearArgs &a, hipStream_t stream);
 // Shapes the GEMM kernel takes (n a multiple of 8, k a multiple of 32), and head sizes it turns.
 bool linear_supports(int64_t n, int64_t k);
 bool linear_turns(int32_t head_dim);
+// The output tile of a call: 128 where 256 x 256 tiles would be fewer than half the compute units `units`, unless
+// linear_tile() has named one for every call (0: by the shape again).  linear_tile returns the setting.
+int linear_tile_of(int64_t rows, int64_t n, int units);
+int linear_tile(int32_t tile);
 
 // Flash attention forward: tk/src/kernels/attention.rs:466-924 (attention_body).
 struct AttnArgs {

@@ -47,19 +47,26 @@ typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 typedef __attribute__((ext_vector_type(4))) int i32x4;
 
 constexpr int kXcds = 8;
-constexpr int kWaves = 8;               // 4 along the rows x 2 along the columns
-constexpr int kBm = 256, kBn = 256;     // the workgroup's output tile
 constexpr int kBk = 64;                 // k-columns a stage: a row of a tile is one 128-byte line
 constexpr int kSteps = kBk / 16;        // k-steps of the matrix instruction a stage
 constexpr int kStages = 2;
 constexpr int kGroup = 8;               // column tiles an XCD's resident workgroups spread over
 constexpr int kRowBytes = kBk * 2;      // a tile row in LDS
-constexpr int kTileBytes = kBm * kRowBytes;           // one operand's tile: 32 KiB
-constexpr int kStageBytes = 2 * kTileBytes;           // W tile, then X tile
-constexpr int kLds = kStages * kStageBytes;           // 128 KiB
-constexpr int kFills = kStageBytes / 1024 / kWaves;   // wave instructions of 1 KiB per wave and stage: 8
 constexpr int kOutPitch = 128 * 2 + 16;               // a wave's row of the finished tile in LDS
-static_assert(kWaves * 32 * kOutPitch <= kLds, "half of the finished tile fits where the ring was");
+// The workgroup's output tile in two sizes.  S = 2: 256 x 256 by 8 waves (4 along the rows x 2 along the columns,
+// 64 rows x 128 columns a wave), the size for a product with tiles enough to fill the part.  S = 1: 128 x 128 by
+// 4 waves (32 rows x 128 columns a wave), two workgroups a compute unit: a product of few rows gets four times the
+// workgroups, at twice the fills a flop.  A wave's 128 columns hold whole heads of 64 or 128 either way.
+template <int S>
+struct Tile {
+  static constexpr int kWaves = 4 * S;
+  static constexpr int kBm = 128 * S, kBn = 128 * S;
+  static constexpr int kTileBytes = kBm * kRowBytes;           // one operand's tile: 32 (16) KiB
+  static constexpr int kStageBytes = 2 * kTileBytes;           // W tile, then X tile
+  static constexpr int kLds = kStages * kStageBytes;           // 128 (64) KiB
+  static constexpr int kFills = kStageBytes / 1024 / kWaves;   // wave instructions of 1 KiB per wave and stage: 8
+  static_assert(kWaves * 32 * kOutPitch <= kLds, "32 rows a wave of the finished tile fit where the ring was");
+};
 
 template <bool F16>
 __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
@@ -109,12 +116,14 @@ __device__ __forceinline__ void load4(const uint16_t *p, float (&out)[4]) {
 
 #if defined(__HIP_DEVICE_COMPILE__)
 // HD: the head size a turning kernel is built for (64 or 128), 0: no turn.
-template <bool F16, int HD>
+template <bool F16, int HD, int S = 2>
 __device__ __forceinline__ void linear_body(uint8_t *smem, const uint16_t *__restrict__ x, const uint16_t *__restrict__ w,
                                             const uint16_t *__restrict__ bias, const uint16_t *__restrict__ cos_t,
                                             const uint16_t *__restrict__ sin_t, uint16_t *__restrict__ y, int64_t y_ld,
                                             int64_t rows, int32_t n, int32_t k, int32_t seq, int32_t heads,
                                             uint32_t tiles_n, uint32_t tiles, uint32_t per_xcd, uint32_t band) {
+  constexpr int kWaves = Tile<S>::kWaves, kBm = Tile<S>::kBm, kBn = Tile<S>::kBn, kTileBytes = Tile<S>::kTileBytes;
+  constexpr int kStageBytes = Tile<S>::kStageBytes, kLds = Tile<S>::kLds, kFills = Tile<S>::kFills;
   const int tid = __builtin_amdgcn_workitem_id_x();
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -193,41 +202,46 @@ __device__ __forceinline__ void linear_body(uint8_t *smem, const uint16_t *__res
 
   // ---- operand reads: A = W rows (the output's columns), B = X rows (the output's rows); fragment
   // (block of 32 rows, k-step ks): row ln of the block, logical chunk 2 * ks + g.
-  const int wave_m = wave & 3, wave_n = wave >> 2;  // 64-row and 128-column shares of the tile
-  int a_read[4], b_read[2];
+  const int wave_m = wave & 3, wave_n = wave >> 2;  // 32 S-row and 128-column shares of the tile
+  int a_read[4], b_read[S];
 #pragma unroll
   for (int cb = 0; cb < 4; cb++) a_read[cb] = (wave_n * 128 + cb * 32 + ln) * kRowBytes;
 #pragma unroll
-  for (int rb = 0; rb < 2; rb++) b_read[rb] = kTileBytes + (wave_m * 64 + rb * 32 + ln) * kRowBytes;
+  for (int rb = 0; rb < S; rb++) b_read[rb] = kTileBytes + (wave_m * 32 * S + rb * 32 + ln) * kRowBytes;
   const int swz = (ln >> 1) & 7;  // every block starts on a multiple of 16 rows
   int chunk_at[kSteps];
 #pragma unroll
   for (int ks = 0; ks < kSteps; ks++) chunk_at[ks] = ((2 * ks + g) ^ swz) << 4;
 
-  f32x16 acc[2][4];
+  f32x16 acc[S][4];
   const f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-  for (int rb = 0; rb < 2; rb++)
+  for (int rb = 0; rb < S; rb++)
 #pragma unroll
     for (int cb = 0; cb < 4; cb++) acc[rb][cb] = zero;
 
-  // One k-step: eight products of the fragment set `set` (four of W: this wave's column blocks; two of X: its
-  // row blocks), and beside the first six of them the six fragment reads of k-step `nks` of stage slot `nslot`
-  // into the other set, so that a product's operands were asked for six to eight products earlier.  The fences
-  // keep the order: left to itself the scheduler gathers the reads in front of the products that want them.
-  u32x4 af[2][4], bf[2][2];
+  // One k-step: the 4 S products of the fragment set `set` (four fragments of W: this wave's column blocks; S of
+  // X: its row blocks), and beside them the 4 + S fragment reads of k-step `nks` of stage slot `nslot` into the
+  // other set (one beside each of the first six of eight products; with four products, two beside the first), so
+  // that a product's operands were asked for a k-step earlier.  The fences keep the order: left to itself the
+  // scheduler gathers the reads in front of the products that want them.
+  constexpr int kReads = 4 + S, kProducts = 4 * S;
+  u32x4 af[2][4], bf[2][S];
   auto read_fragment = [&](int slot, int ks, int i, int set) {
     const uint8_t *st = smem + slot * kStageBytes;
-    if (i < 2)
+    if (i < S)
       bf[set][i] = *reinterpret_cast<const u32x4 *>(st + b_read[i] + chunk_at[ks]);
     else
-      af[set][i - 2] = *reinterpret_cast<const u32x4 *>(st + a_read[i - 2] + chunk_at[ks]);
+      af[set][i - S] = *reinterpret_cast<const u32x4 *>(st + a_read[i - S] + chunk_at[ks]);
   };
   auto step = [&](int set, int nslot, int nks, bool reads) {
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-      acc[i & 1][i >> 1] = mma<F16>(af[set][i >> 1], bf[set][i & 1], acc[i & 1][i >> 1]);
-      if (reads && i < 6) read_fragment(nslot, nks, i, set ^ 1);
+    for (int i = 0; i < kProducts; i++) {
+      acc[i % S][i / S] = mma<F16>(af[set][i / S], bf[set][i % S], acc[i % S][i / S]);
+      if (reads) {
+        if (i < kReads) read_fragment(nslot, nks, i, set ^ 1);
+        if (i == 0 && kReads > kProducts) read_fragment(nslot, nks, kProducts, set ^ 1);
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
   };
@@ -257,7 +271,7 @@ __device__ __forceinline__ void linear_body(uint8_t *smem, const uint16_t *__res
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kFills) : "memory");  // stage 0 is in
   __syncthreads();
 #pragma unroll
-  for (int i = 0; i < 6; i++) read_fragment(0, 0, i, 0);
+  for (int i = 0; i < kReads; i++) read_fragment(0, 0, i, 0);
   for (int s = 0; s < nk; s++) {
     const int slot = s & 1;
     step(0, slot, 1, true);
@@ -286,7 +300,7 @@ __device__ __forceinline__ void linear_body(uint8_t *smem, const uint16_t *__res
         float b4[4];
         load4<F16>(bias + col, b4);
 #pragma unroll
-        for (int rb = 0; rb < 2; rb++)
+        for (int rb = 0; rb < S; rb++)
 #pragma unroll
           for (int e = 0; e < 4; e++) acc[rb][cb][4 * q + e] += b4[e];
       }
@@ -321,8 +335,8 @@ __device__ __forceinline__ void linear_body(uint8_t *smem, const uint16_t *__res
     __syncthreads();
     if (n0 + wave_n * 128 < turned) {
 #pragma unroll
-      for (int rb = 0; rb < 2; rb++) {
-        const int r = wave_m * 64 + rb * 32 + ln;
+      for (int rb = 0; rb < S; rb++) {
+        const int r = wave_m * 32 * S + rb * 32 + ln;
         const uint16_t *cos_row = reinterpret_cast<const uint16_t *>(cos_lds + r * kPitch);
         const uint16_t *sin_row = reinterpret_cast<const uint16_t *>(sin_lds + r * kPitch);
 #pragma unroll
@@ -360,7 +374,7 @@ __device__ __forceinline__ void linear_body(uint8_t *smem, const uint16_t *__res
   const int orow = lane >> 4, ochunk = lane & 15;
   const int col = n0 + wave_n * 128 + ochunk * 8;  // n is a multiple of 8: a run of eight lies inside or outside
 #pragma unroll
-  for (int rb = 0; rb < 2; rb++) {
+  for (int rb = 0; rb < S; rb++) {
     uint8_t *srow = stage + ln * kOutPitch + 8 * g;
 #pragma unroll
     for (int cb = 0; cb < 4; cb++) {
@@ -376,7 +390,7 @@ __device__ __forceinline__ void linear_body(uint8_t *smem, const uint16_t *__res
     for (int it = 0; it < 8; it++) {
       const int r = it * 4 + orow;
       const u32x4 out = *reinterpret_cast<const u32x4 *>(stage + r * kOutPitch + ochunk * 16);
-      const int64_t row = m0 + wave_m * 64 + rb * 32 + r;
+      const int64_t row = m0 + wave_m * 32 * S + rb * 32 + r;
       // Streaming stores: the output is not read again here, and left out of L2 it does not push the operands out.
       if (row < rows && col < n) __builtin_nontemporal_store(out, reinterpret_cast<u32x4 *>(y + row * y_ld + col));
     }
@@ -385,8 +399,8 @@ __device__ __forceinline__ void linear_body(uint8_t *smem, const uint16_t *__res
 #endif  // __HIP_DEVICE_COMPILE__
 
 #if !defined(SVODK_CODE_OBJECT)  // the library's kernel and its launch: not part of a code object build
-template <bool F16, int HD>
-__global__ __launch_bounds__(kWaves * 64, 1) void linear_kernel(const uint16_t *__restrict__ x, const uint16_t *__restrict__ w,
+template <bool F16, int HD, int S>
+__global__ __launch_bounds__(Tile<S>::kWaves * 64, 3 - S) void linear_kernel(const uint16_t *__restrict__ x, const uint16_t *__restrict__ w,
                                                                 const uint16_t *__restrict__ bias,
                                                                 const uint16_t *__restrict__ cos_t,
                                                                 const uint16_t *__restrict__ sin_t, uint16_t *__restrict__ y,
@@ -396,12 +410,13 @@ __global__ __launch_bounds__(kWaves * 64, 1) void linear_kernel(const uint16_t *
                                                                 uint32_t band) {
 #if defined(__HIP_DEVICE_COMPILE__)
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
-  linear_body<F16, HD>(smem, x, w, bias, cos_t, sin_t, y, y_ld, rows, n, k, seq, heads, tiles_n, tiles, per_xcd, band);
+  linear_body<F16, HD, S>(smem, x, w, bias, cos_t, sin_t, y, y_ld, rows, n, k, seq, heads, tiles_n, tiles, per_xcd, band);
 #endif
 }
 
-template <bool F16, int HD>
+template <bool F16, int HD, int S>
 hipError_t launch(const LinearArgs &a, hipStream_t stream) {
+  constexpr int kBm = Tile<S>::kBm, kBn = Tile<S>::kBn, kLds = Tile<S>::kLds, kWaves = Tile<S>::kWaves;
   const int64_t tiles_m = (a.rows + kBm - 1) / kBm, tiles_n = (a.n + kBn - 1) / kBn;
   const int64_t tiles = tiles_m * tiles_n;
   if (tiles == 0) return hipSuccess;
@@ -409,7 +424,7 @@ hipError_t launch(const LinearArgs &a, hipStream_t stream) {
   const int64_t band = tiles_m >= 2 * kXcds ? (tiles_m + kXcds - 1) / kXcds : 0;
   const int64_t per_xcd = band > 0 ? band * tiles_n : (tiles + kXcds - 1) / kXcds;
   if (per_xcd * kXcds > 0x7fffffffLL) return hipErrorInvalidConfiguration;
-  auto kernel = linear_kernel<F16, HD>;
+  auto kernel = linear_kernel<F16, HD, S>;
   static std::atomic<uint64_t> configured{0};  // a bit per device ordinal, devices past 63 always ask
   int device = 0;
   hipError_t e = hipGetDevice(&device);
@@ -443,6 +458,7 @@ __device__ __forceinline__ void linear_entry(uint8_t *smem, const uint16_t *x, c
                                              const uint16_t *cos_t, const uint16_t *sin_t, uint16_t *y, int32_t rows,
                                              int32_t n, int32_t k, int32_t seq, int32_t heads) {
   if (rows <= 0 || n <= 0 || k <= 0) return;
+  constexpr int kBm = Tile<2>::kBm, kBn = Tile<2>::kBn;  // the code objects hold the 256 x 256 form
   const uint32_t tiles_m = ((uint32_t)rows + kBm - 1) / kBm, tiles_n = ((uint32_t)n + kBn - 1) / kBn;
   const uint32_t tiles = tiles_m * tiles_n;
   // The library's launch geometry (see launch below in the library build): bands of row tiles per XCD
@@ -454,11 +470,11 @@ __device__ __forceinline__ void linear_entry(uint8_t *smem, const uint16_t *x, c
 }
 
 #define SVODK_LINEAR_ENTRY(NAME, F16, HD)                                                                             \
-  extern "C" __global__ __launch_bounds__(kWaves * 64, 1) void NAME(                                                  \
+  extern "C" __global__ __launch_bounds__(Tile<2>::kWaves * 64, 1) void NAME(                                                  \
       const uint16_t *__restrict__ x, const uint16_t *__restrict__ w, const uint16_t *__restrict__ bias,              \
       const uint16_t *__restrict__ cos_t, const uint16_t *__restrict__ sin_t, uint16_t *__restrict__ y, int32_t rows, \
       int32_t n, int32_t k, int32_t seq, int32_t heads) {                                                             \
-    __shared__ __attribute__((aligned(1024))) uint8_t smem[kLds];                                                     \
+    __shared__ __attribute__((aligned(1024))) uint8_t smem[Tile<2>::kLds];                                                   \
     linear_entry<F16, HD>(smem, x, w, bias, cos_t, sin_t, y, rows, n, k, seq, heads);                                 \
   }
 SVODK_LINEAR_ENTRY(svodk_linear_bf16, false, 0)
@@ -479,13 +495,33 @@ bool linear_supports(int64_t n, int64_t k) { return n > 0 && n % 8 == 0 && k >= 
 
 bool linear_turns(int32_t head_dim) { return head_dim == 64 || head_dim == 128; }
 
+// The tile a call's shape takes: 256 x 256 unless that makes fewer workgroups than half the compute units (256 on
+// this part; read from the device on a launch), where 128 x 128 makes four times as many.
+namespace {
+std::atomic<int> g_linear_tile{0};  // 0: by the shape; 128 or 256: every call
+}
+int linear_tile(int32_t tile) {
+  if (tile == 0 || tile == 128 || tile == 256) g_linear_tile.store(tile, std::memory_order_relaxed);
+  return g_linear_tile.load(std::memory_order_relaxed);
+}
+int linear_tile_of(int64_t rows, int64_t n, int units) {
+  const int named = g_linear_tile.load(std::memory_order_relaxed);
+  if (named != 0) return named;
+  const int64_t wide = ((rows + 255) / 256) * ((n + 255) / 256);
+  return 2 * wide <= units ? 128 : 256;
+}
+
 hipError_t launch_linear(const LinearArgs &a, hipStream_t stream) {
   if (!linear_supports(a.n, a.k)) return hipErrorInvalidValue;
   if (a.cos != nullptr && (!linear_turns(a.head_dim) || a.seq <= 0 || (int64_t)a.heads * a.head_dim > a.n))
     return hipErrorInvalidValue;
   const int hd = a.cos != nullptr ? a.head_dim : 0;
-  if (a.f16) return hd == 0 ? launch<true, 0>(a, stream) : hd == 64 ? launch<true, 64>(a, stream) : launch<true, 128>(a, stream);
-  return hd == 0 ? launch<false, 0>(a, stream) : hd == 64 ? launch<false, 64>(a, stream) : launch<false, 128>(a, stream);
+  if (a.tile == 128) {
+    if (a.f16) return hd == 0 ? launch<true, 0, 1>(a, stream) : hd == 64 ? launch<true, 64, 1>(a, stream) : launch<true, 128, 1>(a, stream);
+    return hd == 0 ? launch<false, 0, 1>(a, stream) : hd == 64 ? launch<false, 64, 1>(a, stream) : launch<false, 128, 1>(a, stream);
+  }
+  if (a.f16) return hd == 0 ? launch<true, 0, 2>(a, stream) : hd == 64 ? launch<true, 64, 2>(a, stream) : launch<true, 128, 2>(a, stream);
+  return hd == 0 ? launch<false, 0, 2>(a, stream) : hd == 64 ? launch<false, 64, 2>(a, stream) : launch<false, 128, 2>(a, stream);
 }
 
 }  // namespace svodk

@@ -174,6 +174,25 @@ bool current_device_has_kernels() {
   return state == 1;
 }
 
+// The compute units of the current device (256 on an MI355X), asked once a device.
+int current_device_units() {
+  int device = -1;
+  if (hipGetDevice(&device) != hipSuccess || device < 0) {
+    (void)hipGetLastError();
+    return 256;
+  }
+  static std::atomic<int> known[64];
+  int units = device < 64 ? known[device].load(std::memory_order_acquire) : 0;
+  if (units == 0) {
+    if (hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || units <= 0) {
+      (void)hipGetLastError();
+      units = 256;
+    }
+    if (device < 64) known[device].store(units, std::memory_order_release);
+  }
+  return units;
+}
+
 // ---- shape gates (tk/src/ops/shape.rs).
 // gate (L92-99): a target with kernels, every operand the same 16-bit type the
 // target has a matrix core for: gfx950 has one for bf16 and for f16, and both have kernels here.
@@ -707,6 +726,7 @@ int svodk_attention_packed(const svodk_tensor *qkv, int32_t heads, int32_t kv_he
 
 void svodk_tune_streaming(int32_t workgroups_per_xcd) { svodk::attention_stream_slots(workgroups_per_xcd); }
 void svodk_tune_decode(int32_t rows) { svodk::attention_decode_rows(rows); }
+void svodk_tune_linear(int32_t tile) { svodk::linear_tile(tile); }
 uint32_t svodk_streaming_next_set(void) { return svodk::next_queue_set(); }
 
 // The batch rows by descending key count, for svodk_attn.row_order (no counterpart in the reference,
@@ -1133,8 +1153,13 @@ int svodk_linear(const svodk_tensor *x, const svodk_tensor *w, const svodk_linea
   a.heads = rope ? rope->heads : 0;
   a.head_dim = rope ? rope->head_dim : 0;
   a.f16 = x->dtype == SVODK_F16;
-  ran(op, "gemm", rope ? "GemmCfg { bm: 256, bn: 256, bk: 64, stages: 2, warps: [4, 2], epilogue: { bias, rope } }"
-                       : "GemmCfg { bm: 256, bn: 256, bk: 64, stages: 2, warps: [4, 2], epilogue: { bias } }");
+  a.tile = svodk::linear_tile_of(rows, n, current_device_units());
+  if (a.tile == 128)
+    ran(op, "gemm", rope ? "GemmCfg { bm: 128, bn: 128, bk: 64, stages: 2, warps: [4, 1], epilogue: { bias, rope } }"
+                         : "GemmCfg { bm: 128, bn: 128, bk: 64, stages: 2, warps: [4, 1], epilogue: { bias } }");
+  else
+    ran(op, "gemm", rope ? "GemmCfg { bm: 256, bn: 256, bk: 64, stages: 2, warps: [4, 2], epilogue: { bias, rope } }"
+                         : "GemmCfg { bm: 256, bn: 256, bk: 64, stages: 2, warps: [4, 2], epilogue: { bias } }");
   const hipError_t e = svodk::launch_linear(a, (hipStream_t)hip_stream);
   if (e != hipSuccess) return fail(SVODK_ERR_LAUNCH, "%s: %s", op, hipGetErrorString(e));
   return SVODK_KERNEL;

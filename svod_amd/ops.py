@@ -139,6 +139,8 @@ def load_library(path: Optional[str] = None) -> ctypes.CDLL:
     lib.svodk_tune_streaming.argtypes = [ctypes.c_int32]
     lib.svodk_tune_decode.restype = None
     lib.svodk_tune_decode.argtypes = [ctypes.c_int32]
+    lib.svodk_tune_linear.restype = None
+    lib.svodk_tune_linear.argtypes = [ctypes.c_int32]
     lib.svodk_supported.restype = ctypes.c_int
     lib.svodk_last_chosen.restype = ctypes.c_char_p
     lib.svodk_last_error.restype = ctypes.c_char_p
@@ -377,6 +379,12 @@ def tune_decode(rows: int) -> None:
     or a bias to run as a decoder step, K and V streamed through registers: 0..4, DECODE_ROWS_DEFAULT unasked;
     0 = every call runs key tiles.  Process-wide; the two paths agree to the op's tolerance, not bit for bit."""
     load_library().svodk_tune_decode(int(rows))
+
+
+def tune_linear(tile: int) -> None:
+    """The output tile of every later ``linear`` call: 256 (8 waves) or 128 (4 waves); 0 = by the shape (128 where
+    256 x 256 tiles would be fewer than half the compute units).  Process-wide; the two give the same bits."""
+    load_library().svodk_tune_linear(int(tile))
 
 
 def attention_packed(qkv: torch.Tensor, heads: int, kv_heads: int, opts: Optional[Attn] = None,

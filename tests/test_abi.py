@@ -25,7 +25,7 @@ def test_every_declared_symbol_is_exported():
     lib = svod_amd.load_library()
     for n in sorted(names):
         assert hasattr(lib, n), n
-    assert lib.svodk_abi_version() == 7
+    assert lib.svodk_abi_version() == 8
 
 
 def test_status_names():

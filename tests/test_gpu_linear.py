@@ -165,3 +165,40 @@ def test_into_stores_a_window_of_a_wider_output(device):
     with pytest.raises(svod_amd.OpError) as e:
         svod_amd.linear(bf16_tensor(x, device), bf16_tensor(w, device), Linear(into=(wide, c - n + 8), **opts))
     assert e.value.kind == "Shape"
+
+
+@pytest.fixture
+def tile_by_shape():
+    yield
+    svod_amd.tune_linear(0)
+
+
+@pytest.mark.parametrize("lead,heads,k,bias", [((2, 300), (4, 2, 128), 256, True), ((1, 37), (12, 12, 64), 96, False),
+                                               ((3, 129), None, 160, True), ((1, 1), None, 32, False)],
+                         ids=["turned 128 across tiles", "turned 64, partial rows", "plain across tiles", "one row"])
+def test_the_two_tiles_give_the_same_bits(device, tile_by_shape, lead, heads, k, bias):
+    """svodk_tune_linear: 128 x 128 tiles by 4 waves against 256 x 256 by 8; a column's k-steps are summed in the
+    same order, so nothing but the launch differs."""
+    n = (heads[0] + 2 * heads[1]) * heads[2] if heads else 8 * 41
+    x, w, bv = case(lead, k, n, seed=51)
+    opts = dict(bias=bf16_tensor(bv, device)) if bias else {}
+    if heads:
+        _, (cos_d, sin_d) = tables(lead[1], heads[2], device)
+        opts["rope"] = Rotary(cos_d, sin_d, heads[0] + heads[1], heads[2])
+    got = {}
+    for tile in (256, 128):
+        svod_amd.tune_linear(tile)
+        got[tile] = svod_amd.linear(bf16_tensor(x, device), bf16_tensor(w, device), Linear(**opts))
+        torch.cuda.synchronize()
+        assert f"bm: {tile}, bn: {tile}" in svod_amd.chosen(), svod_amd.chosen()
+    assert np.array_equal(bits(got[256]), bits(got[128]))
+
+
+def test_the_tile_follows_the_shape(device, tile_by_shape):
+    """Few rows take 128 x 128 tiles (four times the workgroups), a product that fills the part 256 x 256."""
+    svod_amd.tune_linear(0)
+    w = bf16_tensor(np.ones((4096, 64), dtype=np.float32), device)
+    for rows, tile in ((512, 128), (2048, 128), (4096, 256), (16384, 256)):
+        svod_amd.linear(bf16_tensor(np.ones((rows, 64), dtype=np.float32), device), w)
+        torch.cuda.synchronize()
+        assert f"bm: {tile}, bn: {tile}" in svod_amd.chosen(), (rows, svod_amd.chosen())

@@ -142,8 +142,12 @@ def test_projections_that_draw_every_option_match_the_reference(device):
             at = 8 * rng.choice([0, 1, 16])
             wide = torch.full((batch, t, n + at + 8 * rng.choice([0, 3])), 3.0, dtype=torch.bfloat16, device=device)
             opts["into"] = (wide, at)
-        y = svod_amd.linear(bf16_tensor(x, device), bf16_tensor(w, device), Linear(**opts))
-        torch.cuda.synchronize()
+        svod_amd.tune_linear((256, 128, 0)[case % 3])  # both tiles, and the shape's own choice
+        try:
+            y = svod_amd.linear(bf16_tensor(x, device), bf16_tensor(w, device), Linear(**opts))
+            torch.cuda.synchronize()
+        finally:
+            svod_amd.tune_linear(0)
         assert svod_amd.chosen().startswith('Kernel { op: "linear", family: "gemm"'), (name, svod_amd.chosen())
         if wide is not None:
             assert y is wide, name
